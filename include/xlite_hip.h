@@ -1,0 +1,230 @@
+/*
+ * xlite_hip.h — C ABI of the MI355X (gfx950) attention hot path.
+ *
+ * Every entry point replaces one host launcher of the Xlite runtime
+ * (xlite/csrc/op.h) together with the device kernel it starts. Arguments are
+ * plain device pointers and scalars: no framework types cross this boundary.
+ *
+ * Conventions
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream). Work
+ *     is enqueued on it and the call returns without synchronising.
+ *   - Every function returns XLITE_HIP_OK (0) or a negative XLITE_HIP_E* code;
+ *     xlite_hip_last_error() then holds a message for the calling thread.
+ *   - All tensors are dense row-major ("contiguous"); index tensors are int32
+ *     except `position`, which is int64 (xlite/csrc/kernels/rope_and_cache.h:452).
+ *   - `dtype` selects the 16-bit element type of activations and caches.
+ */
+#ifndef XLITE_HIP_H_
+#define XLITE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XLITE_HIP_OK 0
+#define XLITE_HIP_EINVAL (-1)   /* bad argument / unsupported combination */
+#define XLITE_HIP_ERUNTIME (-2) /* HIP runtime reported an error */
+#define XLITE_HIP_ENOSPC (-3)   /* workspace too small */
+
+/* element types (same order as xlite/csrc/base.h XDtype FP16/BF16) */
+#define XLITE_HIP_FP16 0
+#define XLITE_HIP_BF16 1
+/* KV cache element types: the activation dtype, or int8 with fp32 scales */
+#define XLITE_HIP_KV_SAME 0
+#define XLITE_HIP_KV_INT8 1
+
+/* Message of the last failed call on this thread ("" if none). */
+const char *xlite_hip_last_error(void);
+
+/* Library / device probe: returns the ABI version, fills optional outputs. */
+int xlite_hip_version(void);
+int xlite_hip_device_info(int device, int *num_cu, int *lds_bytes_per_cu, char *arch, size_t arch_len);
+
+/* ------------------------------------------------------------------------
+ * rope_and_cache — replaces XliteOpRopeCache (xlite/csrc/op.cpp:905-943) +
+ * kernel rope_and_cache<Dtype> (xlite/csrc/kernels/rope_and_cache.h:206-610).
+ *
+ * inout      [num_tokens, (n_heads + 2*n_kv_heads) * head_dim]  q | k | v, updated in place
+ * k_cache    [num_blocks, block_size, n_kv_heads, head_dim]
+ * v_cache    same shape
+ * position   [num_tokens] int64, or [3, num_tokens] when an mrope mask is non-zero
+ * cosin      [max_pos, rot_dim]  row = cos(rot_dim/2) | sin(rot_dim/2), in `dtype`
+ * slot_mapping [num_tokens] int32, slot = block * block_size + offset (used unsigned)
+ * NeoX (half-split) rotation only; q is additionally scaled by 1/sqrt(head_dim).
+ * ---------------------------------------------------------------------- */
+int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_cache,
+                             const int64_t *position, const void *cosin,
+                             const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads,
+                             uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim,
+                             uint32_t block_size, int is_neox, uint64_t mrope_mask_h,
+                             uint64_t mrope_mask_w, int dtype);
+
+/* ------------------------------------------------------------------------
+ * attention — replaces XliteOpAttention and XliteOpFlashAttention
+ * (xlite/csrc/op.cpp:945-993) + kernels attention.h / flash_attention.h.
+ *
+ * qkv         [total_tokens, (n_heads + 2*n_kv_heads) * head_dim]; only q is read,
+ *             already rotated and scaled by rope_and_cache
+ * k_cache/v_cache  paged caches as above; when kv_dtype == XLITE_HIP_KV_INT8 they
+ *             hold int8 and k_scale/v_scale [num_blocks, block_size, n_kv_heads]
+ *             fp32 hold the per-token-per-head scales (x = q8 * scale)
+ * output      [total_tokens, n_heads * head_dim]
+ * query_start_loc, lens, cached_lens  [batch] int32
+ * block_tables [batch * max_num_block] int32
+ * Row r of sequence i attends to cache positions 0 .. cached_lens[i] + r.
+ * No softmax scale is applied here (q arrives pre-scaled).
+ *
+ * workspace   device scratch of at least xlite_hip_attention_workspace_bytes();
+ *             its first XLITE_HIP_WS_COUNTER_BYTES must be zero before the first
+ *             call and are left zero by every call.
+ * ---------------------------------------------------------------------- */
+#define XLITE_HIP_WS_COUNTER_BYTES 65536
+
+size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
+                                           uint32_t head_dim, uint32_t block_size,
+                                           uint32_t batch, uint32_t max_num_block);
+
+int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, const void *v_cache,
+                        void *output, const int32_t *query_start_loc, const int32_t *lens,
+                        const int32_t *cached_lens, const int32_t *block_tables,
+                        uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                        uint32_t head_dim, uint32_t block_size, uint32_t batch,
+                        uint32_t max_num_block, int dtype, int kv_dtype, const float *k_scale,
+                        const float *v_scale, void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * mla_attention — replaces XliteOpMLAV2 / XliteOpFlashMLAV2
+ * (xlite/csrc/op.cpp:995-1058) + kernels mla_v2.h / flash_mla_v2.h: the absorbed
+ * MLA attention between the two einsums of the mla_v2 operator.
+ *
+ * q_absorb  [total_tokens, n_heads, kv_lora_rank]
+ * qr        [total_tokens, n_heads, rope_head_dim]
+ * k_cache   [num_blocks, block_size, kv_lora_rank]   (latent)
+ * pe_cache  [num_blocks, block_size, rope_head_dim]  (rotated key slice)
+ * o_absorb  [total_tokens, n_heads, kv_lora_rank]
+ * scores = (q_absorb . k + qr . pe) * scale, causal as in attention.
+ * topk_indices [total_tokens, top_k] int32 (top_k == 0: dense, pointer unused):
+ * when top_k > 0 a row attends only to the listed positions that are also
+ * inside its causal range. bf16 only (xlite/csrc/op.cpp:1014).
+ * ---------------------------------------------------------------------- */
+size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t kv_lora_rank,
+                                     uint32_t block_size, uint32_t batch, uint32_t max_num_blocks);
+
+int xlite_hip_mla_attention(void *stream, const void *q_absorb, const void *qr,
+                            const void *k_cache, const void *pe_cache, void *o_absorb,
+                            const int32_t *query_start_loc, const int32_t *lens,
+                            const int32_t *cached_lens, const int32_t *block_tables,
+                            uint32_t total_tokens, uint32_t n_heads, uint32_t rope_head_dim,
+                            uint32_t kv_lora_rank, uint32_t block_size, uint32_t batch,
+                            uint32_t max_num_blocks, float scale, const int32_t *topk_indices,
+                            uint32_t top_k, int dtype, void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * mla_v3 — replaces XliteOpMLAV3 (xlite/csrc/op.cpp:1086-1104) + kernel mla_v3.h:
+ * absorbed MLA attention over a contiguous per-sequence cache
+ * k_dense [batch, index_topk, kv_lora_rank], pe_dense [batch, index_topk, rope_head_dim];
+ * every query row of sequence i attends to the first
+ * min(cached_lens[i] + lens[i], index_topk) entries, no causal structure.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_mla_v3(void *stream, const void *q_absorb, const void *qr, const void *k_dense,
+                     const void *pe_dense, void *o_absorb, const int32_t *query_start_loc,
+                     const int32_t *lens, const int32_t *cached_lens, uint32_t total_tokens,
+                     uint32_t n_heads, uint32_t rope_head_dim, uint32_t kv_lora_rank,
+                     uint32_t batch, uint32_t index_topk, float scale, int dtype, void *workspace,
+                     size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * gather_sparse_kv_cache — replaces XliteOpGatherSparseKVCache
+ * (xlite/csrc/op.cpp:1060-1084) + kernel gather_sparse_kv_cache.h:15-134.
+ * dense[b, i] = paged[block_tables[b*max_num_blocks + tok / block_size], tok % block_size]
+ * with tok = topk_indices[b, i], for i < min(query_lens[b] + cached_lens[b], index_topk).
+ * Other dense slots are left untouched. kv_heads must be 1.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_gather_sparse_kv_cache(void *stream, const void *k_cache, const void *pe_cache,
+                                     const int32_t *block_tables, const int32_t *topk_indices,
+                                     const int32_t *query_lens, const int32_t *cached_lens,
+                                     void *k_dense, void *pe_dense, uint32_t batch,
+                                     uint32_t index_topk, uint32_t block_size,
+                                     uint32_t max_num_blocks, uint32_t kv_lora_rank,
+                                     uint32_t rope_head_dim, uint32_t kv_heads, int dtype);
+
+/* ------------------------------------------------------------------------
+ * rope_complex — replaces XliteOpRopeComplex (xlite/csrc/op.cpp:1106-1126) +
+ * kernel rope_complex_and_cache.h:12-241 in its "no cache" mode.
+ * input  [num_tokens, n_local_heads, step_dim]; the last rope_dim elements of each
+ *        head are interleaved (re, im) pairs
+ * freqs  [max_pos, rope_dim/2] complex64 == interleaved fp32 (cos, sin)
+ * output [num_tokens, n_local_heads, rope_dim] = [re... | im...] of x * freqs[position]
+ * ---------------------------------------------------------------------- */
+int xlite_hip_rope_complex(void *stream, uint32_t num_tokens, uint32_t n_local_heads,
+                           uint32_t step_dim, uint32_t rope_dim, const void *input,
+                           const float *freqs, const int64_t *position, void *output, int dtype);
+
+/* ------------------------------------------------------------------------
+ * mla_prepare — replaces XliteOpMlaPrepare (xlite/csrc/op.cpp:1151-1175) +
+ * kernel mla_prepare.h:14-39 (two RMSNorms + rope_complex_and_cache).
+ * attn_qkvc [num_tokens, q_lora_rank + kv_lora_rank + rope_head_dim]; the rope slice
+ * is rotated in place. attn_norm_qc / attn_norm_kvc receive rms(x)*w + b of the first
+ * two slices; the latter is also written to k_cache[slot], the rotated slice to
+ * pe_cache[slot]. block_size == 0 disables both cache writes.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_mla_prepare(void *stream, void *attn_qkvc, const void *q_norm,
+                          const void *q_norm_bias, void *attn_norm_qc, const void *kv_norm,
+                          const void *kv_norm_bias, void *attn_norm_kvc, const float *freqs,
+                          const int64_t *position, uint32_t num_tokens, uint32_t q_lora_rank,
+                          uint32_t kv_lora_rank, uint32_t rope_head_dim, uint32_t block_size,
+                          void *k_cache, void *pe_cache, const int32_t *slot_mapping,
+                          float norm_eps, int dtype);
+
+/* ------------------------------------------------------------------------
+ * einsum_mht_htd_mhd / einsum_mht_hdt_mhd — replace XliteOpEinsumMhtHtdMhd /
+ * XliteOpEinsumMhtHdtMhd (xlite/csrc/op.cpp:1872-1918).
+ * mhd[m, h, :d] = sum_t mht[m, h, t] * w[h, t, d]   (w_is_hdt == 0, w = [h, t, d])
+ *                                   * w[h, d, t]   (w_is_hdt != 0, w = [h, d, t])
+ * `t_stride` is the distance in elements between consecutive heads of mht
+ * (>= t; the mla_v2 operator reads the first `nope` of each [nope + rope] head).
+ * ---------------------------------------------------------------------- */
+int xlite_hip_einsum_mht_mhd(void *stream, const void *mht, const void *w, void *mhd, uint32_t m,
+                             uint32_t h, uint32_t t, uint32_t d, uint32_t t_stride, int w_is_hdt,
+                             int dtype);
+
+/* ------------------------------------------------------------------------
+ * get_tile_size_of_cached_kv — replaces GetTileSizeOfCachedKV
+ * (xlite/csrc/auto_tuner.cpp:163-210). Host-only, same integer results.
+ * Returns the tile size, or a negative error code.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_get_tile_size_of_cached_kv(const uint32_t *cached_lens, const uint32_t *query_lens,
+                                         uint32_t batch, uint32_t head_num_in_group,
+                                         uint32_t n_kv_heads, uint32_t block_size,
+                                         uint32_t aic_num);
+
+/* ------------------------------------------------------------------------
+ * prepare_attn — replaces the host part of XRuntime::PrepareAttn
+ * (xlite/csrc/runtime.cpp:404-550): from per-sequence lens / cached_lens and a
+ * ragged block table (block_table_rows[i] points at row_lens[i] int32 entries)
+ * fill query_start_loc[batch], position[sum lens], slot_mapping[sum lens] and the
+ * dense block table [batch, *max_num_blocks]. Host memory only. Outputs must be
+ * large enough (dense_tables: batch * ceil(max(lens+cached)/block_size)).
+ * `is_decode` is set to 1 when every len == 1.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_prepare_attn(const uint32_t *lens, const uint32_t *cached_lens, uint32_t batch,
+                           const int32_t *const *block_table_rows, const uint32_t *row_lens,
+                           uint32_t block_size, int32_t *query_start_loc, int64_t *position,
+                           int32_t *slot_mapping, int32_t *dense_tables, size_t dense_capacity,
+                           uint32_t *max_num_blocks, uint32_t *batched_tokens, int *is_decode);
+
+/* ------------------------------------------------------------------------
+ * int8 KV-cache helper (no counterpart in the reference, whose caches are always
+ * the activation dtype): quantise rows of `src` [rows, head_dim] into `dst` int8
+ * with one fp32 scale per row, scale = absmax/127, q = clamp(rint(x/scale), -127, 127).
+ * ---------------------------------------------------------------------- */
+int xlite_hip_quantize_kv_int8(void *stream, const void *src, int8_t *dst, float *scales,
+                               uint64_t rows, uint32_t head_dim, int dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XLITE_HIP_H_ */

@@ -1,0 +1,448 @@
+"""CPU oracle for the Xlite attention hot path.
+
+TEST INFRASTRUCTURE ONLY. Nothing in the shipped package may import this
+module; it is the checker for the HIP kernels (tests, the smoke check and the
+CPU-baseline leg of the benchmark), never the thing measured or shipped.
+
+Every function restates, in plain PyTorch on CPU tensors, the arithmetic of one
+piece of the reference (paths under /root/reference/):
+
+  rope_and_cache_ref   xlite/tests/kernels/rope_and_cache.py:27-41,84-103 (golden) with the
+                       rounding order and cache write of
+                       xlite/csrc/kernels/rope_and_cache.h:93-129,486-501,563-600
+  gather_paged         xlite/tests/kernels/attention.py:186-220 (paged layout),
+                       xlite/csrc/kernels/attention.h:147,156
+  attention_ref        xlite/tests/kernels/attention.py:109-117,139-184;
+                       xlite/tests/models/llama.py:207-259
+  mla_attention_ref    xlite/tests/kernels/mla.py:163-202, top-k mask :293-333;
+                       xlite/tests/models/deepseek_v3.py:675-690
+  mla_v2_ref           xlite/csrc/_C.cpp:1234-1301 (einsum + attention + einsum)
+  mla_v3_ref           xlite/tests/kernels/mla_v3.py:163-192; xlite/csrc/kernels/mla_v3.h:534-536
+  gather_sparse_kv_cache_ref  xlite/tests/kernels/gather_sparse_kv_cache.py:102-116
+  rope_complex_ref     xlite/tests/kernels/rope_complex.py:31-41 with the fp32 operation order of
+                       xlite/csrc/kernels/rope_complex_and_cache.h:165-205
+  mla_prepare_ref      xlite/tests/kernels/mla_prepare.py:27-45,90-109
+  einsum_ref           xlite/tests/kernels/einsum_mht_mhd.py:44
+  prepare_attn_ref     xlite/csrc/runtime.cpp:438-534
+  get_tile_size_of_cached_kv_ref  xlite/csrc/auto_tuner.cpp:10-210
+  quantize_kv_int8 / dequantize_kv_int8   not in the reference (its caches are never
+                       quantised); definition from the benchmark contract:
+                       scale = absmax/127 per (token, kv head), symmetric.
+
+Pinning status (what independent evidence each function is checked against in
+tests/test_oracle_pins.py):
+  attention_ref, mla_attention_ref, mla_v3_ref: fp64 triple-loop C restatement
+      (oracle/brute.c), torch scaled_dot_product_attention on gathered dense K/V,
+      closed forms (single key -> v0; equal keys -> mean of V), block-permutation
+      invariance, prefill rows == the same rows issued as decode steps, absorbed
+      MLA == naive per-head MLA in fp64.
+  rope_and_cache_ref, rope_complex_ref: C restatement with explicit bf16/fp16
+      rounding (oracle/brute.c), rotation by position 0 is the identity, norm
+      preservation, complex-multiply identity in fp64.
+  mla_prepare_ref: composition of the two pinned pieces + RMSNorm closed forms.
+  gather_*: brute-force Python loops.
+  get_tile_size_of_cached_kv_ref, prepare_attn_ref: hand-computed cases.
+  int8 KV: parity unpinned by the reference (feature absent there); pinned only by
+      the round-trip bound |x - dequant(quant(x))| <= scale/2.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+MAX_KV_TILE_SIZE = 8192          # xlite/csrc/auto_tuner.h:13
+MIN_KV_TILE_SIZE = 4096          # xlite/csrc/auto_tuner.h:12
+SINGLE_BATCH_MIN_KV_TILE_SIZE = 1024  # xlite/csrc/auto_tuner.h:11
+XLITE_MAX_M0 = 128               # xlite/csrc/kernels/kernel_param.h:33
+
+
+# --------------------------------------------------------------------------
+# paged layout
+# --------------------------------------------------------------------------
+def gather_paged(cache: torch.Tensor, table_row: Sequence[int], n_tokens: int) -> torch.Tensor:
+    """Tokens 0..n_tokens-1 of one sequence: token p lives at cache[table[p // bs], p % bs]."""
+    bs = cache.shape[1]
+    nblk = (n_tokens + bs - 1) // bs
+    idx = torch.as_tensor(list(table_row[:nblk]), dtype=torch.long)
+    flat = cache[idx].reshape(nblk * bs, *cache.shape[2:])
+    return flat[:n_tokens]
+
+
+# --------------------------------------------------------------------------
+# rope_and_cache
+# --------------------------------------------------------------------------
+def _neox_rotate(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, rot_dim: int) -> torch.Tensor:
+    """x [T, H, D] in fp16/bf16; cos/sin [T, rot_dim/2] same dtype. Each product is rounded to
+    the storage dtype before the add/sub, then the sum is rounded again."""
+    dt = x.dtype
+    half = rot_dim // 2
+    x1 = x[..., :half].float()
+    x2 = x[..., half:rot_dim].float()
+    c = cos.float().unsqueeze(1)
+    s = sin.float().unsqueeze(1)
+    a = (x1 * c).to(dt).float()
+    b = (x2 * s).to(dt).float()
+    e = (x2 * c).to(dt).float()
+    f = (x1 * s).to(dt).float()
+    out = x.clone()
+    out[..., :half] = (a - b).to(dt)
+    out[..., half:rot_dim] = (e + f).to(dt)
+    return out
+
+
+def rope_and_cache_ref(inout, k_cache, v_cache, position, cosin, slot_mapping, n_heads, n_kv_heads,
+                       head_dim, rot_dim, block_size, mrope_mask_h: int = 0, mrope_mask_w: int = 0):
+    """In place on CPU tensors, same contract as the operator."""
+    T = inout.shape[0]
+    dt = inout.dtype
+    half = rot_dim // 2
+    row = inout.view(T, n_heads + 2 * n_kv_heads, head_dim)
+    q = row[:, :n_heads]
+    k = row[:, n_heads:n_heads + n_kv_heads]
+    v = row[:, n_heads + n_kv_heads:]
+    if mrope_mask_h or mrope_mask_w:
+        pos = position.view(3, T).long()
+        cs_t, cs_h, cs_w = cosin[pos[0]], cosin[pos[1]], cosin[pos[2]]
+        lane = torch.arange(half)
+        in_h = torch.tensor([(mrope_mask_h >> int(j)) & 1 for j in lane], dtype=torch.bool)
+        in_w = torch.tensor([(mrope_mask_w >> int(j)) & 1 for j in lane], dtype=torch.bool)
+        cos = torch.where(in_h, cs_h[:, :half], torch.where(in_w, cs_w[:, :half], cs_t[:, :half]))
+        sin = torch.where(in_h, cs_h[:, half:], torch.where(in_w, cs_w[:, half:], cs_t[:, half:]))
+    else:
+        cs = cosin[position.view(-1).long()]
+        cos, sin = cs[:, :half], cs[:, half:]
+    k_new = _neox_rotate(k, cos, sin, rot_dim)
+    q_new = _neox_rotate(q, cos, sin, rot_dim)
+    scale = 1.0 / math.sqrt(float(head_dim))
+    if dt == torch.float16:
+        # the fp16 kernel multiplies by the scale rounded to fp16 (rope_and_cache.h:219,595)
+        scale_t = torch.tensor(scale, dtype=torch.float32).to(torch.float16).float()
+    else:
+        scale_t = torch.tensor(scale, dtype=torch.float32)
+    q_new = (q_new.float() * scale_t).to(dt)
+    slots = slot_mapping.view(-1).long() & 0xFFFFFFFF
+    blk = slots // block_size
+    off = slots % block_size
+    for t in range(T):  # sequential: a later token wins on duplicate slots
+        k_cache[blk[t], off[t]] = k_new[t]
+        v_cache[blk[t], off[t]] = v[t]
+    k.copy_(k_new)
+    q.copy_(q_new)
+
+
+# --------------------------------------------------------------------------
+# attention
+# --------------------------------------------------------------------------
+def causal_mask(qlen: int, clen: int) -> torch.Tensor:
+    """[qlen, clen + qlen] additive mask: column j is visible to row r iff j <= clen + r."""
+    cols = torch.arange(clen + qlen).unsqueeze(0)
+    rows = torch.arange(qlen).unsqueeze(1)
+    m = torch.zeros(qlen, clen + qlen, dtype=torch.float32)
+    m[cols > clen + rows] = float("-inf")
+    return m
+
+
+def attention_ref(qkv, k_cache, v_cache, query_start_loc, lens, cached_lens, block_tables, n_heads,
+                  n_kv_heads, head_dim, block_size, batch, max_num_block,
+                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                  seqs: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Returns fp32 [T, n_heads*head_dim] (rows of sequences not in `seqs` stay zero).
+
+    fp32 accumulation from the 16-bit inputs; no softmax scale (q is pre-scaled). With
+    k_scale/v_scale the caches are int8 and are dequantised first.
+    """
+    T = qkv.shape[0]
+    g = n_heads // n_kv_heads
+    out = torch.zeros(T, n_heads * head_dim, dtype=torch.float32)
+    qsl = [int(x) for x in query_start_loc]
+    ql = [int(x) for x in lens]
+    cl = [int(x) for x in cached_lens]
+    tables = block_tables.view(batch, max_num_block)
+    q_all = qkv.view(T, n_heads + 2 * n_kv_heads, head_dim)[:, :n_heads]
+    for i in (range(batch) if seqs is None else seqs):
+        qlen, clen, st = ql[i], cl[i], qsl[i]
+        if qlen == 0:
+            continue
+        n = clen + qlen
+        row = tables[i].tolist()
+        keys = gather_paged(k_cache, row, n).float()
+        vals = gather_paged(v_cache, row, n).float()
+        if k_scale is not None:
+            keys = keys * gather_paged(k_scale, row, n).float().unsqueeze(-1)
+            vals = vals * gather_paged(v_scale, row, n).float().unsqueeze(-1)
+        q = q_all[st:st + qlen].float()                       # [qlen, nH, d]
+        keys = keys.repeat_interleave(g, dim=1)                # [n, nH, d]
+        vals = vals.repeat_interleave(g, dim=1)
+        scores = torch.einsum("qhd,nhd->hqn", q, keys) + causal_mask(qlen, clen).unsqueeze(0)
+        probs = torch.softmax(scores, dim=-1)
+        o = torch.einsum("hqn,nhd->qhd", probs, vals)
+        out[st:st + qlen] = o.reshape(qlen, n_heads * head_dim)
+    return out
+
+
+# --------------------------------------------------------------------------
+# MLA
+# --------------------------------------------------------------------------
+def mla_attention_ref(q_absorb, qr, k_cache, pe_cache, query_start_loc, lens, cached_lens,
+                      block_tables, n_heads, rope_head_dim, kv_lora_rank, block_size, batch,
+                      max_num_blocks, scale, topk_indices: Optional[torch.Tensor] = None,
+                      top_k: int = 0, seqs: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Absorbed MLA attention, fp32 [T, n_heads, kv_lora_rank]."""
+    T = q_absorb.shape[0]
+    out = torch.zeros(T, n_heads, kv_lora_rank, dtype=torch.float32)
+    qa = q_absorb.view(T, n_heads, kv_lora_rank)
+    qrr = qr.view(T, n_heads, rope_head_dim)
+    kc = k_cache.view(k_cache.shape[0], block_size, kv_lora_rank)
+    pc = pe_cache.view(pe_cache.shape[0], block_size, rope_head_dim)
+    tables = block_tables.view(batch, max_num_blocks)
+    for i in (range(batch) if seqs is None else seqs):
+        qlen, clen, st = int(lens[i]), int(cached_lens[i]), int(query_start_loc[i])
+        if qlen == 0:
+            continue
+        n = clen + qlen
+        row = tables[i].tolist()
+        lat = gather_paged(kc, row, n).float()
+        pe = gather_paged(pc, row, n).float()
+        s = torch.einsum("qhc,nc->qhn", qa[st:st + qlen].float(), lat)
+        s = s + torch.einsum("qhr,nr->qhn", qrr[st:st + qlen].float(), pe)
+        s = s * scale + causal_mask(qlen, clen).unsqueeze(1)
+        if top_k > 0:
+            idx = topk_indices.view(T, top_k)[st:st + qlen].long()
+            keep = torch.full((qlen, n), float("-inf"))
+            keep.scatter_(1, idx.clamp(max=n - 1), 0.0)
+            s = s + keep.unsqueeze(1)
+        p = torch.softmax(s, dim=-1)
+        p = torch.nan_to_num(p, nan=0.0)  # a row with no visible key yields zeros
+        out[st:st + qlen] = torch.einsum("qhn,nc->qhc", p, lat)
+    return out
+
+
+def einsum_ref(mht: torch.Tensor, w: torch.Tensor, w_is_hdt: bool = False) -> torch.Tensor:
+    """fp32 result of einsum('mht,htd->mhd') (or 'mht,hdt->mhd')."""
+    if w_is_hdt:
+        return torch.einsum("mht,hdt->mhd", mht.float(), w.float())
+    return torch.einsum("mht,htd->mhd", mht.float(), w.float())
+
+
+def mla_v2_ref(q_with_qr, qr, k_cache, pe_cache, wuk_t, wuv, query_start_loc, lens, cached_lens,
+               block_tables, n_heads, rope_head_dim, nope_head_dim, v_head_dim, kv_lora_rank,
+               block_size, batch, max_num_blocks, scale, topk_indices=None, top_k=0,
+               round_intermediates: bool = True) -> torch.Tensor:
+    """The three-stage operator. The reference stores q_absorb and o_absorb in the activation
+    dtype between stages (xlite/csrc/_C.cpp:1257-1262), which `round_intermediates` reproduces."""
+    T = q_with_qr.shape[0]
+    dt = q_with_qr.dtype
+    q_nope = q_with_qr.view(T, n_heads, nope_head_dim + rope_head_dim)[..., :nope_head_dim]
+    q_abs = einsum_ref(q_nope, wuk_t.view(n_heads, nope_head_dim, kv_lora_rank))
+    if round_intermediates:
+        q_abs = q_abs.to(dt)
+    o_abs = mla_attention_ref(q_abs, qr, k_cache, pe_cache, query_start_loc, lens, cached_lens,
+                              block_tables, n_heads, rope_head_dim, kv_lora_rank, block_size, batch,
+                              max_num_blocks, scale, topk_indices, top_k)
+    if round_intermediates:
+        o_abs = o_abs.to(dt)
+    return einsum_ref(o_abs, wuv.view(n_heads, kv_lora_rank, v_head_dim))
+
+
+def mla_v3_ref(q_absorb, qr, k_dense, pe_dense, query_start_loc, lens, cached_lens, n_heads,
+               rope_head_dim, kv_lora_rank, batch, index_topk, scale) -> torch.Tensor:
+    T = q_absorb.shape[0]
+    out = torch.zeros(T, n_heads, kv_lora_rank, dtype=torch.float32)
+    qa = q_absorb.view(T, n_heads, kv_lora_rank)
+    qrr = qr.view(T, n_heads, rope_head_dim)
+    kd = k_dense.view(batch, index_topk, kv_lora_rank)
+    pd = pe_dense.view(batch, index_topk, rope_head_dim)
+    for i in range(batch):
+        qlen, clen, st = int(lens[i]), int(cached_lens[i]), int(query_start_loc[i])
+        n = min(clen + qlen, index_topk)
+        if qlen == 0 or n <= 0:
+            continue
+        lat = kd[i, :n].float()
+        pe = pd[i, :n].float()
+        s = torch.einsum("qhc,nc->qhn", qa[st:st + qlen].float(), lat)
+        s = (s + torch.einsum("qhr,nr->qhn", qrr[st:st + qlen].float(), pe)) * scale
+        p = torch.softmax(s, dim=-1)
+        out[st:st + qlen] = torch.einsum("qhn,nc->qhc", p, lat)
+    return out
+
+
+def gather_sparse_kv_cache_ref(k_cache, pe_cache, block_tables, topk_indices, query_lens,
+                               cached_lens, k_dense, pe_dense, batch, index_topk, block_size,
+                               max_num_blocks, kv_lora_rank, rope_head_dim):
+    """In place; slots beyond min(qlen + clen, index_topk) are not touched."""
+    kc = k_cache.view(-1, block_size, kv_lora_rank)
+    pc = pe_cache.view(-1, block_size, rope_head_dim)
+    kd = k_dense.view(batch, index_topk, kv_lora_rank)
+    pd = pe_dense.view(batch, index_topk, rope_head_dim)
+    tables = block_tables.view(batch, max_num_blocks)
+    idx = topk_indices.view(batch, index_topk)
+    for b in range(batch):
+        valid = min(int(query_lens[b]) + int(cached_lens[b]), index_topk)
+        for i in range(valid):
+            tok = int(idx[b, i])
+            phys = int(tables[b, tok // block_size])
+            kd[b, i] = kc[phys, tok % block_size]
+            pd[b, i] = pc[phys, tok % block_size]
+
+
+# --------------------------------------------------------------------------
+# rope_complex / mla_prepare
+# --------------------------------------------------------------------------
+def _freqs_as_cos_sin(freqs: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    f = torch.view_as_real(freqs) if freqs.is_complex() else freqs.view(freqs.shape[0], -1, 2)
+    return f[..., 0].float(), f[..., 1].float()
+
+
+def _rope_interleaved(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [..., rope_dim] interleaved (re, im) pairs in fp32; cos/sin broadcastable [..., rope_dim/2].
+    Four fp32 products, one fp32 add/sub each, output [re... | im...] (still fp32)."""
+    xe = x[..., 0::2]
+    xo = x[..., 1::2]
+    re = xe * cos - xo * sin     # torch evaluates the two products separately, then subtracts
+    im = xe * sin + xo * cos
+    return torch.cat([re, im], dim=-1)
+
+
+def rope_complex_ref(n_local_heads, step_dim, rope_dim, input_with_r, freqs, position):
+    """Returns [T, n_local_heads, rope_dim] in the input dtype."""
+    T = input_with_r.shape[0]
+    dt = input_with_r.dtype
+    x = input_with_r.view(T, n_local_heads, step_dim)[..., step_dim - rope_dim:].float()
+    cos, sin = _freqs_as_cos_sin(freqs)
+    pos = position.view(-1).long()
+    y = _rope_interleaved(x, cos[pos].unsqueeze(1), sin[pos].unsqueeze(1))
+    return y.to(dt)
+
+
+def rmsnorm_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float) -> torch.Tensor:
+    xf = x.float()
+    var = xf.pow(2).mean(-1, keepdim=True)
+    y = xf * torch.rsqrt(var + eps)
+    return (weight.float() * y + bias.float()).to(x.dtype)
+
+
+def mla_prepare_ref(attn_qkvc, q_norm, q_norm_bias, attn_norm_qc, kv_norm, kv_norm_bias,
+                    attn_norm_kvc, freqs, position, q_lora_rank, kv_lora_rank, rope_head_dim,
+                    block_size, k_cache, pe_cache, slot_mapping, norm_eps):
+    """In place on CPU tensors."""
+    T = attn_qkvc.shape[0]
+    dt = attn_qkvc.dtype
+    rows = attn_qkvc.view(T, q_lora_rank + kv_lora_rank + rope_head_dim)
+    attn_norm_qc.view(T, q_lora_rank).copy_(rmsnorm_ref(rows[:, :q_lora_rank], q_norm, q_norm_bias, norm_eps))
+    kvc = rmsnorm_ref(rows[:, q_lora_rank:q_lora_rank + kv_lora_rank], kv_norm, kv_norm_bias, norm_eps)
+    attn_norm_kvc.view(T, kv_lora_rank).copy_(kvc)
+    cos, sin = _freqs_as_cos_sin(freqs)
+    pos = position.view(-1).long()
+    pe = _rope_interleaved(rows[:, q_lora_rank + kv_lora_rank:].float(), cos[pos], sin[pos]).to(dt)
+    rows[:, q_lora_rank + kv_lora_rank:] = pe
+    if block_size:
+        kc = k_cache.view(-1, block_size, kv_lora_rank)
+        pc = pe_cache.view(-1, block_size, rope_head_dim)
+        slots = slot_mapping.view(-1).long() & 0xFFFFFFFF
+        for t in range(T):
+            kc[slots[t] // block_size, slots[t] % block_size] = kvc[t]
+            pc[slots[t] // block_size, slots[t] % block_size] = pe[t]
+
+
+# --------------------------------------------------------------------------
+# host metadata
+# --------------------------------------------------------------------------
+def prepare_attn_ref(lens: Sequence[int], cached_lens: Sequence[int],
+                     block_tables: Sequence[Sequence[int]], block_size: int):
+    batch = len(lens)
+    if batch == 0:
+        raise RuntimeError("invalid batchSize: 0")
+    qsl, pos, slots, nblk = [], [], [], []
+    start = 0
+    for i in range(batch):
+        qsl.append(start)
+        start += lens[i]
+        nblk.append((lens[i] + cached_lens[i] + block_size - 1) // block_size)
+    max_nb = max(nblk)
+    for i in range(batch):
+        if len(block_tables[i]) < nblk[i]:
+            raise RuntimeError("block table too small")
+        for j in range(lens[i]):
+            p = cached_lens[i] + j
+            pos.append(p)
+            slots.append(block_tables[i][p // block_size] * block_size + p % block_size)
+    dense = np.zeros((batch, max_nb), dtype=np.int32)
+    for i in range(batch):
+        dense[i, :nblk[i]] = block_tables[i][:nblk[i]]
+    return dict(query_start_loc=qsl, position=pos, slot_mapping=slots, block_tables=dense,
+                max_num_blocks=max_nb, batched_tokens=start,
+                is_decode=all(l == 1 for l in lens))
+
+
+def _calc_task_num(clen, qlen, g, n_kv, tile):
+    qtile = XLITE_MAX_M0 // g
+    if qtile == 0:
+        qtile = XLITE_MAX_M0
+    qnum = (qlen + qtile - 1) // qtile
+    kvnum = (clen + qlen + tile - 1) // tile
+    valid = 0
+    for idx in range(qnum * n_kv * kvnum):
+        kvidx = idx % kvnum
+        qidx = idx // (kvnum * n_kv)
+        qstart = qidx * qtile
+        qtl = min(qtile, qlen - qstart)
+        if clen + qstart + qtl > kvidx * tile:
+            valid += 1
+    return valid
+
+
+def get_tile_size_of_cached_kv_ref(cached_lens: List[int], query_lens: List[int],
+                                   head_num_in_group: int, n_kv_heads: int, block_size: int,
+                                   aic_num: int) -> int:
+    f32 = np.float32
+    if any(q != 1 for q in query_lens):
+        return 6016 if aic_num == 24 else 8192
+    batch = len(query_lens)
+    if batch == 1:
+        clen = float(cached_lens[0])
+        tasks = int(round(1.5 * math.sqrt(clen / 1024.0) + 3))
+        tasks = max(1, min(tasks, aic_num))
+        tile = (int(math.ceil(clen)) + tasks - 1) // tasks
+        tile = (tile + block_size - 1) // block_size * block_size
+        return max(SINGLE_BATCH_MIN_KV_TILE_SIZE, min(tile, MAX_KV_TILE_SIZE))
+    best, best_score = MAX_KV_TILE_SIZE, f32(-1.0)
+    tile = MAX_KV_TILE_SIZE
+    while tile >= MIN_KV_TILE_SIZE:
+        tot, cnt, total_tasks = f32(0.0), 0, 0
+        for c, q in zip(cached_lens, query_lens):
+            kv = c + q
+            if kv == 1:
+                continue
+            rem = kv % tile
+            tot = f32(tot + (f32(1.0) if rem == 0 else f32(rem) / f32(tile)))
+            cnt += 1
+            total_tasks += _calc_task_num(c, q, head_num_in_group, n_kv_heads, tile)
+        kv_score = f32(0.0) if cnt == 0 else f32(tot / f32(cnt))
+        rem = total_tasks % aic_num
+        task_score = f32(1.0) if rem == 0 else f32(rem) / f32(aic_num)
+        size_score = f32(tile) / f32(MAX_KV_TILE_SIZE)
+        score = f32(f32(f32(kv_score * f32(0.7)) + f32(task_score * f32(0.2))) + f32(size_score * f32(0.1)))
+        if score > best_score:
+            best_score, best = score, tile
+        tile -= block_size
+    return best
+
+
+# --------------------------------------------------------------------------
+# int8 KV cache
+# --------------------------------------------------------------------------
+def quantize_kv_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [..., head_dim] -> (int8 same shape, fp32 scale [...]); scale = absmax/127."""
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1)
+    scale = amax / 127.0
+    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+    q = torch.clamp(torch.round(xf / safe.unsqueeze(-1)), -127, 127).to(torch.int8)
+    return q, scale
+
+
+def dequantize_kv_int8(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    return q.float() * scale.unsqueeze(-1)

@@ -1,0 +1,301 @@
+"""Pins for the CPU oracle: every check here is independent of the oracle's own formula
+(brute-force fp64 C loops, closed forms, library routines, invariances)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import brute
+from oracle import xlite_oracle as O
+
+
+def _paged_case(seed, batch, lens, clens, nH, nKV, d, bs, dtype, permute=True):
+    g = torch.Generator().manual_seed(seed)
+    T = sum(lens)
+    maxblk = max((l + c + bs - 1) // bs for l, c in zip(lens, clens))
+    NB = batch * maxblk + 3
+    qkv = (torch.randn(T, (nH + 2 * nKV) * d, generator=g) * 0.5).to(dtype)
+    kc = torch.randn(NB, bs, nKV, d, generator=g).to(dtype)
+    vc = torch.randn(NB, bs, nKV, d, generator=g).to(dtype)
+    perm = torch.randperm(NB, generator=g) if permute else torch.arange(NB)
+    tables = perm[: batch * maxblk].to(torch.int32).view(batch, maxblk)
+    qsl = np.cumsum([0] + lens[:-1]).tolist()
+    return qkv, kc, vc, qsl, tables, maxblk, T
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nH,nKV,d", [(4, 2, 64), (5, 1, 128), (2, 2, 32)])
+def test_attention_vs_fp64_bruteforce(dtype, nH, nKV, d):
+    bs = 16
+    lens, clens = [1, 7, 3], [37, 0, 20]
+    qkv, kc, vc, qsl, tables, maxblk, T = _paged_case(1, 3, lens, clens, nH, nKV, d, bs, dtype)
+    ref = brute.attention(qkv, kc, vc, qsl, lens, clens, tables.flatten(), nH, nKV, d, bs, 3, maxblk)
+    got = O.attention_ref(qkv, kc, vc, qsl, lens, clens, tables.flatten(), nH, nKV, d, bs, 3, maxblk)
+    assert torch.allclose(got.double(), ref, atol=2e-5, rtol=1e-4)
+
+
+def test_attention_vs_torch_sdpa():
+    """Library cross-check: dense K/V gathered by hand, torch's own fused attention."""
+    nH, nKV, d, bs = 6, 2, 64, 8
+    lens, clens = [5], [11]
+    qkv, kc, vc, qsl, tables, maxblk, T = _paged_case(2, 1, lens, clens, nH, nKV, d, bs, torch.bfloat16)
+    n = 16
+    keys = torch.stack([kc[tables[0, p // bs], p % bs] for p in range(n)]).float()
+    vals = torch.stack([vc[tables[0, p // bs], p % bs] for p in range(n)]).float()
+    q = qkv.view(T, nH + 2 * nKV, d)[:, :nH].float().transpose(0, 1).unsqueeze(0)  # [1,nH,q,d]
+    k = keys.repeat_interleave(nH // nKV, 1).transpose(0, 1).unsqueeze(0)
+    v = vals.repeat_interleave(nH // nKV, 1).transpose(0, 1).unsqueeze(0)
+    allowed = torch.arange(n).unsqueeze(0) <= (11 + torch.arange(5)).unsqueeze(1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=allowed, scale=1.0)
+    ref = ref[0].transpose(0, 1).reshape(T, nH * d)
+    got = O.attention_ref(qkv, kc, vc, qsl, lens, clens, tables.flatten(), nH, nKV, d, bs, 1, maxblk)
+    assert torch.allclose(got, ref, atol=2e-5, rtol=1e-4)
+
+
+def test_attention_closed_forms():
+    nH, nKV, d, bs = 4, 2, 32, 4
+    # a single visible key: the output is exactly v0 of the matching kv head
+    qkv, kc, vc, qsl, tables, maxblk, T = _paged_case(3, 1, [1], [0], nH, nKV, d, bs, torch.bfloat16)
+    got = O.attention_ref(qkv, kc, vc, qsl, [1], [0], tables.flatten(), nH, nKV, d, bs, 1, maxblk)
+    v0 = vc[tables[0, 0], 0].float().repeat_interleave(nH // nKV, 0).reshape(1, nH * d)
+    assert torch.equal(got, v0)
+    # all keys equal: uniform probabilities, output = mean of V
+    qkv, kc, vc, qsl, tables, maxblk, T = _paged_case(4, 1, [1], [9], nH, nKV, d, bs, torch.bfloat16)
+    kc[:] = kc[0, 0]
+    got = O.attention_ref(qkv, kc, vc, qsl, [1], [9], tables.flatten(), nH, nKV, d, bs, 1, maxblk)
+    vals = torch.stack([vc[tables[0, p // bs], p % bs] for p in range(10)]).float().mean(0)
+    assert torch.allclose(got, vals.repeat_interleave(nH // nKV, 0).reshape(1, -1), atol=1e-6)
+
+
+def test_attention_block_permutation_invariance_and_decode_equivalence():
+    nH, nKV, d, bs = 4, 1, 64, 8
+    lens, clens = [6], [13]
+    qkv, kc, vc, qsl, tables, maxblk, T = _paged_case(5, 1, lens, clens, nH, nKV, d, bs, torch.bfloat16)
+    a = O.attention_ref(qkv, kc, vc, qsl, lens, clens, tables.flatten(), nH, nKV, d, bs, 1, maxblk)
+    # identity table over a re-packed cache gives bit-identical results
+    ident = torch.arange(maxblk, dtype=torch.int32)
+    kc2, vc2 = kc[tables[0].long()].clone(), vc[tables[0].long()].clone()
+    b = O.attention_ref(qkv, kc2, vc2, qsl, lens, clens, ident, nH, nKV, d, bs, 1, maxblk)
+    assert torch.equal(a, b)
+    # each prefill row equals the same row issued alone as a decode step
+    for r in range(6):
+        one = O.attention_ref(qkv[r:r + 1], kc, vc, [0], [1], [13 + r], tables.flatten(), nH, nKV,
+                              d, bs, 1, maxblk)
+        assert torch.allclose(one[0], a[r], atol=1e-6)
+
+
+def _mla_case(seed, lens, clens, nH, R, C, bs):
+    g = torch.Generator().manual_seed(seed)
+    batch, T = len(lens), sum(lens)
+    maxblk = max((l + c + bs - 1) // bs for l, c in zip(lens, clens))
+    NB = batch * maxblk + 2
+    qa = (torch.randn(T, nH, C, generator=g) * 0.3).bfloat16()
+    qr = (torch.randn(T, nH, R, generator=g) * 0.3).bfloat16()
+    kc = torch.randn(NB, bs, C, generator=g).bfloat16()
+    pc = torch.randn(NB, bs, R, generator=g).bfloat16()
+    tables = torch.randperm(NB, generator=g)[: batch * maxblk].to(torch.int32)
+    qsl = np.cumsum([0] + lens[:-1]).tolist()
+    return qa, qr, kc, pc, qsl, tables, maxblk, T
+
+
+def test_mla_vs_fp64_bruteforce_dense_and_topk():
+    nH, R, C, bs = 3, 8, 32, 8
+    lens, clens = [1, 5], [20, 3]
+    qa, qr, kc, pc, qsl, tables, maxblk, T = _mla_case(6, lens, clens, nH, R, C, bs)
+    scale = 0.17
+    ref = brute.mla(qa, qr, kc, pc, qsl, lens, clens, tables, nH, R, C, bs, 2, maxblk, scale)
+    got = O.mla_attention_ref(qa, qr, kc, pc, qsl, lens, clens, tables, nH, R, C, bs, 2, maxblk, scale)
+    assert torch.allclose(got.double(), ref, atol=2e-5, rtol=1e-4)
+    g = torch.Generator().manual_seed(7)
+    top_k = 4
+    topk = torch.stack([torch.sort(torch.randperm(8, generator=g)[:top_k]).values for _ in range(T)]).int()
+    ref = brute.mla(qa, qr, kc, pc, qsl, lens, clens, tables, nH, R, C, bs, 2, maxblk, scale, topk, top_k)
+    got = O.mla_attention_ref(qa, qr, kc, pc, qsl, lens, clens, tables, nH, R, C, bs, 2, maxblk,
+                              scale, topk, top_k)
+    assert torch.allclose(got.double(), ref, atol=2e-5, rtol=1e-4)
+
+
+def test_mla_absorbed_equals_naive_per_head_fp64():
+    """The absorbed form must equal the textbook per-head MLA (k = W_UK latent, v = W_UV^T latent)."""
+    g = torch.Generator().manual_seed(8)
+    nH, nope, rope, vdim, C, n = 2, 6, 4, 5, 8, 9
+    q_nope = torch.randn(1, nH, nope, generator=g, dtype=torch.float64)
+    q_rope = torch.randn(1, nH, rope, generator=g, dtype=torch.float64)
+    lat = torch.randn(n, C, generator=g, dtype=torch.float64)
+    pe = torch.randn(n, rope, generator=g, dtype=torch.float64)
+    wuk_t = torch.randn(nH, nope, C, generator=g, dtype=torch.float64)   # [h, nope, C]
+    wuv = torch.randn(nH, C, vdim, generator=g, dtype=torch.float64)     # [h, C, v]
+    scale = (nope + rope) ** -0.5
+    k_nope = torch.einsum("nc,hdc->nhd", lat, wuk_t)
+    v = torch.einsum("nc,hcv->nhv", lat, wuv)
+    s = (torch.einsum("qhd,nhd->hqn", q_nope, k_nope) + torch.einsum("qhr,nr->hqn", q_rope, pe)) * scale
+    naive = torch.einsum("hqn,nhv->qhv", torch.softmax(s, -1), v)
+    # run the oracle on values that are exact in bf16 so no rounding enters
+    def exact(x):
+        return (x * 4).round().div(4).clamp(-3, 3)
+    q_nope, q_rope, lat, pe, wuk_t, wuv = map(exact, (q_nope, q_rope, lat, pe, wuk_t, wuv))
+    k_nope = torch.einsum("nc,hdc->nhd", lat, wuk_t)
+    v = torch.einsum("nc,hcv->nhv", lat, wuv)
+    s = (torch.einsum("qhd,nhd->hqn", q_nope, k_nope) + torch.einsum("qhr,nr->hqn", q_rope, pe)) * scale
+    naive = torch.einsum("hqn,nhv->qhv", torch.softmax(s, -1), v)
+    qwq = torch.cat([q_nope, q_rope], -1).bfloat16()
+    kc = torch.zeros(2, 8, C).bfloat16(); pc = torch.zeros(2, 8, rope).bfloat16()
+    kc.view(16, C)[:n] = lat.bfloat16(); pc.view(16, rope)[:n] = pe.bfloat16()
+    out = O.mla_v2_ref(qwq, q_rope.bfloat16(), kc, pc, wuk_t.bfloat16(), wuv.bfloat16(), [0], [1],
+                       [n - 1], torch.tensor([0, 1], dtype=torch.int32), nH, rope, nope, vdim, C, 8,
+                       1, 2, scale, round_intermediates=False)
+    assert torch.allclose(out.double(), naive, atol=1e-5, rtol=1e-5)
+
+
+def test_mla_v3_matches_dense_prefix_of_paged():
+    nH, R, C, bs = 2, 8, 16, 4
+    qa, qr, kc, pc, qsl, tables, maxblk, T = _mla_case(9, [1], [10], nH, R, C, bs)
+    topk = 16
+    kd = torch.zeros(1, topk, C).bfloat16(); pd = torch.zeros(1, topk, R).bfloat16()
+    idx = torch.arange(topk, dtype=torch.int32).clamp(max=10).view(1, topk)
+    O.gather_sparse_kv_cache_ref(kc, pc, tables, idx, [1], [10], kd, pd, 1, topk, bs, maxblk, C, R)
+    assert torch.equal(kd[0, 11:], torch.zeros(5, C).bfloat16())       # padding tail untouched
+    a = O.mla_v3_ref(qa, qr, kd, pd, [0], [1], [10], nH, R, C, 1, topk, 0.3)
+    b = O.mla_attention_ref(qa, qr, kc, pc, [0], [1], [10], tables, nH, R, C, bs, 1, maxblk, 0.3)
+    assert torch.allclose(a, b, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d,rot", [(64, 64), (128, 128), (128, 64)])
+def test_rope_and_cache_bit_exact_vs_c(dtype, d, rot):
+    g = torch.Generator().manual_seed(10)
+    T, nH, nKV, bs, NB = 9, 3, 2, 4, 5
+    inout = torch.randn(T, (nH + 2 * nKV) * d, generator=g).to(dtype)
+    kc = torch.full((NB, bs, nKV, d), 7.0).to(dtype); vc = torch.full((NB, bs, nKV, d), -7.0).to(dtype)
+    fr = torch.outer(torch.arange(32).float(), 1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot)))
+    cosin = torch.cat([fr.cos(), fr.sin()], -1).to(dtype)
+    pos = torch.randint(0, 32, (T,), generator=g)
+    slots = torch.randperm(NB * bs, generator=g)[:T].int()
+    a, b, c = brute.rope_and_cache(inout, kc, vc, pos, cosin, slots, nH, nKV, d, rot, bs)
+    O.rope_and_cache_ref(inout, kc, vc, pos, cosin, slots, nH, nKV, d, rot, bs)
+    for x, y in ((a, inout), (b, kc), (c, vc)):
+        assert torch.equal(x.view(torch.int16), y.view(torch.int16))
+    # untouched slots keep their sentinel, touched ones hold the updated k / the raw v
+    touched = torch.zeros(NB * bs, dtype=torch.bool); touched[slots.long()] = True
+    assert torch.equal(kc.view(NB * bs, -1)[~touched], torch.full((NB * bs - T, nKV * d), 7.0).to(dtype))
+    row = inout.view(T, nH + 2 * nKV, d)
+    assert torch.equal(kc.view(NB * bs, nKV, d)[slots.long()], row[:, nH:nH + nKV])
+    assert torch.equal(vc.view(NB * bs, nKV, d)[slots.long()], row[:, nH + nKV:])
+
+
+def test_rope_matches_reference_golden_formula_and_identities():
+    """Same shape as the reference's own golden (rotate_half form, dtype arithmetic)."""
+    g = torch.Generator().manual_seed(11)
+    T, nH, nKV, d, bs = 4, 2, 2, 64, 8
+    x = torch.randn(T, (nH + 2 * nKV) * d, generator=g).bfloat16()
+    fr = torch.outer(torch.arange(16).float(), 1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d)))
+    cosin = torch.cat([fr.cos(), fr.sin()], -1).bfloat16()
+    pos = torch.tensor([0, 3, 7, 15])
+    y = x.clone()
+    kc = torch.zeros(1, bs, nKV, d).bfloat16(); vc = torch.zeros(1, bs, nKV, d).bfloat16()
+    O.rope_and_cache_ref(y, kc, vc, pos, cosin, torch.arange(T).int(), nH, nKV, d, d, bs)
+    xr = x.view(T, nH + 2 * nKV, d); yr = y.view(T, nH + 2 * nKV, d)
+    cos = cosin[pos][:, None, : d // 2].repeat(1, 1, 2); sin = cosin[pos][:, None, d // 2:].repeat(1, 1, 2)
+    k = xr[:, nH:nH + nKV]
+    half = torch.cat([-k[..., d // 2:], k[..., : d // 2]], -1)
+    golden_k = k * cos + half * sin                     # bf16 tensor arithmetic, as in the golden
+    assert torch.equal(yr[:, nH:nH + nKV], golden_k)
+    q = xr[:, :nH]
+    halfq = torch.cat([-q[..., d // 2:], q[..., : d // 2]], -1)
+    golden_q = (q * cos + halfq * sin) * d ** -0.5
+    assert torch.equal(yr[:, :nH], golden_q)
+    assert torch.equal(yr[0, nH:nH + nKV], xr[0, nH:nH + nKV])     # position 0 = identity
+    assert torch.equal(yr[:, nH + nKV:], xr[:, nH + nKV:])         # v is never modified
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rope_complex_vs_c_and_complex_product(dtype):
+    g = torch.Generator().manual_seed(12)
+    T, H, step, rope = 6, 3, 48, 16
+    x = torch.randn(T, H, step, generator=g).to(dtype)
+    ang = torch.outer(torch.arange(20).float(), 1.0 / (10000.0 ** (torch.arange(0, rope, 2).float() / rope)))
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    pos = torch.randint(0, 20, (T,), generator=g)
+    got = O.rope_complex_ref(H, step, rope, x, freqs, pos)
+    ref = brute.rope_complex(x, torch.view_as_real(freqs).reshape(20, rope), pos, H, step, rope)
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    xc = torch.view_as_complex(x[..., step - rope:].double().reshape(T, H, rope // 2, 2))
+    yc = xc * freqs[pos].to(torch.complex128).unsqueeze(1)
+    exact = torch.cat([yc.real, yc.imag], -1)
+    assert torch.allclose(got.double(), exact, atol=0.02, rtol=1e-2)
+    assert torch.allclose(got.double().pow(2).sum(-1), x[..., step - rope:].double().pow(2).sum(-1), rtol=2e-2)
+
+
+def test_rmsnorm_closed_forms_and_mla_prepare_composition():
+    x = torch.full((2, 8), 3.0).bfloat16()
+    out = O.rmsnorm_ref(x, torch.full((8,), 2.0).bfloat16(), torch.full((8,), 0.5).bfloat16(), 0.0)
+    assert torch.equal(out, torch.full((2, 8), 2.5).bfloat16())          # x/rms = 1
+    g = torch.Generator().manual_seed(13)
+    T, ql, kl, rp, bs = 5, 16, 8, 4, 4
+    row = (torch.randn(T, ql + kl + rp, generator=g) / 10).bfloat16()
+    w1, b1 = torch.randn(ql, generator=g).bfloat16(), torch.randn(ql, generator=g).bfloat16()
+    w2, b2 = torch.randn(kl, generator=g).bfloat16(), torch.randn(kl, generator=g).bfloat16()
+    ang = torch.outer(torch.arange(8).float(), 1.0 / (10000.0 ** (torch.arange(0, rp, 2).float() / rp)))
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    pos = torch.tensor([0, 1, 2, 3, 4]); slots = torch.tensor([3, 0, 5, 6, 1]).int()
+    qc = torch.zeros(T, ql).bfloat16(); kvc = torch.zeros(T, kl).bfloat16()
+    kcache = torch.zeros(2, bs, kl).bfloat16(); pcache = torch.zeros(2, bs, rp).bfloat16()
+    before = row.clone()
+    O.mla_prepare_ref(row, w1, b1, qc, w2, b2, kvc, freqs, pos, ql, kl, rp, bs, kcache, pcache, slots, 1e-6)
+    xf = before[:, :ql].double()
+    manual = (xf / (xf.pow(2).mean(-1, keepdim=True) + 1e-6).sqrt()) * w1.double() + b1.double()
+    assert torch.allclose(qc.double(), manual, atol=0.02, rtol=1e-2)
+    assert torch.equal(row[:, :ql + kl], before[:, :ql + kl])
+    assert torch.equal(kcache.view(8, kl)[slots.long()], kvc)
+    assert torch.equal(pcache.view(8, rp)[slots.long()], row[:, ql + kl:])
+    assert torch.equal(row[:, ql + kl:], O.rope_complex_ref(1, rp, rp, before[:, ql + kl:].contiguous(), freqs, pos).view(T, rp))
+
+
+def test_prepare_attn_hand_case():
+    m = O.prepare_attn_ref([3, 1], [5, 9], [[7, 2], [4, 9, 1]], 4)
+    assert m["query_start_loc"] == [0, 3]
+    assert m["position"] == [5, 6, 7, 9]
+    assert m["slot_mapping"] == [2 * 4 + 1, 2 * 4 + 2, 2 * 4 + 3, 1 * 4 + 1]
+    assert m["max_num_blocks"] == 3 and m["batched_tokens"] == 4 and not m["is_decode"]
+    assert m["block_tables"].tolist() == [[7, 2, 0], [4, 9, 1]]
+
+
+def test_tile_size_hand_cases():
+    # prefill -> fixed values by core count (auto_tuner.cpp:177-184)
+    assert O.get_tile_size_of_cached_kv_ref([0], [100], 4, 8, 128, 24) == 6016
+    assert O.get_tile_size_of_cached_kv_ref([0], [100], 4, 8, 128, 20) == 8192
+    # batch 1 decode, cached 65536: tasks = round(1.5*8+3) = 15 -> ceil(65536/15)=4370 -> 4480
+    assert O.get_tile_size_of_cached_kv_ref([65536], [1], 4, 8, 128, 24) == 4480
+    # short context clamps to the 1024 floor
+    assert O.get_tile_size_of_cached_kv_ref([2000], [1], 4, 8, 128, 24) == 1024
+    # batch 2 decode with kv length 8192 each: tile 8192 scores 0.7*1 + 0.2*(16 % 24)/24 + 0.1
+    # and no smaller tile reaches a kv remainder score of 1, so 8192 wins
+    assert O.get_tile_size_of_cached_kv_ref([8191, 8191], [1, 1], 4, 8, 128, 24) == 8192
+
+
+def test_int8_roundtrip_bound():
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(7, 3, 128, generator=g).bfloat16()
+    q, s = O.quantize_kv_int8(x)
+    assert q.dtype == torch.int8 and int(q.abs().max()) == 127
+    err = (O.dequantize_kv_int8(q, s) - x.float()).abs()
+    assert bool((err <= s.unsqueeze(-1) * 0.5 + 1e-7).all())
+    z, sz = O.quantize_kv_int8(torch.zeros(2, 8))
+    assert int(z.abs().max()) == 0 and float(sz.max()) == 0.0
+
+
+def test_fp16_conversions_in_c_match_torch():
+    g = torch.Generator().manual_seed(15)
+    vals = torch.cat([torch.randn(2000, generator=g) * 10 ** torch.randint(-9, 6, (2000,), generator=g).float(),
+                      torch.tensor([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 6e-8, 6.1e-5, float("inf")])])
+    L = brute.lib()
+    for v in vals.tolist():
+        want = torch.tensor(v, dtype=torch.float32).half().view(torch.int16).item() & 0xFFFF
+        assert L.brute_f32_to_f16(v) == want, v
+        wantb = torch.tensor(v, dtype=torch.float32).bfloat16().view(torch.int16).item() & 0xFFFF
+        assert L.brute_f32_to_bf16(v) == wantb, v
+    for h in range(0, 65536, 7):
+        f = L.brute_f16_to_f32(h)
+        t = torch.tensor(h if h < 32768 else h - 65536, dtype=torch.int16).view(torch.float16).float().item()
+        assert (math.isnan(f) and math.isnan(t)) or f == t
