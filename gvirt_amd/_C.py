@@ -1,0 +1,406 @@
+"""Python operator API of the MI355X attention path, with the names, argument order, defaults and
+error behaviour of the reference's `xlite._C` extension (xlite/xlite/_C.pyi) for the attention
+operators: Runtime, rope_and_cache, attention, mla_v2, mla_v3, gather_sparse_kv_cache,
+mla_prepare, rope_complex, einsum_mht_htd_mhd, einsum_mht_hdt_mhd, get_tile_size_of_cached_kv.
+
+Tensors are borrowed for the call and results are written in place, as in the reference
+(xlite/csrc/_C.cpp:174-194). Differences, all deliberate:
+  * contiguity, device and dtype are checked and raise RuntimeError (the reference assumes them);
+  * kernels run on torch's current HIP stream; the call blocks until they finish unless
+    `Runtime.blocking` is set to False (the reference always synchronises, _C.cpp:1182);
+  * `attention` accepts keyword-only `k_scale` / `v_scale` for an int8 KV cache.
+PyTorch is used only to own device memory and streams.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float16: 0, torch.bfloat16: 1}
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _req(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dev(name: str, t: torch.Tensor, dtype=None) -> None:
+    _req(isinstance(t, torch.Tensor), "%s: expected a tensor" % name)
+    _req(t.is_cuda, "%s: expected a GPU tensor, got %s" % (name, t.device))
+    _req(t.is_contiguous(), "%s: tensor must be contiguous" % name)
+    if dtype is not None:
+        _req(t.dtype == dtype, "%s: dtype %s unsupported! (expected %s)" % (name, t.dtype, dtype))
+
+
+def _act_dtype(name: str, *tensors: torch.Tensor) -> int:
+    dt = tensors[0].dtype
+    _req(dt in _DT, "%s: dtype %s unsupported!" % (name, dt))
+    for t in tensors:
+        _req(t.dtype == dt, "%s: mixed dtypes %s / %s unsupported!" % (name, dt, t.dtype))
+    return _DT[dt]
+
+
+class Runtime:
+    """Device + scratch handle passed as first argument of every operator
+    (reference: XRuntime, xlite/csrc/runtime.h:60-229; Python stub _C.pyi:14-94).
+
+    `size` is the initial scratch pool in MB (the reference's tensor pool); the pool holds the
+    split-KV partial results and grows on demand. The parallel-group arguments are accepted for
+    signature compatibility; this build runs on one GPU, so any size other than 1 is refused.
+    """
+
+    def __init__(self, devid: int, size: int = 0, rank: int = 0, tp_size: int = 1, dp_size: int = 1,
+                 moe_tp_size: int = 1, moe_ep_size: int = 1) -> None:
+        if tp_size != 1 or dp_size != 1 or moe_tp_size != 1 or moe_ep_size != 1:
+            raise RuntimeError("Runtime: this build runs on a single GPU (all group sizes must be 1)")
+        self._lib = _lib.load()
+        if not torch.cuda.is_available():
+            raise RuntimeError("Runtime: no HIP device available")
+        self.devid = int(devid)
+        self.device = torch.device("cuda", self.devid)
+        self.rank = rank
+        self.task_id = 0
+        self.notify = None
+        self.peer_notify = None
+        self.multi_task_parallel = False
+        self.blocking = True
+        ncu = ctypes.c_int(0)
+        lds = ctypes.c_int(0)
+        arch = ctypes.create_string_buffer(64)
+        _lib.check(self._lib.xlite_hip_device_info(self.devid, ctypes.byref(ncu), ctypes.byref(lds), arch, 64))
+        self.num_cu = ncu.value
+        self.arch = arch.value.decode()
+        # names of the reference's core counts, for callers that read them
+        self.aic_num = self.num_cu
+        self.aiv_num = self.num_cu
+        self._pool: Optional[torch.Tensor] = None
+        self.init_tensor_pool(size)
+
+    # -- reference API ---------------------------------------------------------------------
+    def update_core_num(self, util: float) -> None:
+        self.aic_num = max(1, int(round(self.num_cu * util)))
+        self.aiv_num = self.aic_num
+
+    def init_tensor_pool(self, size: int) -> int:
+        if size:
+            self._grow(int(size) << 20)
+        return 0
+
+    def set_current_context(self) -> None:
+        torch.cuda.set_device(self.devid)
+
+    def configure_swizzle(self, swizzle: int, use_swizzle_table: bool) -> None:
+        return None  # matmul tiling knob of the reference; nothing on this path uses it
+
+    # -- scratch -------------------------------------------------------------------------------
+    def _grow(self, nbytes: int) -> None:
+        nbytes = max(nbytes, 1 << 20)
+        if self._pool is None or self._pool.numel() < nbytes:
+            if self._pool is not None:
+                torch.cuda.synchronize(self.device)
+            # zero-filled: the first 64 KiB are ticket counters that every call leaves at zero
+            self._pool = torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
+
+    def workspace(self, nbytes: int) -> torch.Tensor:
+        self._grow(nbytes)
+        return self._pool
+
+    def stream(self) -> ctypes.c_void_p:
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def finish(self) -> None:
+        if self.blocking:
+            torch.cuda.current_stream(self.device).synchronize()
+
+    def synchronize(self) -> None:
+        torch.cuda.current_stream(self.device).synchronize()
+
+
+def rope_and_cache(rt: Runtime, inout: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   position: torch.Tensor, cosin: torch.Tensor, slot_mapping: torch.Tensor, n_heads: int,
+                   n_kv_heads: int, head_dim: int, rot_dim: int, block_size: int, is_neox: bool,
+                   mrope_mask_h: int = 0, mrope_mask_w: int = 0) -> None:
+    if not is_neox:
+        raise RuntimeError("rope_and_cache: unsupported rope type gptj")
+    for n, t in (("inout", inout), ("k_cache", k_cache), ("v_cache", v_cache), ("cosin", cosin)):
+        _dev(n, t)
+    _dev("position", position, torch.int64)
+    _dev("slot_mapping", slot_mapping, torch.int32)
+    dt = _act_dtype("rope_and_cache", inout, k_cache, v_cache, cosin)
+    T = inout.shape[0]
+    _req(inout.numel() == T * (n_heads + 2 * n_kv_heads) * head_dim, "rope_and_cache: inout shape mismatch")
+    _req(k_cache.shape == v_cache.shape, "rope_and_cache: cache shapes differ")
+    _req(k_cache.numel() % (block_size * n_kv_heads * head_dim) == 0, "rope_and_cache: cache shape mismatch")
+    mrope = bool(mrope_mask_h or mrope_mask_w)
+    _req(position.numel() == (3 * T if mrope else T), "rope_and_cache: position shape mismatch")
+    _req(slot_mapping.numel() >= T, "rope_and_cache: slot_mapping too short")
+    _req(cosin.shape[-1] == rot_dim, "rope_and_cache: cosin row must hold rot_dim values")
+    _lib.check(rt._lib.xlite_hip_rope_and_cache(
+        rt.stream(), _ptr(inout), _ptr(k_cache), _ptr(v_cache), _ptr(position), _ptr(cosin), _ptr(slot_mapping),
+        T, n_heads, n_kv_heads, head_dim, rot_dim, block_size, 1, mrope_mask_h, mrope_mask_w, dt))
+    rt.finish()
+
+
+def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              output: torch.Tensor, query_start_loc: torch.Tensor, lens: torch.Tensor,
+              cached_lens: torch.Tensor, block_tables: torch.Tensor, n_heads: int, n_kv_heads: int,
+              head_dim: int, block_size: int, batch: int, max_num_block: int,
+              enable_flash_attention: bool = False, tile_size_of_cached_kv: int = 8192, *,
+              k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+    """Paged GQA attention, decode and causal (chunked) prefill. `enable_flash_attention` and
+    `tile_size_of_cached_kv` select between two kernels in the reference; here they are hints
+    only (the KV split is chosen from the batch shape)."""
+    for n, t in (("qkv", qkv), ("k_cache", k_cache), ("v_cache", v_cache), ("output", output)):
+        _dev(n, t)
+    for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens),
+                 ("block_tables", block_tables)):
+        _dev(n, t, torch.int32)
+    dt = _act_dtype("attention", qkv, output)
+    int8 = k_scale is not None or v_scale is not None
+    if int8:
+        _req(k_scale is not None and v_scale is not None, "attention: k_scale and v_scale go together")
+        _dev("k_scale", k_scale, torch.float32)
+        _dev("v_scale", v_scale, torch.float32)
+        _req(k_cache.dtype == torch.int8 and v_cache.dtype == torch.int8,
+             "attention: scales given but the caches are not int8")
+        _req(k_scale.numel() * head_dim == k_cache.numel() and v_scale.numel() * head_dim == v_cache.numel(),
+             "attention: one scale per (block, slot, kv head) expected")
+    else:
+        _req(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
+             "attention: qkv %s kCache %s vCache %s unsupported!" % (qkv.dtype, k_cache.dtype, v_cache.dtype))
+    T = qkv.shape[0]
+    _req(n_kv_heads > 0 and n_heads % n_kv_heads == 0, "attention: n_heads must be a multiple of n_kv_heads")
+    _req(qkv.numel() == T * (n_heads + 2 * n_kv_heads) * head_dim, "attention: qkv shape mismatch")
+    _req(output.numel() == T * n_heads * head_dim, "attention: output shape mismatch")
+    _req(min(query_start_loc.numel(), lens.numel(), cached_lens.numel()) >= batch, "attention: metadata shorter than batch")
+    _req(block_tables.numel() >= batch * max_num_block, "attention: block_tables shorter than batch * max_num_block")
+    need = rt._lib.xlite_hip_attention_workspace_bytes(T, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block)
+    ws = rt.workspace(need)
+    _lib.check(rt._lib.xlite_hip_attention(
+        rt.stream(), _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(output), _ptr(query_start_loc), _ptr(lens),
+        _ptr(cached_lens), _ptr(block_tables), T, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
+        dt, 1 if int8 else 0, _ptr(k_scale), _ptr(v_scale), _ptr(ws), ws.numel()))
+    rt.finish()
+
+
+def _einsum(rt: Runtime, name: str, mht, w, mhd, m, h, t, d, weight_nz, hdt: bool, t_stride: Optional[int] = None):
+    if weight_nz:
+        raise RuntimeError(name + ": the NZ (Ascend fractal) weight layout has no meaning on this device")
+    for n, x in (("mht", mht), ("w", w), ("mhd", mhd)):
+        _dev(n, x)
+    dt = _act_dtype(name, mht, w, mhd)
+    ts = t if t_stride is None else t_stride
+    _req(mht.numel() >= m * h * ts, name + ": mht too small")
+    _req(w.numel() == h * t * d, name + ": weight shape mismatch")
+    _req(mhd.numel() == m * h * d, name + ": mhd shape mismatch")
+    _lib.check(rt._lib.xlite_hip_einsum_mht_mhd(rt.stream(), _ptr(mht), _ptr(w), _ptr(mhd), m, h, t, d, ts,
+                                                1 if hdt else 0, dt))
+
+
+def einsum_mht_htd_mhd(rt: Runtime, mht: torch.Tensor, htd: torch.Tensor, mhd: torch.Tensor, m: int, h: int,
+                       t: int, d: int, weight_nz: bool = False) -> None:
+    _einsum(rt, "einsum_mht_htd_mhd", mht, htd, mhd, m, h, t, d, weight_nz, False)
+    rt.finish()
+
+
+def einsum_mht_hdt_mhd(rt: Runtime, mht: torch.Tensor, hdt: torch.Tensor, mhd: torch.Tensor, m: int, h: int,
+                       t: int, d: int, weight_nz: bool = False) -> None:
+    _einsum(rt, "einsum_mht_hdt_mhd", mht, hdt, mhd, m, h, t, d, weight_nz, True)
+    rt.finish()
+
+
+def mla_attention(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_cache: torch.Tensor,
+                  pe_cache: torch.Tensor, o_absorb: torch.Tensor, query_start_loc: torch.Tensor,
+                  lens: torch.Tensor, cached_lens: torch.Tensor, block_tables: torch.Tensor, n_heads: int,
+                  rope_head_dim: int, kv_lora_rank: int, block_size: int, batch: int, max_num_blocks: int,
+                  scale: float, topk_indices: Optional[torch.Tensor] = None, top_k: int = 0) -> None:
+    """The attention stage of mla_v2 alone (q_absorb, qr -> o_absorb); the reference runs it as
+    XliteOpMLAV2 / XliteOpFlashMLAV2 inside the mla_v2 binding (xlite/csrc/_C.cpp:1264-1294)."""
+    for n, t in (("q_absorb", q_absorb), ("qr", qr), ("k_cache", k_cache), ("pe_cache", pe_cache),
+                 ("o_absorb", o_absorb)):
+        _dev(n, t)
+    for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens),
+                 ("block_tables", block_tables)):
+        _dev(n, t, torch.int32)
+    _req(q_absorb.dtype == torch.bfloat16, "mla: qAbsorb dtype %s unsupported!" % q_absorb.dtype)
+    dt = _act_dtype("mla", q_absorb, qr, k_cache, pe_cache, o_absorb)
+    if top_k > 2048:
+        raise RuntimeError("mla: topK should be less than or equal to 2048")
+    T = q_absorb.shape[0]
+    _req(q_absorb.numel() == T * n_heads * kv_lora_rank and o_absorb.numel() == q_absorb.numel(),
+         "mla: q_absorb / o_absorb shape mismatch")
+    _req(qr.numel() == T * n_heads * rope_head_dim, "mla: qr shape mismatch")
+    _req(block_tables.numel() >= batch * max_num_blocks, "mla: block_tables too short")
+    if top_k:
+        _dev("topk_indices", topk_indices, torch.int32)
+        _req(topk_indices.numel() >= T * top_k, "mla: topk_indices too short")
+    need = rt._lib.xlite_hip_mla_workspace_bytes(T, n_heads, kv_lora_rank, block_size, batch, max_num_blocks)
+    ws = rt.workspace(need)
+    _lib.check(rt._lib.xlite_hip_mla_attention(
+        rt.stream(), _ptr(q_absorb), _ptr(qr), _ptr(k_cache), _ptr(pe_cache), _ptr(o_absorb),
+        _ptr(query_start_loc), _ptr(lens), _ptr(cached_lens), _ptr(block_tables), T, n_heads, rope_head_dim,
+        kv_lora_rank, block_size, batch, max_num_blocks, float(scale), _ptr(topk_indices) if top_k else None,
+        top_k, dt, _ptr(ws), ws.numel()))
+
+
+def mla_v2(rt: Runtime, q_with_qr: torch.Tensor, qr: torch.Tensor, k_cache: torch.Tensor,
+           pe_cache: torch.Tensor, wuk_t: torch.Tensor, wuv: torch.Tensor, output: torch.Tensor,
+           query_start_loc: torch.Tensor, lens: torch.Tensor, cached_lens: torch.Tensor,
+           block_tables: torch.Tensor, n_heads: int, rope_head_dim: int, nope_head_dim: int, v_head_dim: int,
+           kv_lora_rank: int, block_size: int, batch: int, max_num_blocks: int, scale: float,
+           topk_indices: torch.Tensor, top_k: int = 0, nz: bool = False, enable_flash_attention: bool = False,
+           tile_size_of_cached_kv: int = 8192) -> None:
+    """W_UK absorb einsum + absorbed MLA attention + W_UV einsum (xlite/csrc/_C.cpp:1234-1301)."""
+    if nz:
+        raise RuntimeError("mla_v2: the NZ (Ascend fractal) weight layout has no meaning on this device")
+    T = q_with_qr.shape[0]
+    _dev("q_with_qr", q_with_qr)
+    q_absorb = torch.empty(T, n_heads * kv_lora_rank, dtype=q_with_qr.dtype, device=q_with_qr.device)
+    o_absorb = torch.empty_like(q_absorb)
+    _einsum(rt, "mla_v2", q_with_qr, wuk_t, q_absorb, T, n_heads, nope_head_dim, kv_lora_rank, False, False,
+            t_stride=nope_head_dim + rope_head_dim)
+    mla_attention(rt, q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
+                  n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks, scale, topk_indices,
+                  top_k)
+    _einsum(rt, "mla_v2", o_absorb, wuv, output, T, n_heads, kv_lora_rank, v_head_dim, False, False)
+    rt.finish()
+
+
+def gather_sparse_kv_cache(rt: Runtime, k_cache: torch.Tensor, pe_cache: torch.Tensor, block_tables: torch.Tensor,
+                           topk_indices: torch.Tensor, query_lens: torch.Tensor, cached_lens: torch.Tensor,
+                           k_dense_cache: torch.Tensor, pe_dense_cache: torch.Tensor, batch: int, index_topk: int,
+                           block_size: int, max_num_blocks: int, kv_lora_rank: int, rope_head_dim: int,
+                           kv_heads: int = 1) -> None:
+    if kv_heads != 1:
+        raise RuntimeError("gather_sparse_kv_cache: kvHeads should be less than or equal to 1")
+    for n, t in (("k_cache", k_cache), ("pe_cache", pe_cache), ("k_dense_cache", k_dense_cache),
+                 ("pe_dense_cache", pe_dense_cache)):
+        _dev(n, t)
+    for n, t in (("block_tables", block_tables), ("topk_indices", topk_indices), ("query_lens", query_lens),
+                 ("cached_lens", cached_lens)):
+        _dev(n, t, torch.int32)
+    dt = _act_dtype("gather_sparse_kv_cache", k_cache, pe_cache, k_dense_cache, pe_dense_cache)
+    _req(k_dense_cache.numel() == batch * index_topk * kv_lora_rank, "gather_sparse_kv_cache: k_dense shape mismatch")
+    _req(pe_dense_cache.numel() == batch * index_topk * rope_head_dim, "gather_sparse_kv_cache: pe_dense shape mismatch")
+    _req(topk_indices.numel() >= batch * index_topk, "gather_sparse_kv_cache: topk_indices too short")
+    _req(block_tables.numel() >= batch * max_num_blocks, "gather_sparse_kv_cache: block_tables too short")
+    _lib.check(rt._lib.xlite_hip_gather_sparse_kv_cache(
+        rt.stream(), _ptr(k_cache), _ptr(pe_cache), _ptr(block_tables), _ptr(topk_indices), _ptr(query_lens),
+        _ptr(cached_lens), _ptr(k_dense_cache), _ptr(pe_dense_cache), batch, index_topk, block_size,
+        max_num_blocks, kv_lora_rank, rope_head_dim, kv_heads, dt))
+    rt.finish()
+
+
+def mla_v3(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_dense_cache: torch.Tensor,
+           pe_dense_cache: torch.Tensor, o_absorb: torch.Tensor, query_start_loc: torch.Tensor, lens: torch.Tensor,
+           cached_lens: torch.Tensor, n_heads: int, rope_head_dim: int, kv_lora_rank: int, batch: int,
+           index_topk: int, scale: float) -> None:
+    for n, t in (("q_absorb", q_absorb), ("qr", qr), ("k_dense_cache", k_dense_cache),
+                 ("pe_dense_cache", pe_dense_cache), ("o_absorb", o_absorb)):
+        _dev(n, t)
+    for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens)):
+        _dev(n, t, torch.int32)
+    _req(q_absorb.dtype == torch.bfloat16, "mla_v3: qAbsorb dtype %s unsupported!" % q_absorb.dtype)
+    dt = _act_dtype("mla_v3", q_absorb, qr, k_dense_cache, pe_dense_cache, o_absorb)
+    T = q_absorb.shape[0]
+    _req(k_dense_cache.numel() == batch * index_topk * kv_lora_rank, "mla_v3: k_dense shape mismatch")
+    _req(pe_dense_cache.numel() == batch * index_topk * rope_head_dim, "mla_v3: pe_dense shape mismatch")
+    need = rt._lib.xlite_hip_mla_workspace_bytes(T, n_heads, kv_lora_rank, 1, batch, index_topk)
+    ws = rt.workspace(need)
+    _lib.check(rt._lib.xlite_hip_mla_v3(
+        rt.stream(), _ptr(q_absorb), _ptr(qr), _ptr(k_dense_cache), _ptr(pe_dense_cache), _ptr(o_absorb),
+        _ptr(query_start_loc), _ptr(lens), _ptr(cached_lens), T, n_heads, rope_head_dim, kv_lora_rank, batch,
+        index_topk, float(scale), dt, _ptr(ws), ws.numel()))
+    rt.finish()
+
+
+def _freqs_f32(freqs: torch.Tensor, rope_dim: int) -> torch.Tensor:
+    """complex64 [max_pos, rope_dim/2] is read as interleaved fp32 (cos, sin), as the reference does."""
+    _req(freqs.is_cuda and freqs.is_contiguous(), "freqs: contiguous GPU tensor expected")
+    f = torch.view_as_real(freqs) if freqs.is_complex() else freqs
+    _req(f.dtype == torch.float32, "freqs: complex64 / float32 expected")
+    _req(f.numel() % rope_dim == 0, "freqs: row must hold rope_dim floats")
+    return f
+
+
+def rope_complex(rt: Runtime, n_local_heads: int, step_dim: int, rope_dim: int, input_with_r: torch.Tensor,
+                 freqs: torch.Tensor, position: torch.Tensor, output: torch.Tensor) -> None:
+    _dev("input_with_r", input_with_r)
+    _dev("output", output)
+    _dev("position", position, torch.int64)
+    dt = _act_dtype("rope_complex", input_with_r, output)
+    f = _freqs_f32(freqs, rope_dim)
+    T = input_with_r.shape[0]
+    _req(input_with_r.numel() == T * n_local_heads * step_dim, "rope_complex: input shape mismatch")
+    _req(output.numel() == T * n_local_heads * rope_dim, "rope_complex: output shape mismatch")
+    _req(position.numel() >= T, "rope_complex: position too short")
+    _lib.check(rt._lib.xlite_hip_rope_complex(rt.stream(), T, n_local_heads, step_dim, rope_dim,
+                                              _ptr(input_with_r), _ptr(f), _ptr(position), _ptr(output), dt))
+    rt.finish()
+
+
+def mla_prepare(rt: Runtime, attn_qkvc: torch.Tensor, q_norm: torch.Tensor, q_norm_bias: torch.Tensor,
+                attn_norm_qc: torch.Tensor, kv_norm: torch.Tensor, kv_norm_bias: torch.Tensor,
+                attn_norm_kvc: torch.Tensor, freqs: torch.Tensor, position: torch.Tensor, q_lora_rank: int,
+                kv_lora_rank: int, rope_head_dim: int, block_size: int, k_cache: torch.Tensor,
+                pe_cache: torch.Tensor, slot_mapping: torch.Tensor, norm_eps: float) -> None:
+    for n, t in (("attn_qkvc", attn_qkvc), ("q_norm", q_norm), ("q_norm_bias", q_norm_bias),
+                 ("attn_norm_qc", attn_norm_qc), ("kv_norm", kv_norm), ("kv_norm_bias", kv_norm_bias),
+                 ("attn_norm_kvc", attn_norm_kvc)):
+        _dev(n, t)
+    _dev("position", position, torch.int64)
+    dt = _act_dtype("mla_prepare", attn_qkvc, q_norm, q_norm_bias, attn_norm_qc, kv_norm, kv_norm_bias,
+                    attn_norm_kvc)
+    f = _freqs_f32(freqs, rope_head_dim)
+    T = attn_qkvc.shape[0]
+    _req(attn_qkvc.numel() == T * (q_lora_rank + kv_lora_rank + rope_head_dim), "mla_prepare: attn_qkvc shape mismatch")
+    _req(attn_norm_qc.numel() == T * q_lora_rank and attn_norm_kvc.numel() == T * kv_lora_rank,
+         "mla_prepare: output shape mismatch")
+    if block_size:
+        _dev("k_cache", k_cache, attn_qkvc.dtype)
+        _dev("pe_cache", pe_cache, attn_qkvc.dtype)
+        _dev("slot_mapping", slot_mapping, torch.int32)
+        _req(slot_mapping.numel() >= T, "mla_prepare: slot_mapping too short")
+    _lib.check(rt._lib.xlite_hip_mla_prepare(
+        rt.stream(), _ptr(attn_qkvc), _ptr(q_norm), _ptr(q_norm_bias), _ptr(attn_norm_qc), _ptr(kv_norm),
+        _ptr(kv_norm_bias), _ptr(attn_norm_kvc), _ptr(f), _ptr(position), T, q_lora_rank, kv_lora_rank,
+        rope_head_dim, block_size, _ptr(k_cache) if block_size else None, _ptr(pe_cache) if block_size else None,
+        _ptr(slot_mapping) if block_size else None, float(norm_eps), dt))
+    rt.finish()
+
+
+def get_tile_size_of_cached_kv(cached_lens: List[int], query_lens: List[int], head_num_in_group: int,
+                               n_kv_heads: int, block_size: int, aic_num: int) -> int:
+    """Host-only; same integer results as the reference tuner (xlite/csrc/auto_tuner.cpp:163-210)."""
+    lib = _lib.load()
+    n = len(query_lens)
+    if len(cached_lens) != n:
+        raise RuntimeError("get_tile_size_of_cached_kv: cached_lens and query_lens differ in length")
+    arr = ctypes.c_uint32 * max(n, 1)
+    rc = lib.xlite_hip_get_tile_size_of_cached_kv(arr(*cached_lens), arr(*query_lens), n, head_num_in_group,
+                                                  n_kv_heads, block_size, aic_num)
+    if rc < 0:
+        _lib.check(rc)
+    return rc
+
+
+def quantize_kv_int8(rt: Runtime, x: torch.Tensor):
+    """x [..., head_dim] (fp16/bf16) -> (int8 tensor of the same shape, fp32 scales [...]).
+    Not part of the reference API (its caches are never quantised)."""
+    _dev("x", x)
+    dt = _act_dtype("quantize_kv_int8", x)
+    d = x.shape[-1]
+    rows = x.numel() // d
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    _lib.check(rt._lib.xlite_hip_quantize_kv_int8(rt.stream(), _ptr(x), _ptr(q), _ptr(s), rows, d, dt))
+    rt.finish()
+    return q, s

@@ -1,0 +1,143 @@
+// C entry points of the attention operators: argument checks and kernel selection.
+#include "attention_common.h"
+
+using namespace xlite;
+
+namespace {
+
+bool is_decode_batch(uint32_t total_tokens, uint32_t batch)
+{
+    // every sequence contributes at least one row, so equality means one row each
+    return total_tokens == batch;
+}
+
+}  // namespace
+
+extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
+                                                      uint32_t n_kv_heads, uint32_t head_dim,
+                                                      uint32_t block_size, uint32_t batch,
+                                                      uint32_t max_num_block)
+{
+    if (total_tokens == 0 || batch == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || head_dim < 8) {
+        return XLITE_HIP_WS_COUNTER_BYTES;
+    }
+    const uint32_t max_ctx = max_num_block * block_size;
+    if (is_decode_batch(total_tokens, batch)) {
+        uint32_t g_kernel, head_chunks, nkv_wg, zdim;
+        decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
+        const uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);
+        return XLITE_HIP_WS_COUNTER_BYTES +
+               decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile));
+    }
+    const uint32_t splits =
+        mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx, 64);
+    return mfma_workspace_bytes(total_tokens, n_heads, head_dim, splits + 1);
+}
+
+extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache,
+                                   const void *v_cache, void *output,
+                                   const int32_t *query_start_loc, const int32_t *lens,
+                                   const int32_t *cached_lens, const int32_t *block_tables,
+                                   uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                                   uint32_t head_dim, uint32_t block_size, uint32_t batch,
+                                   uint32_t max_num_block, int dtype, int kv_dtype,
+                                   const float *k_scale, const float *v_scale, void *workspace,
+                                   size_t workspace_bytes)
+{
+    XL_REQUIRE(dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16, "qkv/kCache/vCache/output dtype unsupported!");
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || kv_dtype == XLITE_HIP_KV_INT8, "kv cache dtype unsupported!");
+    XL_REQUIRE(qkv && k_cache && v_cache && output && query_start_loc && lens && cached_lens && block_tables,
+               "null tensor");
+    XL_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+               "n_heads must be a positive multiple of n_kv_heads");
+    XL_REQUIRE(block_size > 0 && max_num_block > 0, "block_size and max_num_block must be positive");
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || (k_scale && v_scale), "int8 KV cache needs k_scale and v_scale");
+    XL_REQUIRE(total_tokens >= batch, "fewer query tokens than sequences");
+    if (batch == 0 || total_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
+    AttentionArgs a{qkv, k_cache, v_cache, output, query_start_loc, lens, cached_lens, block_tables,
+                    total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
+                    dtype, kv_dtype, k_scale, v_scale, workspace, workspace_bytes};
+    hipStream_t s = as_stream(stream);
+    if (is_decode_batch(total_tokens, batch)) {
+        XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");
+        uint32_t g_kernel, head_chunks, nkv_wg, zdim;
+        decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
+        uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);
+        // shrink the split count to what the caller's workspace can hold
+        const uint32_t max_ctx = max_num_block * block_size;
+        while (ceil_div(max_ctx, tile) > 1 &&
+               (workspace == nullptr ||
+                XLITE_HIP_WS_COUNTER_BYTES + decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile)) > workspace_bytes)) {
+            tile *= 2;
+        }
+        int rc = launch_decode(s, a, tile);
+        if (rc != XLITE_HIP_OK) {
+            return rc;
+        }
+        XL_LAUNCH_CHECK();
+        return XLITE_HIP_OK;
+    }
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME, "the int8 KV cache is supported for decode batches only");
+    XL_REQUIRE(mfma_gqa_supported(head_dim), "head_dim must be 64 or 128");
+    return launch_mfma_gqa(s, a);
+}
+
+extern "C" size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
+                                                uint32_t kv_lora_rank, uint32_t block_size,
+                                                uint32_t batch, uint32_t max_num_blocks)
+{
+    const uint32_t max_ctx = max_num_blocks * block_size;
+    const uint32_t splits = mfma_pick_splits(total_tokens, n_heads, batch, 1, max_ctx, 32);
+    return mfma_workspace_bytes(total_tokens, n_heads, kv_lora_rank, splits + 1);
+}
+
+extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const void *qr,
+                                       const void *k_cache, const void *pe_cache, void *o_absorb,
+                                       const int32_t *query_start_loc, const int32_t *lens,
+                                       const int32_t *cached_lens, const int32_t *block_tables,
+                                       uint32_t total_tokens, uint32_t n_heads,
+                                       uint32_t rope_head_dim, uint32_t kv_lora_rank,
+                                       uint32_t block_size, uint32_t batch, uint32_t max_num_blocks,
+                                       float scale, const int32_t *topk_indices, uint32_t top_k,
+                                       int dtype, void *workspace, size_t workspace_bytes)
+{
+    XL_REQUIRE(dtype == XLITE_HIP_BF16, "qAbsorb/qr/kCache/peCache/oAbsorb dtype unsupported!");
+    XL_REQUIRE(top_k <= 2048, "topK should be less than or equal to 2048");
+    XL_REQUIRE(top_k == 0, "top-k index masks are not built yet");
+    XL_REQUIRE(q_absorb && qr && k_cache && pe_cache && o_absorb && query_start_loc && lens &&
+                   cached_lens && block_tables,
+               "null tensor");
+    XL_REQUIRE(n_heads > 0 && block_size > 0 && max_num_blocks > 0, "zero head count or block geometry");
+    XL_REQUIRE(total_tokens >= batch, "fewer query tokens than sequences");
+    (void)topk_indices;
+    if (batch == 0 || total_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
+    MlaArgs a{q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
+              total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks,
+              0, scale, topk_indices, top_k, dtype, workspace, workspace_bytes};
+    return launch_mfma_mla(as_stream(stream), a);
+}
+
+extern "C" int xlite_hip_mla_v3(void *stream, const void *q_absorb, const void *qr,
+                                const void *k_dense, const void *pe_dense, void *o_absorb,
+                                const int32_t *query_start_loc, const int32_t *lens,
+                                const int32_t *cached_lens, uint32_t total_tokens, uint32_t n_heads,
+                                uint32_t rope_head_dim, uint32_t kv_lora_rank, uint32_t batch,
+                                uint32_t index_topk, float scale, int dtype, void *workspace,
+                                size_t workspace_bytes)
+{
+    XL_REQUIRE(dtype == XLITE_HIP_BF16, "qAbsorb/qr/kDenseCache/peDenseCache/oAbsorb dtype unsupported!");
+    XL_REQUIRE(q_absorb && qr && k_dense && pe_dense && o_absorb && query_start_loc && lens && cached_lens,
+               "null tensor");
+    XL_REQUIRE(n_heads > 0 && index_topk > 0, "zero head count or dense length");
+    if (batch == 0 || total_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
+    MlaArgs a{q_absorb, qr, k_dense, pe_dense, o_absorb, query_start_loc, lens, cached_lens, nullptr,
+              total_tokens, n_heads, rope_head_dim, kv_lora_rank, 1, batch, index_topk,
+              index_topk, scale, nullptr, 0, dtype, workspace, workspace_bytes};
+    return launch_mfma_mla(as_stream(stream), a);
+}

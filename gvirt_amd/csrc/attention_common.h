@@ -1,0 +1,63 @@
+// Argument bundles and launcher declarations shared by the attention entry points.
+#pragma once
+
+#include "common.h"
+
+namespace xlite {
+
+struct AttentionArgs {
+    const void *qkv;
+    const void *k_cache;
+    const void *v_cache;
+    void *output;
+    const int32_t *query_start_loc;
+    const int32_t *lens;
+    const int32_t *cached_lens;
+    const int32_t *block_tables;
+    uint32_t total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block;
+    int dtype, kv_dtype;
+    const float *k_scale;
+    const float *v_scale;
+    void *workspace;
+    size_t workspace_bytes;
+};
+
+struct MlaArgs {
+    const void *q_absorb;
+    const void *qr;
+    const void *k_cache;     // paged [blocks, block_size, kv_lora_rank] or dense [batch, index_topk, ...]
+    const void *pe_cache;
+    void *o_absorb;
+    const int32_t *query_start_loc;
+    const int32_t *lens;
+    const int32_t *cached_lens;
+    const int32_t *block_tables;   // nullptr: dense per-sequence cache (mla_v3)
+    uint32_t total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks;
+    uint32_t dense_len;            // mla_v3: entries per sequence, attention is not causal
+    float scale;
+    const int32_t *topk_indices;
+    uint32_t top_k;
+    int dtype;
+    void *workspace;
+    size_t workspace_bytes;
+};
+
+// decode_attention.hip
+bool decode_supported(uint32_t head_dim);
+void decode_geometry(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t *g_kernel,
+                     uint32_t *head_chunks, uint32_t *nkv_wg, uint32_t *zdim);
+uint32_t decode_pick_tile(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size,
+                          uint32_t max_num_block, uint32_t zdim);
+size_t decode_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim,
+                              uint32_t max_tiles);
+int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_tokens);
+
+// mfma_attention.hip
+bool mfma_gqa_supported(uint32_t head_dim);
+size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits);
+uint32_t mfma_pick_splits(uint32_t total_tokens, uint32_t rows_per_token, uint32_t batch,
+                          uint32_t parallel_heads, uint32_t max_ctx, uint32_t tile);
+int launch_mfma_gqa(hipStream_t stream, const AttentionArgs &a);
+int launch_mfma_mla(hipStream_t stream, const MlaArgs &a);
+
+}  // namespace xlite

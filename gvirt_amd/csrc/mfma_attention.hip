@@ -1,0 +1,570 @@
+// Dense attention on the bf16/fp16 matrix cores: chunked causal prefill over the paged GQA cache
+// and DeepSeek-style absorbed MLA (paged or dense latent cache).
+//
+// One workgroup = 4 wavefronts = 128 "M rows", an M row being one (query position, query head)
+// pair of a kv head (GQA) or of the single latent head (MLA). Each wave owns 32 M rows and keeps
+// their query vectors in registers as the B operand of v_mfma_f32_32x32x16; the workgroup walks
+// the visible KV positions in tiles of BN tokens staged in LDS:
+//     S^T[token][m]  = K[token][:] . Q[m][:]          (A = K rows from LDS, B = Q registers)
+//     O^T[d][m]     += V^T[d][token] . P^T[token][m]   (A = transposed V from LDS, B = P registers)
+// Computing the transposed products keeps one M row per lane column, so the online softmax needs
+// a single cross-lane exchange per tile, and the probabilities leave the QK accumulators already
+// in the register layout the PV product wants (the token order inside a 16-token group is
+// permuted identically on the V^T side). Scores and outputs accumulate in fp32; P is rounded to
+// the 16-bit storage type before the second product, as in the reference (softmax_attn_aiv.h:904-908).
+//
+// The KV range of an M tile can be split across workgroups (grid.x); partial (max, sum, O) are
+// merged by the last workgroup to finish.
+//
+// Replaces attention.h / flash_attention.h for batches with multi-token queries
+// (xlite/csrc/kernels/attention.h:308-492) and mla_v2.h / flash_mla_v2.h / mla_v3.h.
+#include "attention_common.h"
+
+namespace xlite {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kMTile = kWaves * 32;
+
+template <typename T>
+struct Mfma;
+template <>
+struct Mfma<BF16> {
+    static __device__ __forceinline__ f32x16_t run(const uint4 &a, const uint4 &b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<FP16> {
+    static __device__ __forceinline__ f32x16_t run(const uint4 &a, const uint4 &b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+};
+
+struct MfmaParams {
+    const uint16_t *q0;   // first DQ0 columns of a query row
+    const uint16_t *q1;   // remaining DQ1 columns (MLA rope part)
+    const uint16_t *k0;   // cache rows matching q0
+    const uint16_t *k1;   // cache rows matching q1
+    const uint16_t *v;    // separate value cache (GQA)
+    uint16_t *out;
+    const int32_t *query_start_loc;
+    const int32_t *lens;
+    const int32_t *cached_lens;
+    const int32_t *block_tables;  // nullptr: dense cache of dense_len rows per sequence, no causality
+    int32_t *counters;
+    float *part_acc;
+    float *part_ml;
+    uint32_t q0_tok_stride, q0_head_stride, q1_tok_stride, q1_head_stride;
+    uint32_t k0_tok_stride, k1_tok_stride;   // elements between consecutive cache rows
+    uint32_t out_tok_stride;
+    uint32_t rows_per_pos;       // G: query heads sharing the kv head
+    uint32_t n_heads;
+    uint32_t batch;
+    uint32_t block_size;
+    int32_t block_shift;
+    uint32_t max_num_block;
+    uint32_t dense_len;
+    uint32_t split_len;
+    uint32_t max_splits;
+    float scale_log2e;
+};
+
+// position inside a 16-token group at which token offset o is stored in the transposed V tile, so
+// that the eight tokens a lane's P registers hold are contiguous
+__device__ __forceinline__ uint32_t vt_pos(uint32_t o)
+{
+    return (o & ~15u) | (((o >> 2) & 1u) << 3) | (((o >> 3) & 1u) << 2) | (o & 3u);
+}
+
+template <typename T, int DQ0, int DQ1, int DV, int BN, bool SEPARATE_V>
+__global__ void __launch_bounds__(kThreads)
+mfma_attention_kernel(const MfmaParams p)
+{
+    constexpr int DQK = DQ0 + DQ1;
+    constexpr int KS = DQK / 16;             // k-steps of the QK product
+    constexpr int NT = BN / 32;              // 32-token sub tiles
+    constexpr int DT = DV / 32;              // 32-row tiles of O^T
+    constexpr int KSTRIDE = DQK + 8;         // LDS row stride of the K tile, elements
+    constexpr int VSTRIDE = BN + 8;          // LDS row stride of the V^T tile, elements
+    constexpr int CPR = DQK / 8;             // 16-byte chunks per K row
+    constexpr int CPR0 = DQ0 / 8;
+    constexpr int VCPR = DV / 8;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    uint16_t *Ks = reinterpret_cast<uint16_t *>(smem_raw);
+    uint16_t *Vt = Ks + BN * KSTRIDE;
+    uint64_t *rowidx = reinterpret_cast<uint64_t *>(Vt + DV * VSTRIDE);
+    int32_t *flag = reinterpret_cast<int32_t *>(rowidx + BN);
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t col = lane & 31;
+    const uint32_t half = lane >> 5;
+    const uint32_t split = blockIdx.x;
+    const uint32_t kvh = blockIdx.z;
+    const uint32_t G = p.rows_per_pos;
+
+    // ---- locate the M tile: tiles are numbered sequence by sequence ---------------------------
+    uint32_t seq = 0, mt = blockIdx.y;
+    int32_t qlen = 0;
+    for (; seq < p.batch; seq++) {
+        qlen = p.lens[seq];
+        const uint32_t tiles = ceil_div(static_cast<uint32_t>(qlen > 0 ? qlen : 0) * G, kMTile);
+        if (mt < tiles) {
+            break;
+        }
+        mt -= tiles;
+    }
+    if (seq >= p.batch) {
+        return;
+    }
+    const int32_t clen = p.cached_lens[seq];
+    const int32_t qstart = p.query_start_loc[seq];
+    const uint32_t m_rows = static_cast<uint32_t>(qlen) * G;
+    const uint32_t m_first = mt * kMTile;
+    const uint32_t m_last = min(m_rows, m_first + kMTile) - 1;
+    const bool dense = p.block_tables == nullptr;
+    const uint32_t total_kv = dense ? min(static_cast<uint32_t>(clen + qlen), p.dense_len)
+                                    : static_cast<uint32_t>(clen + qlen);
+    // keys visible to at least one row of the tile
+    const uint32_t limit_max = dense ? total_kv : static_cast<uint32_t>(clen) + m_last / G + 1;
+    const uint32_t n_splits = ceil_div(limit_max, p.split_len);
+    if (split >= n_splits) {
+        return;
+    }
+    const uint32_t range_begin = split * p.split_len;
+    const uint32_t range_end = min(limit_max, range_begin + p.split_len);
+
+    // ---- this lane's M row -----------------------------------------------------------------------
+    const uint32_t m = m_first + wave * 32 + col;
+    const bool m_valid = m < m_rows;
+    const uint32_t qpos = m_valid ? m / G : 0;
+    const uint32_t hh = m_valid ? m % G : 0;
+    const uint32_t head = kvh * G + hh;
+    const uint32_t tok = static_cast<uint32_t>(qstart) + qpos;
+    const uint32_t vis = !m_valid ? 0u
+                         : min(range_end, dense ? total_kv : static_cast<uint32_t>(clen) + qpos + 1);
+
+    uint4 qreg[KS];
+    {
+        const uint16_t *src0 = p.q0 + static_cast<uint64_t>(tok) * p.q0_tok_stride + static_cast<uint64_t>(head) * p.q0_head_stride;
+        const uint16_t *src1 = DQ1 ? p.q1 + static_cast<uint64_t>(tok) * p.q1_tok_stride + static_cast<uint64_t>(head) * p.q1_head_stride : nullptr;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int c = ks * 16 + half * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (m_valid) {
+                v = (ks * 16 < DQ0) ? *reinterpret_cast<const uint4 *>(src0 + c)
+                                    : *reinterpret_cast<const uint4 *>(src1 + (c - DQ0));
+            }
+            qreg[ks] = v;
+        }
+    }
+
+    f32x16_t O[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            O[dt][k] = 0.f;
+        }
+    }
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int32_t *table = dense ? nullptr : p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
+
+    for (uint32_t j0 = range_begin; j0 < range_end; j0 += BN) {
+        // ---- cache row of every token of the tile ------------------------------------------------
+        __syncthreads();  // previous tile fully consumed
+        if (threadIdx.x < BN) {
+            uint32_t t = j0 + threadIdx.x;
+            t = t < range_end ? t : range_end - 1;
+            uint64_t row;
+            if (dense) {
+                row = static_cast<uint64_t>(seq) * p.dense_len + t;
+            } else {
+                const uint32_t b = p.block_shift >= 0 ? t >> p.block_shift : t / p.block_size;
+                const uint32_t o = p.block_shift >= 0 ? t & (p.block_size - 1) : t % p.block_size;
+                row = static_cast<uint64_t>(static_cast<uint32_t>(table[b])) * p.block_size + o;
+            }
+            rowidx[threadIdx.x] = row;
+        }
+        __syncthreads();
+
+        // ---- stage K (row major) and V (transposed) ------------------------------------------------
+        for (uint32_t c = threadIdx.x; c < BN * CPR; c += kThreads) {
+            const uint32_t r = c / CPR, cc = c % CPR;
+            const bool live = j0 + r < range_end;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (live) {
+                const uint64_t row = rowidx[r];
+                if (DQ1 == 0 || cc < CPR0) {
+                    val = *reinterpret_cast<const uint4 *>(p.k0 + row * p.k0_tok_stride + (SEPARATE_V ? kvh * DQ0 : 0) + cc * 8);
+                } else {
+                    val = *reinterpret_cast<const uint4 *>(p.k1 + row * p.k1_tok_stride + (cc - CPR0) * 8);
+                }
+            }
+            *reinterpret_cast<uint4 *>(Ks + r * KSTRIDE + cc * 8) = val;
+            if (!SEPARATE_V && cc < VCPR) {
+                const uint32_t pos = vt_pos(r);
+                const uint16_t *e = reinterpret_cast<const uint16_t *>(&val);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    Vt[(cc * 8 + i) * VSTRIDE + pos] = e[i];
+                }
+            }
+        }
+        if (SEPARATE_V) {
+            for (uint32_t c = threadIdx.x; c < BN * VCPR; c += kThreads) {
+                const uint32_t r = c / VCPR, cc = c % VCPR;
+                const bool live = j0 + r < range_end;
+                uint4 val = make_uint4(0, 0, 0, 0);
+                if (live) {
+                    val = *reinterpret_cast<const uint4 *>(p.v + rowidx[r] * p.k0_tok_stride + kvh * DV + cc * 8);
+                }
+                const uint32_t pos = vt_pos(r);
+                const uint16_t *e = reinterpret_cast<const uint16_t *>(&val);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    Vt[(cc * 8 + i) * VSTRIDE + pos] = e[i];
+                }
+            }
+        }
+        __syncthreads();
+
+        // ---- S^T = K . Q^T ----------------------------------------------------------------------------
+        f32x16_t S[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                S[nt][k] = 0.f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const uint4 a = *reinterpret_cast<const uint4 *>(Ks + (nt * 32 + col) * KSTRIDE + ks * 16 + half * 8);
+                S[nt] = Mfma<T>::run(a, qreg[ks], S[nt]);
+            }
+        }
+
+        // ---- online softmax over the tile -----------------------------------------------------------------
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                const uint32_t t = j0 + nt * 32 + (k / 4) * 8 + half * 4 + (k % 4);
+                const float s = t < vis ? S[nt][k] * p.scale_log2e : -INFINITY;
+                S[nt][k] = s;
+                mx = fmaxf(mx, s);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        m_run = m_new;
+        uint4 pb[NT][2];
+        float psum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+            uint32_t w[8];
+#pragma unroll
+            for (int k = 0; k < 16; k += 2) {
+                const float e0 = fast_exp2(S[nt][k] - m_safe);
+                const float e1 = fast_exp2(S[nt][k + 1] - m_safe);
+                psum += e0 + e1;
+                w[k / 2] = T::pack(e0, e1);
+            }
+            pb[nt][0] = make_uint4(w[0], w[1], w[2], w[3]);
+            pb[nt][1] = make_uint4(w[4], w[5], w[6], w[7]);
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                O[dt][k] *= alpha;
+            }
+        }
+
+        // ---- O^T += V^T . P^T -------------------------------------------------------------------------------
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(Vt + (dt * 32 + col) * VSTRIDE + nt * 32 + kk * 16 + half * 8);
+                    O[dt] = Mfma<T>::run(a, pb[nt][kk], O[dt]);
+                }
+            }
+        }
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+
+    if (n_splits == 1) {
+        if (m_valid) {
+            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            uint16_t *dst = p.out + static_cast<uint64_t>(tok) * p.out_tok_stride + static_cast<uint64_t>(head) * DV;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                for (int kg = 0; kg < 4; kg++) {
+                    uint2 o;
+                    o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
+                    o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
+                    *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- partial result, ticket, merge by the last split to finish ------------------------------------------
+    if (m_valid) {
+        const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head) * p.max_splits + split;
+        float *dst = p.part_acc + slot * DV;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+            for (int kg = 0; kg < 4; kg++) {
+                *reinterpret_cast<float4 *>(dst + dt * 32 + kg * 8 + half * 4) =
+                    make_float4(O[dt][kg * 4], O[dt][kg * 4 + 1], O[dt][kg * 4 + 2], O[dt][kg * 4 + 3]);
+            }
+        }
+        if (half == 0) {
+            *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+        }
+    }
+    __threadfence();
+    __syncthreads();
+    int32_t *counter = p.counters + static_cast<uint64_t>(blockIdx.z) * gridDim.y + blockIdx.y;
+    if (threadIdx.x == 0) {
+        *flag = atomicAdd(counter, 1);
+    }
+    __syncthreads();
+    if (*flag != static_cast<int32_t>(n_splits) - 1) {
+        return;
+    }
+    __threadfence();
+
+    constexpr int CH = DV / 4;  // float4 chunks per row
+    const uint32_t rows = m_last - m_first + 1;
+    for (uint32_t it = threadIdx.x; it < rows * CH; it += kThreads) {
+        const uint32_t mm = m_first + it / CH, c = it % CH;
+        const uint32_t t2 = static_cast<uint32_t>(qstart) + mm / G;
+        const uint32_t h2 = kvh * G + mm % G;
+        const uint64_t base = (static_cast<uint64_t>(t2) * p.n_heads + h2) * p.max_splits;
+        float mxx = -INFINITY;
+        for (uint32_t s = 0; s < n_splits; s++) {
+            mxx = fmaxf(mxx, p.part_ml[(base + s) * 2]);
+        }
+        const float ms = mxx == -INFINITY ? 0.f : mxx;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float lsum = 0.f;
+        for (uint32_t s = 0; s < n_splits; s++) {
+            const float2 ml = *reinterpret_cast<const float2 *>(p.part_ml + (base + s) * 2);
+            const float w = fast_exp2(ml.x - ms);
+            lsum += ml.y * w;
+            const float4 x = *reinterpret_cast<const float4 *>(p.part_acc + (base + s) * DV + c * 4);
+            acc.x += x.x * w;
+            acc.y += x.y * w;
+            acc.z += x.z * w;
+            acc.w += x.w * w;
+        }
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+        uint2 o;
+        o.x = T::pack(acc.x * inv, acc.y * inv);
+        o.y = T::pack(acc.z * inv, acc.w * inv);
+        *reinterpret_cast<uint2 *>(p.out + static_cast<uint64_t>(t2) * p.out_tok_stride + static_cast<uint64_t>(h2) * DV + c * 4) = o;
+    }
+    if (threadIdx.x == 0) {
+        *counter = 0;
+    }
+}
+
+template <int DQK, int DV, int BN>
+constexpr size_t lds_bytes()
+{
+    return static_cast<size_t>(BN) * (DQK + 8) * 2 + static_cast<size_t>(DV) * (BN + 8) * 2 + BN * 8 + 16;
+}
+
+template <typename T, int DQ0, int DQ1, int DV, int BN, bool SEPARATE_V>
+int launch_kernel(hipStream_t stream, const MfmaParams &p, dim3 grid)
+{
+    constexpr size_t lds = lds_bytes<DQ0 + DQ1, DV, BN>();
+    auto kernel = mfma_attention_kernel<T, DQ0, DQ1, DV, BN, SEPARATE_V>;
+    if (lds > 64 * 1024) {
+        static bool configured = false;  // per instantiation
+        if (!configured) {
+            XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            configured = true;
+        }
+    }
+    kernel<<<grid, kThreads, lds, stream>>>(p);
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+void fill_common(MfmaParams &p, void *workspace, uint32_t total_tokens, uint32_t n_heads, uint32_t dv,
+                 uint32_t max_splits)
+{
+    char *ws = static_cast<char *>(workspace);
+    p.counters = reinterpret_cast<int32_t *>(ws);
+    p.part_acc = ws ? reinterpret_cast<float *>(ws + XLITE_HIP_WS_COUNTER_BYTES) : nullptr;
+    p.part_ml = ws ? p.part_acc + static_cast<size_t>(total_tokens) * n_heads * max_splits * dv : nullptr;
+}
+
+}  // namespace
+
+bool mfma_gqa_supported(uint32_t head_dim) { return head_dim == 64 || head_dim == 128; }
+
+size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits)
+{
+    if (splits <= 1) {
+        return XLITE_HIP_WS_COUNTER_BYTES;
+    }
+    return XLITE_HIP_WS_COUNTER_BYTES +
+           static_cast<size_t>(total_tokens) * n_heads * splits * (dv + 2) * sizeof(float);
+}
+
+// Number of KV splits so that about two workgroups per compute unit exist; the split length is a
+// multiple of `tile` tokens.
+uint32_t mfma_pick_splits(uint32_t total_tokens, uint32_t rows_per_token, uint32_t batch,
+                          uint32_t parallel_heads, uint32_t max_ctx, uint32_t tile)
+{
+    const uint64_t m_tiles = (static_cast<uint64_t>(total_tokens) * rows_per_token + kMTile - 1) / kMTile + batch;
+    const uint64_t base = m_tiles * parallel_heads;
+    const uint64_t want = 512;
+    if (base >= want) {
+        return 1;
+    }
+    uint64_t splits = (want + base - 1) / base;
+    const uint64_t max_by_len = (max_ctx + 4 * tile - 1) / (4 * tile);  // at least four tiles each
+    if (splits > max_by_len) {
+        splits = max_by_len;
+    }
+    return static_cast<uint32_t>(splits < 1 ? 1 : splits);
+}
+
+int launch_mfma_gqa(hipStream_t stream, const AttentionArgs &a)
+{
+    constexpr int BN = 64;
+    const uint32_t G = a.n_heads / a.n_kv_heads;
+    const uint32_t max_ctx = a.max_num_block * a.block_size;
+    uint32_t splits = mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, max_ctx, BN);
+    const uint32_t m_tiles = ceil_div(a.total_tokens * G, kMTile) + a.batch;
+    if (static_cast<size_t>(m_tiles) * a.n_kv_heads * sizeof(int32_t) > XLITE_HIP_WS_COUNTER_BYTES ||
+        a.workspace == nullptr ||
+        a.workspace_bytes < mfma_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, splits)) {
+        splits = 1;  // no scratch: every M tile walks its whole KV range
+    }
+    uint32_t split_len = ceil_div(ceil_div(max_ctx, splits), BN) * BN;
+    if (split_len == 0) {
+        split_len = BN;
+    }
+    const uint32_t max_splits = ceil_div(max_ctx, split_len);
+
+    MfmaParams p{};
+    const uint32_t row = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
+    p.q0 = static_cast<const uint16_t *>(a.qkv);
+    p.q0_tok_stride = row;
+    p.q0_head_stride = a.head_dim;
+    p.k0 = static_cast<const uint16_t *>(a.k_cache);
+    p.v = static_cast<const uint16_t *>(a.v_cache);
+    p.k0_tok_stride = a.n_kv_heads * a.head_dim;
+    p.out = static_cast<uint16_t *>(a.output);
+    p.out_tok_stride = a.n_heads * a.head_dim;
+    p.query_start_loc = a.query_start_loc;
+    p.lens = a.lens;
+    p.cached_lens = a.cached_lens;
+    p.block_tables = a.block_tables;
+    p.rows_per_pos = G;
+    p.n_heads = a.n_heads;
+    p.batch = a.batch;
+    p.block_size = a.block_size;
+    p.block_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
+    p.max_num_block = a.max_num_block;
+    p.dense_len = 0;
+    p.split_len = split_len;
+    p.max_splits = max_splits;
+    p.scale_log2e = kLog2e;
+    fill_common(p, a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_splits);
+
+    dim3 grid(max_splits, m_tiles, a.n_kv_heads);
+    const bool bf = a.dtype == XLITE_HIP_BF16;
+    if (a.head_dim == 128) {
+        return bf ? launch_kernel<BF16, 128, 0, 128, BN, true>(stream, p, grid)
+                  : launch_kernel<FP16, 128, 0, 128, BN, true>(stream, p, grid);
+    }
+    return bf ? launch_kernel<BF16, 64, 0, 64, BN, true>(stream, p, grid)
+              : launch_kernel<FP16, 64, 0, 64, BN, true>(stream, p, grid);
+}
+
+int launch_mfma_mla(hipStream_t stream, const MlaArgs &a)
+{
+    constexpr int BN = 32;
+    const bool dense = a.block_tables == nullptr;
+    const uint32_t max_ctx = dense ? a.dense_len : a.max_num_blocks * a.block_size;
+    uint32_t splits = mfma_pick_splits(a.total_tokens, a.n_heads, a.batch, 1, max_ctx, BN);
+    const uint32_t m_tiles = ceil_div(a.total_tokens * a.n_heads, kMTile) + a.batch;
+    if (static_cast<size_t>(m_tiles) * sizeof(int32_t) > XLITE_HIP_WS_COUNTER_BYTES || a.workspace == nullptr ||
+        a.workspace_bytes < mfma_workspace_bytes(a.total_tokens, a.n_heads, a.kv_lora_rank, splits)) {
+        splits = 1;
+    }
+    uint32_t split_len = ceil_div(ceil_div(max_ctx, splits), BN) * BN;
+    if (split_len == 0) {
+        split_len = BN;
+    }
+    const uint32_t max_splits = ceil_div(max_ctx, split_len);
+
+    MfmaParams p{};
+    p.q0 = static_cast<const uint16_t *>(a.q_absorb);
+    p.q0_tok_stride = a.n_heads * a.kv_lora_rank;
+    p.q0_head_stride = a.kv_lora_rank;
+    p.q1 = static_cast<const uint16_t *>(a.qr);
+    p.q1_tok_stride = a.n_heads * a.rope_head_dim;
+    p.q1_head_stride = a.rope_head_dim;
+    p.k0 = static_cast<const uint16_t *>(a.k_cache);
+    p.k1 = static_cast<const uint16_t *>(a.pe_cache);
+    p.v = nullptr;
+    p.k0_tok_stride = a.kv_lora_rank;
+    p.k1_tok_stride = a.rope_head_dim;
+    p.out = static_cast<uint16_t *>(a.o_absorb);
+    p.out_tok_stride = a.n_heads * a.kv_lora_rank;
+    p.query_start_loc = a.query_start_loc;
+    p.lens = a.lens;
+    p.cached_lens = a.cached_lens;
+    p.block_tables = a.block_tables;
+    p.rows_per_pos = a.n_heads;
+    p.n_heads = a.n_heads;
+    p.batch = a.batch;
+    p.block_size = dense ? 1 : a.block_size;
+    p.block_shift = dense ? 0 : ((a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1);
+    p.max_num_block = a.max_num_blocks;
+    p.dense_len = a.dense_len;
+    p.split_len = split_len;
+    p.max_splits = max_splits;
+    p.scale_log2e = a.scale * kLog2e;
+    fill_common(p, a.workspace, a.total_tokens, a.n_heads, a.kv_lora_rank, max_splits);
+
+    dim3 grid(max_splits, m_tiles, 1);
+    if (a.kv_lora_rank == 512 && a.rope_head_dim == 64) {
+        return launch_kernel<BF16, 512, 64, 512, BN, false>(stream, p, grid);
+    }
+    return fail(XLITE_HIP_EINVAL, __func__,
+                "only kv_lora_rank 512 with rope_head_dim 64 is built for the matrix-core path");
+}
+
+}  // namespace xlite

@@ -84,8 +84,9 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
 #define XLITE_HIP_WS_COUNTER_BYTES 65536
 
 size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
-                                           uint32_t head_dim, uint32_t block_size,
-                                           uint32_t batch, uint32_t max_num_block);
+                                           uint32_t n_kv_heads, uint32_t head_dim,
+                                           uint32_t block_size, uint32_t batch,
+                                           uint32_t max_num_block);
 
 int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, const void *v_cache,
                         void *output, const int32_t *query_start_loc, const int32_t *lens,

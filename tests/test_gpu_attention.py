@@ -1,0 +1,191 @@
+"""GPU parity of the GQA attention operator (decode, prefill, int8 KV) against the CPU oracle.
+Tolerance for bf16/fp16 outputs: max abs <= 2e-2 and mean abs <= 2e-3 (5e-2 max for int8 KV)."""
+import numpy as np
+import pytest
+import torch
+
+from gvirt_amd import workloads as W
+from oracle import xlite_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MAX_ABS, MEAN_ABS, MAX_ABS_INT8 = 2e-2, 2e-3, 5e-2
+
+
+def run_attention(rt, w, **kw):
+    from gvirt_amd._C import attention
+    s = w["shape"]
+    d = W.to_device(w, DEV)
+    d["output"].zero_()
+    attention(rt, d["qkv"], d["k_cache"], d["v_cache"], d["output"], d["query_start_loc"], d["lens"],
+              d["cached_lens"], d["block_tables"], s.n_heads, s.n_kv_heads, s.head_dim, s.block_size, w["batch"],
+              w["max_num_block"], k_scale=d.get("k_scale"), v_scale=d.get("v_scale"), **kw)
+    return d["output"].float().cpu()
+
+
+def oracle_attention(w, seqs=None):
+    s = w["shape"]
+    return O.attention_ref(w["qkv"], w["k_cache"], w["v_cache"], w["query_start_loc"], w["lens"], w["cached_lens"],
+                           w["block_tables"], s.n_heads, s.n_kv_heads, s.head_dim, s.block_size, w["batch"],
+                           w["max_num_block"], w.get("k_scale"), w.get("v_scale"), seqs=seqs)
+
+
+def check(got, ref, max_abs=MAX_ABS, mean_abs=MEAN_ABS, rows=None):
+    if rows is not None:
+        got, ref = got[rows], ref[rows]
+    err = (got - ref).abs()
+    assert float(err.max()) <= max_abs, "max abs err %g" % float(err.max())
+    assert float(err.mean()) <= mean_abs, "mean abs err %g" % float(err.mean())
+
+
+def generic_case(seed, lens, clens, nH, nKV, d, bs, dtype, rms=False):
+    g = torch.Generator().manual_seed(seed)
+    batch, T = len(lens), sum(lens)
+    maxblk = max((l + c + bs - 1) // bs for l, c in zip(lens, clens))
+    NB = batch * maxblk + 1
+    qkv = torch.randn(T, nH + 2 * nKV, d, generator=g)
+    kc = torch.randn(NB, bs, nKV, d, generator=g)
+    vc = torch.randn(NB, bs, nKV, d, generator=g)
+    if rms:  # the reference test normalises q, k, v rows (xlite/tests/kernels/attention.py:72-75)
+        qkv, kc, vc = [x / x.pow(2).mean(-1, keepdim=True).add(1e-6).sqrt() for x in (qkv, kc, vc)]
+    else:
+        qkv[:, :nH] *= d ** -0.5
+    tables = torch.randperm(NB, generator=g)[: batch * maxblk].int()
+    shape = W.GqaShape("t", nH, nKV, d, bs, dtype)
+    return dict(shape=shape, batch=batch, qkv=qkv.reshape(T, -1).to(dtype), k_cache=kc.to(dtype), v_cache=vc.to(dtype),
+                output=torch.zeros(T, nH * d, dtype=dtype), query_start_loc=torch.tensor(np.cumsum([0] + lens[:-1]), dtype=torch.int32),
+                lens=torch.tensor(lens, dtype=torch.int32), cached_lens=torch.tensor(clens, dtype=torch.int32),
+                block_tables=tables, max_num_block=maxblk)
+
+
+def test_config1_qwen2_05b_decode(rt):
+    """Benchmark configuration 1 in full: also the one the CPU golden path runs completely."""
+    w = W.gqa_decode(W.QWEN2_05B, W.c1_context_lengths(), W.SEED_BASE + 1)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
+# model shapes of xlite/tests/kernels/attention.py:28-39
+MODELS = [(1, 1, 64, torch.float16), (1, 1, 64, torch.bfloat16), (1, 1, 128, torch.bfloat16), (14, 2, 64, torch.bfloat16),
+          (5, 1, 128, torch.bfloat16), (8, 1, 128, torch.bfloat16), (4, 1, 128, torch.bfloat16), (32, 32, 128, torch.float16),
+          (20, 20, 128, torch.float16), (32, 8, 128, torch.bfloat16)]
+# decode workloads of the same file (:50-59), contexts bounded to what the CPU oracle does in seconds
+DECODE_WORK = [([0], [1]), ([1800], [1]), ([8, 13, 65, 11, 5], [1] * 5), ([4000] * 2, [1] * 2), ([16000, 127], [1] * 2),
+               ([127, 128, 129, 255, 256, 257], [1] * 6)]
+
+
+@pytest.mark.parametrize("model", MODELS)
+@pytest.mark.parametrize("work", DECODE_WORK)
+def test_decode_model_grid(rt, model, work):
+    nH, nKV, d, dtype = model
+    clens, lens = work
+    w = generic_case(11, lens, clens, nH, nKV, d, 128, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
+def test_decode_special_cases(rt):
+    # single visible key: the output is v0 exactly (softmax of one element is 1.0)
+    w = generic_case(12, [1, 1], [0, 0], 8, 2, 128, 128, torch.bfloat16)
+    got = run_attention(rt, w)
+    v0 = torch.stack([w["v_cache"][w["block_tables"][i].long(), 0] for i in range(2)]).float()
+    assert torch.equal(got, v0.repeat_interleave(4, 1).reshape(2, -1))
+    # block permutation invariance: identity table over a re-packed cache gives identical bits
+    w = generic_case(13, [1] * 3, [700, 300, 511], 14, 2, 64, 128, torch.bfloat16)
+    a = run_attention(rt, w)
+    t = w["block_tables"].long()
+    w2 = dict(w); w2["k_cache"] = w["k_cache"][t].contiguous(); w2["v_cache"] = w["v_cache"][t].contiguous()
+    w2["block_tables"] = torch.arange(t.numel(), dtype=torch.int32)
+    assert torch.equal(a, run_attention(rt, w2))
+    # idempotence: the ticket counters are left at zero, a second call gives the same bits
+    assert torch.equal(a, run_attention(rt, w))
+    # non power-of-two block size and a block size smaller than the split granularity
+    for bs in (48, 16):
+        w = generic_case(14, [1] * 2, [1000, 37], 8, 2, 128, bs, torch.bfloat16)
+        check(run_attention(rt, w), oracle_attention(w))
+
+
+def test_decode_int8_kv(rt):
+    ctx = [129, 4100, 640, 17, 2048, 9000]
+    w = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=True)
+    got = run_attention(rt, w)
+    check(got, oracle_attention(w), max_abs=MAX_ABS_INT8)
+    # and against the unquantised cache the error stays within the int8 budget as well
+    w16 = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=False)
+    check(got, oracle_attention(w16), max_abs=MAX_ABS_INT8, mean_abs=1e-2)
+
+
+def test_config2_llama3_8b_decode_sampled(rt):
+    """Configuration 2 at full size on the GPU; the oracle checks a sample of sequences, and the
+    reshape-and-cache step of the 64 new tokens is checked bit-exactly first."""
+    from gvirt_amd._C import rope_and_cache
+    w = W.gqa_decode(W.LLAMA3_8B, [4096] * 64, W.SEED_BASE + 2, device=DEV)
+    s = w["shape"]
+    r = W.rope_inputs(s, w, W.SEED_BASE + 2)
+    sample = [0, 17, 63]
+    tables = w["block_tables"].view(64, -1)
+    before = {i: (w["k_cache"][tables[i].long()].cpu(), w["v_cache"][tables[i].long()].cpu()) for i in sample}
+    inout_cpu = r["inout"].cpu()
+    rope_and_cache(rt, r["inout"], w["k_cache"], w["v_cache"], r["position"], r["cosin"], r["slot_mapping"],
+                   s.n_heads, s.n_kv_heads, s.head_dim, s.head_dim, s.block_size, True)
+    # oracle on a compact copy: the sampled sequences' blocks re-packed with an identity table
+    for i in sample:
+        kc, vc = before[i]
+        pos = r["position"][i:i + 1].cpu()
+        slot = torch.tensor([int(pos) // 128 * 128 + int(pos) % 128], dtype=torch.int32)
+        row = inout_cpu[i:i + 1].clone()
+        O.rope_and_cache_ref(row, kc, vc, pos, r["cosin"].cpu(), slot, s.n_heads, s.n_kv_heads, s.head_dim, s.head_dim, 128)
+        assert torch.equal(w["k_cache"][tables[i].long()].cpu().view(torch.int16), kc.view(torch.int16))
+        assert torch.equal(w["v_cache"][tables[i].long()].cpu().view(torch.int16), vc.view(torch.int16))
+        assert torch.equal(r["inout"][i:i + 1].cpu().view(torch.int16), row.view(torch.int16))
+    w["qkv"] = r["inout"]
+    got = run_attention(rt, w)
+    wc = W.to_device({k: v for k, v in w.items() if k != "shape"}, "cpu"); wc["shape"] = s
+    ref = oracle_attention(wc, seqs=sample)
+    check(got, ref, rows=sample)
+    # size-independent property on all 64 sequences: each output row is a convex combination of V
+    # rows, so it is bounded by the column-wise extremes of the V rows the sequence can see
+    out = got.view(64, s.n_kv_heads, 4, s.head_dim)
+    for i in range(0, 64, 7):
+        v = w["v_cache"][tables[i].long()].reshape(-1, s.n_kv_heads, s.head_dim)[:4096].float().cpu()
+        assert bool((out[i] <= v.max(0).values.unsqueeze(1) + 1e-2).all())
+        assert bool((out[i] >= v.min(0).values.unsqueeze(1) - 1e-2).all())
+
+
+PREFILL_WORK = [([0], [30]), ([0], [77]), ([0], [1800]), ([128], [1800]), ([0] * 8, [789, 65, 13, 2545, 24, 190, 1432, 124]),
+                ([300, 0, 4000], [5, 130, 1])]
+
+
+@pytest.mark.parametrize("model", [(1, 1, 64, torch.float16), (1, 1, 128, torch.bfloat16), (14, 2, 64, torch.bfloat16),
+                                   (5, 1, 128, torch.bfloat16), (8, 1, 128, torch.bfloat16), (28, 4, 128, torch.bfloat16)])
+@pytest.mark.parametrize("work", PREFILL_WORK)
+def test_prefill_model_grid(rt, model, work):
+    """Prefill / chunked-prefill workloads of xlite/tests/kernels/attention.py:42-60 (bounded)."""
+    nH, nKV, d, dtype = model
+    clens, lens = work
+    w = generic_case(21, lens, clens, nH, nKV, d, 128, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
+def test_prefill_rows_equal_decode_steps(rt):
+    """Row r of a prefill chunk must match the same row issued alone as a decode step."""
+    w = generic_case(22, [40], [200], 8, 2, 128, 128, torch.bfloat16)
+    full = run_attention(rt, w)
+    for r in (0, 17, 39):
+        one = dict(w); one["qkv"] = w["qkv"][r:r + 1].contiguous(); one["batch"] = 1
+        one["lens"] = torch.tensor([1], dtype=torch.int32); one["cached_lens"] = torch.tensor([200 + r], dtype=torch.int32)
+        one["query_start_loc"] = torch.tensor([0], dtype=torch.int32); one["output"] = torch.zeros(1, 8 * 128, dtype=torch.bfloat16)
+        assert float((run_attention(rt, one)[0] - full[r]).abs().max()) <= 1e-2
+
+
+def test_config3_qwen25_7b_chunked_prefill_sampled(rt):
+    """Configuration 3 shape with two of the eight sequences (full-length ones are left to the
+    benchmark): every 2048-token chunk attends to the prior paged KV."""
+    lens = [2500, 1024]
+    caches = None
+    for ci in range(2):
+        w = W.gqa_prefill_chunk(W.QWEN25_7B, lens, ci, 2048, W.SEED_BASE + 3, caches=caches)
+        if w is None:
+            break
+        caches = w["caches"]
+        got = run_attention(rt, w)
+        ref = oracle_attention(w)
+        check(got, ref)

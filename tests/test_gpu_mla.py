@@ -1,0 +1,146 @@
+"""GPU parity of the MLA operators (absorbed attention, mla_v2, mla_v3, einsum) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from gvirt_amd import workloads as W
+from oracle import xlite_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def check(got, ref, max_abs=2e-2, mean_abs=2e-3):
+    err = (got - ref).abs()
+    assert float(err.max()) <= max_abs, "max abs err %g" % float(err.max())
+    assert float(err.mean()) <= mean_abs, "mean abs err %g" % float(err.mean())
+
+
+def mla_case(seed, lens, clens, nH, bs=128, C=512, R=64):
+    g = torch.Generator().manual_seed(seed)
+    batch, T = len(lens), sum(lens)
+    maxblk = max((l + c + bs - 1) // bs for l, c in zip(lens, clens))
+    NB = batch * maxblk + 1
+    rms = lambda x: x / x.pow(2).mean(-1, keepdim=True).add(1e-6).sqrt()
+    return dict(batch=batch, T=T, nH=nH, bs=bs, C=C, R=R, maxblk=maxblk,
+                qa=(rms(torch.randn(T, nH, C, generator=g)) * 4).bfloat16(), qr=rms(torch.randn(T, nH, R, generator=g)).bfloat16(),
+                kc=rms(torch.randn(NB, bs, C, generator=g).clamp(0.2, 1)).bfloat16(), pc=rms(torch.randn(NB, bs, R, generator=g)).bfloat16(),
+                qsl=torch.tensor(np.cumsum([0] + lens[:-1]), dtype=torch.int32), lens=torch.tensor(lens, dtype=torch.int32),
+                clens=torch.tensor(clens, dtype=torch.int32), tables=torch.randperm(NB, generator=g)[: batch * maxblk].int())
+
+
+def run_mla(rt, c, scale):
+    from gvirt_amd._C import mla_attention
+    out = torch.zeros(c["T"], c["nH"], c["C"], dtype=torch.bfloat16, device=DEV)
+    mla_attention(rt, c["qa"].to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), out, c["qsl"].to(DEV),
+                  c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), c["nH"], c["R"], c["C"], c["bs"], c["batch"],
+                  c["maxblk"], scale)
+    rt.synchronize()
+    return out.float().cpu()
+
+
+def oracle_mla(c, scale):
+    return O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"],
+                               c["R"], c["C"], c["bs"], c["batch"], c["maxblk"], scale)
+
+
+# workloads of xlite/tests/kernels/mla.py:61-76 (bounded) on its deepseek_v3 (16 heads) and glm5 (8 heads) shapes
+MLA_WORK = [([0], [1]), ([0], [30]), ([0], [77]), ([0], [128]), ([0], [256]), ([100], [30]), ([128], [128]),
+            ([0] * 4, [189, 65, 13, 545]), ([4000] * 2, [1] * 2), ([8, 13, 65, 11, 5], [1] * 5)]
+
+
+@pytest.mark.parametrize("nH", [16, 8, 128])
+@pytest.mark.parametrize("work", MLA_WORK)
+def test_mla_attention_grid(rt, nH, work):
+    clens, lens = work
+    if nH == 128 and sum(lens) > 200:
+        pytest.skip("bounded: the CPU oracle for 128 heads x long prefill takes minutes")
+    c = mla_case(31, lens, clens, nH)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
+def test_config4_deepseek_r1_decode_sampled(rt):
+    """Configuration 4 shape (128 heads, block 64) with 4 of the 32 sequences at full context."""
+    ctx = W.c4_context_lengths()[:4]
+    w = W.mla_decode(W.MlaShape(), ctx, W.SEED_BASE + 4)
+    s = w["shape"]
+    from gvirt_amd._C import mla_attention
+    d = W.to_device(w, DEV)
+    mla_attention(rt, d["q_absorb"], d["qr"], d["k_cache"], d["pe_cache"], d["o_absorb"], d["query_start_loc"], d["lens"],
+                  d["cached_lens"], d["block_tables"], s.n_heads, s.rope_head_dim, s.kv_lora_rank, s.block_size, 4,
+                  w["max_num_blocks"], s.scale)
+    rt.synchronize()
+    ref = O.mla_attention_ref(w["q_absorb"], w["qr"], w["k_cache"], w["pe_cache"], w["query_start_loc"], w["lens"],
+                              w["cached_lens"], w["block_tables"], s.n_heads, s.rope_head_dim, s.kv_lora_rank, s.block_size,
+                              4, w["max_num_blocks"], s.scale)
+    check(d["o_absorb"].float().cpu(), ref)
+
+
+@pytest.mark.parametrize("m,h,t,d", [(3, 4, 192, 512), (3, 4, 512, 192), (3, 4, 128, 512), (3, 4, 512, 128), (530, 4, 256, 512),
+                                     (963, 8, 512, 128), (32, 128, 128, 512)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_einsum(rt, m, h, t, d, dtype):
+    """Cases of xlite/tests/kernels/einsum_mht_mhd.py:19-33 (bounded), both weight layouts."""
+    from gvirt_amd._C import einsum_mht_htd_mhd, einsum_mht_hdt_mhd
+    g = torch.Generator().manual_seed(m + t)
+    a = torch.randn(m, h, t, generator=g).to(dtype)
+    w = (torch.randn(h, t, d, generator=g) / t ** 0.5).to(dtype)
+    ref = O.einsum_ref(a, w)
+    out = torch.zeros(m, h, d, dtype=dtype, device=DEV)
+    einsum_mht_htd_mhd(rt, a.to(DEV), w.to(DEV), out, m, h, t, d)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=2e-2, rtol=1e-2)
+    out2 = torch.zeros(m, h, d, dtype=dtype, device=DEV)
+    einsum_mht_hdt_mhd(rt, a.to(DEV), w.transpose(1, 2).contiguous().to(DEV), out2, m, h, t, d)
+    assert torch.equal(out.cpu().view(torch.int16), out2.cpu().view(torch.int16))
+
+
+@pytest.mark.parametrize("nH,nope,vd", [(16, 128, 128), (8, 192, 256)])
+def test_mla_v2_three_stage(rt, nH, nope, vd):
+    """deepseek_v3 / glm5 shapes of xlite/tests/kernels/mla.py:54-58, rtol 5e-2 as there (:255)."""
+    from gvirt_amd._C import mla_v2
+    c = mla_case(41, [1, 40], [300, 17], nH)
+    g = torch.Generator().manual_seed(42)
+    rms = lambda x: x / x.pow(2).mean(-1, keepdim=True).add(1e-6).sqrt()
+    qwq = rms(torch.randn(c["T"], nH, nope + 64, generator=g)).bfloat16()
+    wkvb = torch.randn(nH, nope + vd, 512, generator=g).clamp(0.2, 1)
+    wuk_t = wkvb[:, :nope].contiguous().bfloat16()
+    wuv = wkvb[:, -vd:].transpose(1, 2).contiguous().bfloat16()
+    scale = (nope + 64) ** -0.5
+    out = torch.zeros(c["T"], nH, vd, dtype=torch.bfloat16, device=DEV)
+    empty = torch.zeros(0, dtype=torch.int32, device=DEV)
+    mla_v2(rt, qwq.to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), wuk_t.to(DEV), wuv.to(DEV), out, c["qsl"].to(DEV),
+           c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), nH, 64, nope, vd, 512, c["bs"], c["batch"], c["maxblk"],
+           scale, empty, 0, False, True, 8192)
+    ref = O.mla_v2_ref(qwq, c["qr"], c["kc"], c["pc"], wuk_t, wuv, c["qsl"], c["lens"], c["clens"], c["tables"], nH, 64, nope, vd,
+                       512, c["bs"], c["batch"], c["maxblk"], scale)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=3e-2, rtol=5e-2)
+    with pytest.raises(RuntimeError, match="NZ"):
+        mla_v2(rt, qwq.to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), wuk_t.to(DEV), wuv.to(DEV), out,
+               c["qsl"].to(DEV), c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), nH, 64, nope, vd, 512, c["bs"],
+               c["batch"], c["maxblk"], scale, empty, 0, True)
+
+
+@pytest.mark.parametrize("cached,topk", [([127], 512), ([2047, 8191, 5841], 2048), ([4096], 512)])
+def test_gather_then_mla_v3(rt, cached, topk):
+    """Decode + sparse path of xlite/tests/kernels/mla_v3.py (bounded): gather, then dense attention."""
+    from gvirt_amd._C import gather_sparse_kv_cache, mla_v3
+    batch = len(cached)
+    c = mla_case(51, [1] * batch, cached, 16)
+    g = torch.Generator().manual_seed(52)
+    idx = []
+    for cl in cached:
+        n = cl + 1
+        p = torch.randperm(n, generator=g)[:topk]
+        if n < topk:
+            p = torch.cat([p, p[-1:].expand(topk - n)])
+        idx.append(torch.sort(p).values)
+    idx = torch.stack(idx).int()
+    kd = torch.zeros(batch, topk, 1, 512, dtype=torch.bfloat16, device=DEV); pd = torch.zeros(batch, topk, 1, 64, dtype=torch.bfloat16, device=DEV)
+    gather_sparse_kv_cache(rt, c["kc"].to(DEV), c["pc"].to(DEV), c["tables"].to(DEV), idx.to(DEV), c["lens"].to(DEV),
+                           c["clens"].to(DEV), kd, pd, batch, topk, c["bs"], c["maxblk"], 512, 64, 1)
+    out = torch.zeros(batch, 16, 512, dtype=torch.bfloat16, device=DEV)
+    mla_v3(rt, c["qa"].to(DEV), c["qr"].to(DEV), kd, pd, out, c["qsl"].to(DEV), c["lens"].to(DEV), c["clens"].to(DEV), 16, 64,
+           512, batch, topk, 192 ** -0.5)
+    ref = O.mla_v3_ref(c["qa"], c["qr"], kd.cpu(), pd.cpu(), c["qsl"], c["lens"], c["clens"], 16, 64, 512, batch, topk, 192 ** -0.5)
+    check(out.float().cpu(), ref)
