@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c3|c4|c5|all]
+
+Default (what the driver runs): configuration 2 of BASELINE.json — Llama-3-8B-shape GQA
+flash-decode, batch 64, every sequence at context 4096, bf16 paged KV cache with block size 128,
+plus the reshape-and-cache (`rope_and_cache`) of the 64 new tokens. One step = one
+`rope_and_cache` + one `attention` call over that batch, inputs resident in HBM. Prints ONE JSON
+line; `value` is KV bytes read per second over the whole step. `roofline` prices the dominant
+kernel (the decode attention kernel) against the 8 TB/s HBM peak; `cpu_baseline` times the CPU
+oracle on a bounded sample of the same workload on the host cores.
+
+Other configurations (`--config`) print the same kind of line for their own workload; `all`
+prints one line per configuration (the first line is still configuration 2).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def _events(torch):
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def _time_region(torch, fn, iters):
+    """Average milliseconds per call of `fn` over `iters` back-to-back asynchronous calls, from HIP
+    events recorded on the stream the kernels are launched on (torch's current stream)."""
+    a, b = _events(torch)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def _cpu_info():
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return model
+
+
+def _cpu_threads(torch):
+    n = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    n = max(1, min(n, os.cpu_count() or 1))
+    torch.set_num_threads(n)
+    return n
+
+
+def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_rope=True):
+    from gvirt_amd import workloads as W
+    from gvirt_amd import _C
+    dev = "cuda:0"
+    w = W.gqa_decode(shape, ctx, seed, device=dev, int8_kv=int8)
+    r = W.rope_inputs(shape, w, seed) if with_rope and not int8 else None
+    s = shape
+    B = w["batch"]
+    rt.blocking = False
+    pristine = r["inout"].clone() if r is not None else None
+
+    def rope():
+        _C.rope_and_cache(rt, r["inout"], w["k_cache"], w["v_cache"], r["position"], r["cosin"], r["slot_mapping"],
+                          s.n_heads, s.n_kv_heads, s.head_dim, s.head_dim, s.block_size, True)
+
+    def attn():
+        _C.attention(rt, r["inout"] if r is not None else w["qkv"], w["k_cache"], w["v_cache"], w["output"],
+                     w["query_start_loc"], w["lens"], w["cached_lens"], w["block_tables"], s.n_heads, s.n_kv_heads,
+                     s.head_dim, s.block_size, B, w["max_num_block"], k_scale=w["k_scale"], v_scale=w["v_scale"])
+
+    def step():
+        if r is not None:
+            rope()
+        attn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # dominant kernel alone: back-to-back launches of the attention op between two events
+    ms_kernel = _time_region(torch, attn, max(args.steps, 20))
+    ms_rope = _time_region(torch, rope, max(args.steps, 20)) if r is not None else 0.0
+
+    kv_bytes = w["kv_bytes"]
+    qo_bytes = 2 * B * s.n_heads * s.head_dim * 2 + sum((c + s.block_size - 1) // s.block_size for c in ctx) * 4
+    alg_bytes = kv_bytes + qo_bytes
+    achieved = alg_bytes / (ms_kernel * 1e-3) / 1e9
+
+    # parity spot check through the oracle (the checker, not the thing measured). rope_and_cache
+    # rotates its rows in place, so the timed steps kept re-rotating the same buffer (same work,
+    # drifting values); one more step from the pristine rows gives the output that is checked.
+    if r is not None:
+        r["inout"].copy_(pristine)
+    step()
+    torch.cuda.synchronize()
+    cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+        from oracle import xlite_oracle as O
+        ncpu = _cpu_threads(torch)
+        sample = list(range(0, B, max(1, B // 4)))[:4]
+        wc = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in w.items()}
+        qkv_c = (r["inout"] if r is not None else w["qkv"]).cpu()
+        got = w["output"].float().cpu()
+
+        def run_oracle():
+            return O.attention_ref(qkv_c, wc["k_cache"], wc["v_cache"], wc["query_start_loc"], wc["lens"],
+                                   wc["cached_lens"], wc["block_tables"], s.n_heads, s.n_kv_heads, s.head_dim,
+                                   s.block_size, B, w["max_num_block"], wc["k_scale"], wc["v_scale"], seqs=sample)
+        ref = run_oracle()  # warm-up + parity
+        err = (got[sample] - ref[sample]).abs()
+        tol = 5e-2 if int8 else 2e-2
+        if float(err.max()) > tol:
+            raise SystemExit("parity check failed in bench: max abs err %g" % float(err.max()))
+        reps, t_cpu = 0, 0.0
+        while reps < 3 and t_cpu < 20.0:
+            t1 = time.perf_counter()
+            run_oracle()
+            t_cpu += time.perf_counter() - t1
+            reps += 1
+        per_elt = 1 if int8 else 2
+        sample_bytes = sum(ctx[i] for i in sample) * s.n_kv_heads * s.head_dim * 2 * per_elt
+        cpu = {"value": round(sample_bytes / (t_cpu / reps) / 1e9, 3), "unit": "GB/s", "cores": ncpu, "kind": "port",
+               "sample": "%d of %d sequences (indices %s), %d timed runs of the PyTorch oracle, %s" %
+                         (len(sample), B, sample, reps, _cpu_info()),
+               "max_abs_err_vs_gpu": float(err.max())}
+
+    tokens_per_s = B / (ms_step * 1e-3)
+    return {
+        "metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X",
+        "value": round(kv_bytes / (ms_step * 1e-3) / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8" if int8 else "bf16", "data": "synthetic",
+        "config": {"workload": name, "batch": B, "n_heads": s.n_heads, "n_kv_heads": s.n_kv_heads,
+                   "head_dim": s.head_dim, "block_size": s.block_size, "ctx_total": int(sum(ctx)),
+                   "ctx_max": int(max(ctx)), "kv_bytes_per_step": int(kv_bytes)},
+        "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "tokens_per_s": round(tokens_per_s, 1),
+        "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
+        "roofline": {"bound": "hbm", "kernel": "decode_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": int(alg_bytes)},
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_prefill(args, torch, rt):
+    from gvirt_amd import workloads as W
+    from gvirt_amd import _C
+    shape = W.QWEN25_7B
+    lens = W.c3_total_lengths()
+    dev = "cuda:0"
+    rt.blocking = False
+    chunks, caches, ci = [], None, 0
+    while True:
+        w = W.gqa_prefill_chunk(shape, lens, ci, 2048, W.SEED_BASE + 3, device=dev, caches=caches)
+        if w is None:
+            break
+        caches = w["caches"]
+        chunks.append(w)
+        ci += 1
+
+    def step():
+        for w in chunks:
+            _C.attention(rt, w["qkv"], w["k_cache"], w["v_cache"], w["output"], w["query_start_loc"], w["lens"],
+                         w["cached_lens"], w["block_tables"], shape.n_heads, shape.n_kv_heads, shape.head_dim,
+                         shape.block_size, w["batch"], w["max_num_block"])
+
+    for _ in range(max(1, args.warmup // 4)):
+        step()
+    steps = max(3, args.steps // 5)
+    ms = _time_region(torch, step, steps)
+    flops = sum(w["flops"] for w in chunks)
+    tokens = sum(w["tokens"] for w in chunks)
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(tf, 2),
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": max(1, args.warmup // 4), "ms_per_step": round(ms, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "c3 qwen2.5-7b chunked causal prefill", "total_lens": lens, "chunk": 2048,
+                       "calls_per_step": len(chunks)},
+            "tokens_per_s": round(tokens / (ms * 1e-3), 1),
+            "roofline": {"bound": "mfma", "kernel": "mfma_attention_kernel", "achieved": round(tf, 2),
+                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                         "traffic": None, "algorithmic_flops_per_step": int(flops)},
+            "cpu_baseline": None}
+
+
+def bench_mla(args, torch, rt):
+    from gvirt_amd import workloads as W
+    from gvirt_amd import _C
+    s = W.MlaShape()
+    ctx = W.c4_context_lengths()
+    w = W.mla_decode(s, ctx, W.SEED_BASE + 4, device="cuda:0")
+    rt.blocking = False
+
+    def step():
+        _C.mla_attention(rt, w["q_absorb"], w["qr"], w["k_cache"], w["pe_cache"], w["o_absorb"], w["query_start_loc"],
+                         w["lens"], w["cached_lens"], w["block_tables"], s.n_heads, s.rope_head_dim, s.kv_lora_rank,
+                         s.block_size, w["batch"], w["max_num_blocks"], s.scale)
+
+    for _ in range(args.warmup):
+        step()
+    ms = _time_region(torch, step, args.steps)
+    gbs = w["kv_bytes"] / (ms * 1e-3) / 1e9
+    tf = w["flops"] / (ms * 1e-3) / 1e12
+    floor_ms = max(w["kv_bytes"] / (HBM_PEAK_GBS * 1e9), w["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12)) * 1e3
+    return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
+            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "c4 deepseek-r1 MLA absorbed decode", "batch": 32, "n_heads": 128, "ctx_total": int(sum(ctx)),
+                       "kv_bytes_per_step": int(w["kv_bytes"]), "flops_per_step": int(w["flops"])},
+            "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1),
+            "roofline": {"bound": "hbm", "kernel": "mfma_attention_kernel", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
+            "cpu_baseline": None}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU's share only (no collectives, no sharding); run with --gpus 1",
+              file=sys.stderr)
+        raise SystemExit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible")
+    from gvirt_amd import workloads as W
+    from gvirt_amd._C import Runtime
+    rt = Runtime(0, 64)
+
+    todo = ["c2", "c1", "c5", "c3", "c4"] if args.config == "all" else [args.config]
+    for c in todo:
+        if c == "c2":
+            out = bench_gqa_decode(args, torch, rt, "c2 llama-3-8b GQA flash-decode + reshape_and_cache", W.LLAMA3_8B,
+                                   [4096] * 64, W.SEED_BASE + 2)
+        elif c == "c1":
+            out = bench_gqa_decode(args, torch, rt, "c1 qwen2-0.5b GQA decode", W.QWEN2_05B, W.c1_context_lengths(),
+                                   W.SEED_BASE + 1)
+        elif c == "c5":
+            out = bench_gqa_decode(args, torch, rt, "c5 llama-3-8b int8-KV decode", W.LLAMA3_8B, W.c5_context_lengths(),
+                                   W.SEED_BASE + 5, int8=True)
+        elif c == "c3":
+            out = bench_prefill(args, torch, rt)
+        elif c == "c4":
+            out = bench_mla(args, torch, rt)
+        else:
+            raise SystemExit("unknown config " + c)
+        print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -46,6 +46,9 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
 {
     XL_REQUIRE(dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16, "qkv/kCache/vCache/output dtype unsupported!");
     XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || kv_dtype == XLITE_HIP_KV_INT8, "kv cache dtype unsupported!");
+    if (batch == 0 || total_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(qkv && k_cache && v_cache && output && query_start_loc && lens && cached_lens && block_tables,
                "null tensor");
     XL_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
@@ -106,6 +109,9 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
     XL_REQUIRE(dtype == XLITE_HIP_BF16, "qAbsorb/qr/kCache/peCache/oAbsorb dtype unsupported!");
     XL_REQUIRE(top_k <= 2048, "topK should be less than or equal to 2048");
     XL_REQUIRE(top_k == 0, "top-k index masks are not built yet");
+    if (batch == 0 || total_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(q_absorb && qr && k_cache && pe_cache && o_absorb && query_start_loc && lens &&
                    cached_lens && block_tables,
                "null tensor");
@@ -130,6 +136,9 @@ extern "C" int xlite_hip_mla_v3(void *stream, const void *q_absorb, const void *
                                 size_t workspace_bytes)
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16, "qAbsorb/qr/kDenseCache/peDenseCache/oAbsorb dtype unsupported!");
+    if (batch == 0 || total_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(q_absorb && qr && k_dense && pe_dense && o_absorb && query_start_loc && lens && cached_lens,
                "null tensor");
     XL_REQUIRE(n_heads > 0 && index_topk > 0, "zero head count or dense length");

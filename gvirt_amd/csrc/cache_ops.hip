@@ -346,6 +346,9 @@ extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache
 {
     XL_REQUIRE(is_neox, "unsupported rope type gptj");
     XL_REQUIRE(dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16, "dtype unsupported!");
+    if (num_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(inout && k_cache && v_cache && position && cosin && slot_mapping, "null tensor");
     XL_REQUIRE(n_heads > 0 && n_kv_heads > 0 && block_size > 0, "zero head count or block size");
     XL_REQUIRE(head_dim % 8 == 0 && head_dim > 0, "head_dim must be a multiple of 8");
@@ -394,6 +397,9 @@ extern "C" int xlite_hip_gather_sparse_kv_cache(void *stream, const void *k_cach
 {
     XL_REQUIRE(kv_heads == 1, "kvHeads should be less than or equal to 1");
     XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype unsupported!");
+    if (batch == 0 || index_topk == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(k_cache && pe_cache && block_tables && topk_indices && query_lens && cached_lens &&
                    k_dense && pe_dense,
                "null tensor");
@@ -418,6 +424,9 @@ extern "C" int xlite_hip_rope_complex(void *stream, uint32_t num_tokens, uint32_
                                       int dtype)
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype TODO");
+    if (num_tokens == 0 || n_local_heads == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(input && freqs && position && output, "null tensor");
     XL_REQUIRE(rope_dim % 2 == 0 && rope_dim > 0 && rope_dim <= step_dim, "bad rope_dim");
     XL_REQUIRE(step_dim % 2 == 0, "step_dim must be even");
@@ -450,6 +459,9 @@ extern "C" int xlite_hip_mla_prepare(void *stream, void *attn_qkvc, const void *
                                      int dtype)
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype unsupported!");
+    if (num_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(attn_qkvc && q_norm && q_norm_bias && attn_norm_qc && kv_norm && kv_norm_bias &&
                    attn_norm_kvc && freqs && position,
                "null tensor");
@@ -485,6 +497,9 @@ extern "C" int xlite_hip_quantize_kv_int8(void *stream, const void *src, int8_t 
                                           uint64_t rows, uint32_t head_dim, int dtype)
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype unsupported!");
+    if (rows == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(src && dst && scales, "null tensor");
     XL_REQUIRE(head_dim > 0, "head_dim must be positive");
     if (rows == 0) {

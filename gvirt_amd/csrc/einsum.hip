@@ -97,6 +97,9 @@ extern "C" int xlite_hip_einsum_mht_mhd(void *stream, const void *mht, const voi
                                         uint32_t t_stride, int w_is_hdt, int dtype)
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "mht/w/mhd dtype unsupported!");
+    if (m == 0 || h == 0) {
+        return XLITE_HIP_OK;
+    }
     XL_REQUIRE(mht && w && mhd, "null tensor");
     XL_REQUIRE(t % 16 == 0 && t > 0, "t must be a positive multiple of 16");
     XL_REQUIRE(d % 32 == 0 && d > 0, "d must be a positive multiple of 32");
