@@ -23,6 +23,11 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
     }
     const uint32_t max_ctx = max_num_block * block_size;
     if (is_decode_batch(total_tokens, batch)) {
+        if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
+            uint32_t tile, n_sub, max_slots;
+            decode_mfma_plan(batch, n_kv_heads, block_size, max_num_block, &tile, &n_sub, &max_slots);
+            return decode_mfma_workspace_bytes(total_tokens, n_heads, head_dim, max_slots);
+        }
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
         const uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);
@@ -65,6 +70,10 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
     hipStream_t s = as_stream(stream);
     if (is_decode_batch(total_tokens, batch)) {
         XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");
+        if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
+            return launch_decode_mfma(s, a);
+        }
+        // block sizes that are not a multiple of 32, or more than 16 query heads per kv head
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
         uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);

@@ -52,6 +52,14 @@ size_t decode_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t 
                               uint32_t max_tiles);
 int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_tokens);
 
+// decode_mfma.hip
+bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
+                           uint32_t total_tokens);
+void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, uint32_t max_num_block,
+                      uint32_t *tile_tokens, uint32_t *n_sub, uint32_t *max_slots);
+size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim, uint32_t max_slots);
+int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
+
 // mfma_attention.hip
 bool mfma_gqa_supported(uint32_t head_dim);
 size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits);
