@@ -106,8 +106,7 @@ class Runtime:
         if self._pool is None or self._pool.numel() < nbytes:
             if self._pool is not None:
                 torch.cuda.synchronize(self.device)
-            # zero-filled: the first 64 KiB are ticket counters that every call leaves at zero
-            self._pool = torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
+            self._pool = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
 
     def workspace(self, nbytes: int) -> torch.Tensor:
         self._grow(nbytes)

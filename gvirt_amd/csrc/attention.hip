@@ -19,7 +19,7 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
                                                       uint32_t max_num_block)
 {
     if (total_tokens == 0 || batch == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || head_dim < 8) {
-        return XLITE_HIP_WS_COUNTER_BYTES;
+        return 0;
     }
     const uint32_t max_ctx = max_num_block * block_size;
     if (is_decode_batch(total_tokens, batch)) {
@@ -31,8 +31,7 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
         const uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);
-        return XLITE_HIP_WS_COUNTER_BYTES +
-               decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile));
+        return decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile));
     }
     const uint32_t splits =
         mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx, 64);
@@ -81,7 +80,7 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         const uint32_t max_ctx = max_num_block * block_size;
         while (ceil_div(max_ctx, tile) > 1 &&
                (workspace == nullptr ||
-                XLITE_HIP_WS_COUNTER_BYTES + decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile)) > workspace_bytes)) {
+                decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile)) > workspace_bytes)) {
             tile *= 2;
         }
         int rc = launch_decode(s, a, tile);

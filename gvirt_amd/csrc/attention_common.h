@@ -42,6 +42,20 @@ struct MlaArgs {
     size_t workspace_bytes;
 };
 
+// merge.hip: scratch for split-KV partial results and their merge.
+// Layout of the workspace: cnt[rows * n_heads] int32 (number of partials of a (row, head); 0 = the
+// producer stored the final value itself), then acc[rows * n_heads][max_slots][dv] and
+// ml[rows * n_heads][max_slots][2] (running maximum in the log2 domain, sum) in fp32.
+struct PartialBuffers {
+    int32_t *cnt;
+    float *acc;
+    float *ml;
+};
+size_t partial_bytes(uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots);
+PartialBuffers carve_partials(void *workspace, uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots);
+int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
+                 uint32_t n_heads, uint32_t dv, uint32_t max_slots);
+
 // decode_attention.hip
 bool decode_supported(uint32_t head_dim);
 void decode_geometry(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t *g_kernel,

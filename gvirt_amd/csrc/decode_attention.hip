@@ -8,8 +8,8 @@
 // heads that share the kv head. Dot products use v_dot2 (two 16-bit products + fp32 add per
 // instruction): K against the packed query, and V against packed probabilities of two
 // consecutive rows. Rows of different lane groups are merged through LDS at the end of the
-// tile; tiles of one query row are merged by the last workgroup to finish (ticket counter),
-// from fp32 partials in the workspace.
+// tile; tiles of one query row leave fp32 partials in the workspace, merged by a second small
+// kernel (merge.hip).
 //
 // Replaces attention.h / flash_attention.h of the reference for batches in which every
 // sequence contributes one query row (xlite/csrc/kernels/flash_attention.h:323-628).
@@ -67,7 +67,7 @@ struct DecodeParams {
     const int32_t *lens;
     const int32_t *cached_lens;
     const int32_t *block_tables;
-    int32_t *counters;
+    int32_t *part_cnt;          // [token][head] number of partial tiles (0: final value stored directly)
     float *part_acc;            // [token][head][tile][D]
     float *part_ml;             // [token][head][tile][2]
     uint32_t q_row_stride;      // elements between query rows
@@ -327,96 +327,36 @@ decode_kernel(const DecodeParams p)
             __syncthreads();
         }
 
-        // ---- phase-0 groups own the tile result ------------------------------------------------
-        if (n_tiles == 1) {
-            if (phase == 0) {
+        // ---- phase-0 groups own the tile result: final value, or a partial for the merge kernel -------
+        if (phase == 0) {
 #pragma unroll
-                for (int h = 0; h < G; h++) {
-                    if (static_cast<uint32_t>(h) < g_valid) {
+            for (int h = 0; h < G; h++) {
+                if (static_cast<uint32_t>(h) < g_valid) {
+                    const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head0 + h;
+                    if (n_tiles == 1) {
                         const float inv = l[h] > 0.f ? 1.0f / l[h] : 0.f;
                         uint4 o;
                         o.x = T::pack(acc[h][0] * inv, acc[h][1] * inv);
                         o.y = T::pack(acc[h][2] * inv, acc[h][3] * inv);
                         o.z = T::pack(acc[h][4] * inv, acc[h][5] * inv);
                         o.w = T::pack(acc[h][6] * inv, acc[h][7] * inv);
-                        *reinterpret_cast<uint4 *>(p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + h) * D + sub * 8) = o;
+                        *reinterpret_cast<uint4 *>(p.out + rh * D + sub * 8) = o;
+                    } else {
+                        const uint64_t slot = rh * p.max_tiles + tile;
+                        float4 *dst = reinterpret_cast<float4 *>(p.part_acc + slot * D + sub * 8);
+                        dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+                        dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
+                        if (sub == 0) {
+                            *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m[h], l[h]);
+                        }
                     }
-                }
-            }
-            continue;
-        }
-
-        if (phase == 0) {
-#pragma unroll
-            for (int h = 0; h < G; h++) {
-                if (static_cast<uint32_t>(h) < g_valid) {
-                    const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head0 + h) * p.max_tiles + tile;
-                    float4 *dst = reinterpret_cast<float4 *>(p.part_acc + slot * D + sub * 8);
-                    dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-                    dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
-                    if (sub == 0) {
-                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m[h], l[h]);
+                    if (sub == 0 && tile == 0 && p.part_cnt != nullptr) {
+                        p.part_cnt[rh] = n_tiles == 1 ? 0 : static_cast<int32_t>(n_tiles);
                     }
                 }
             }
         }
-        // publish, then take a ticket; the last tile of the row merges all of them
-        __threadfence();
-        __syncthreads();
-        int32_t *ticket_flag = reinterpret_cast<int32_t *>(smem);
-        int32_t *counter = p.counters + static_cast<uint64_t>(tok) * gridDim.z + blockIdx.z;
-        if (threadIdx.x == 0) {
-            *ticket_flag = atomicAdd(counter, 1);
-        }
-        __syncthreads();
-        const bool last = *ticket_flag == static_cast<int32_t>(n_tiles) - 1;
-        __syncthreads();  // everyone has read the flag before smem is reused
-        if (!last) {
-            continue;
-        }
-        __threadfence();  // acquire the partials of the other tiles
-
-        // (head, 8-column chunk) items of this workgroup's heads, merged over all tiles in order
-        const uint32_t heads_wg = p.nkv_wg * g_valid;
-        const uint32_t items = heads_wg * LPR;
-        for (uint32_t it = threadIdx.x; it < items; it += NW * 64) {
-            const uint32_t hl = it / LPR, c = it % LPR;
-            const uint32_t head = (zkv * p.nkv_wg + hl / g_valid) * p.group + hchunk * G + hl % g_valid;
-            const uint64_t base = (static_cast<uint64_t>(tok) * p.n_heads + head) * p.max_tiles;
-            float mm = -INFINITY;
-            for (uint32_t t = 0; t < n_tiles; t++) {
-                mm = fmaxf(mm, p.part_ml[(base + t) * 2]);
-            }
-            const float m_safe = mm == -INFINITY ? 0.f : mm;
-            float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            float lsum = 0.f;
-            for (uint32_t t = 0; t < n_tiles; t++) {
-                const float2 ml = *reinterpret_cast<const float2 *>(p.part_ml + (base + t) * 2);
-                const float w = fast_exp2(ml.x - m_safe);
-                lsum += ml.y * w;
-                const float4 *src = reinterpret_cast<const float4 *>(p.part_acc + (base + t) * D + c * 8);
-                const float4 x0 = src[0], x1 = src[1];
-                o[0] += x0.x * w;
-                o[1] += x0.y * w;
-                o[2] += x0.z * w;
-                o[3] += x0.w * w;
-                o[4] += x1.x * w;
-                o[5] += x1.y * w;
-                o[6] += x1.z * w;
-                o[7] += x1.w * w;
-            }
-            const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-            uint4 ov;
-            ov.x = T::pack(o[0] * inv, o[1] * inv);
-            ov.y = T::pack(o[2] * inv, o[3] * inv);
-            ov.z = T::pack(o[4] * inv, o[5] * inv);
-            ov.w = T::pack(o[6] * inv, o[7] * inv);
-            *reinterpret_cast<uint4 *>(p.out + (static_cast<uint64_t>(tok) * p.n_heads + head) * D + c * 8) = ov;
-        }
-        if (threadIdx.x == 0) {
-            *counter = 0;  // leave the workspace ready for the next call
-        }
-        __syncthreads();
+        __syncthreads();  // the LDS tree buffers are reused by the next query row
     }
 }
 
@@ -491,8 +431,7 @@ void decode_geometry(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, u
 size_t decode_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim,
                               uint32_t max_tiles)
 {
-    const size_t slots = static_cast<size_t>(total_tokens) * n_heads * max_tiles;
-    return slots * (head_dim + 2) * sizeof(float);
+    return max_tiles > 1 ? partial_bytes(total_tokens, n_heads, head_dim, max_tiles) : 0;
 }
 
 int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_tokens)
@@ -501,17 +440,13 @@ int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_toke
     decode_geometry(a.n_heads, a.n_kv_heads, a.head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
     const uint32_t max_ctx = a.max_num_block * a.block_size;
     const uint32_t max_tiles = ceil_div(max_ctx, tile_tokens);
-
-    const size_t counters_needed = static_cast<size_t>(a.total_tokens) * zdim * sizeof(int32_t);
-    if (counters_needed > XLITE_HIP_WS_COUNTER_BYTES) {
-        return fail(XLITE_HIP_EINVAL, __func__, "too many (token, head group) pairs for the ticket counters");
-    }
-    const size_t need = XLITE_HIP_WS_COUNTER_BYTES +
-                        decode_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, max_tiles);
+    const size_t need = decode_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, max_tiles);
     if (max_tiles > 1 && (a.workspace == nullptr || a.workspace_bytes < need)) {
         return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
                                                     " bytes, have " + std::to_string(a.workspace_bytes));
     }
+    const PartialBuffers pb = max_tiles > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_tiles)
+                                            : PartialBuffers{};
 
     DecodeParams p;
     p.q = static_cast<const uint16_t *>(a.qkv);
@@ -524,10 +459,9 @@ int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_toke
     p.lens = a.lens;
     p.cached_lens = a.cached_lens;
     p.block_tables = a.block_tables;
-    char *ws = static_cast<char *>(a.workspace);
-    p.counters = reinterpret_cast<int32_t *>(ws);
-    p.part_acc = reinterpret_cast<float *>(ws + XLITE_HIP_WS_COUNTER_BYTES);
-    p.part_ml = p.part_acc + static_cast<size_t>(a.total_tokens) * a.n_heads * max_tiles * a.head_dim;
+    p.part_cnt = pb.cnt;
+    p.part_acc = pb.acc;
+    p.part_ml = pb.ml;
     p.q_row_stride = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
     p.n_heads = a.n_heads;
     p.n_kv_heads = a.n_kv_heads;
@@ -543,20 +477,27 @@ int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_toke
     const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
     const bool bf = a.dtype == XLITE_HIP_BF16;
     const uint32_t g = g_kernel;
+    int rc;
     if (a.head_dim == 128) {
         if (bf) {
-            return kv8 ? launch_decode_d<BF16, 128, true>(stream, p, a.batch, zdim, g)
-                       : launch_decode_d<BF16, 128, false>(stream, p, a.batch, zdim, g);
+            rc = kv8 ? launch_decode_d<BF16, 128, true>(stream, p, a.batch, zdim, g)
+                     : launch_decode_d<BF16, 128, false>(stream, p, a.batch, zdim, g);
+        } else {
+            rc = kv8 ? launch_decode_d<FP16, 128, true>(stream, p, a.batch, zdim, g)
+                     : launch_decode_d<FP16, 128, false>(stream, p, a.batch, zdim, g);
         }
-        return kv8 ? launch_decode_d<FP16, 128, true>(stream, p, a.batch, zdim, g)
-                   : launch_decode_d<FP16, 128, false>(stream, p, a.batch, zdim, g);
+    } else if (bf) {
+        rc = kv8 ? launch_decode_d<BF16, 64, true>(stream, p, a.batch, zdim, g)
+                 : launch_decode_d<BF16, 64, false>(stream, p, a.batch, zdim, g);
+    } else {
+        rc = kv8 ? launch_decode_d<FP16, 64, true>(stream, p, a.batch, zdim, g)
+                 : launch_decode_d<FP16, 64, false>(stream, p, a.batch, zdim, g);
     }
-    if (bf) {
-        return kv8 ? launch_decode_d<BF16, 64, true>(stream, p, a.batch, zdim, g)
-                   : launch_decode_d<BF16, 64, false>(stream, p, a.batch, zdim, g);
+    if (rc != XLITE_HIP_OK || max_tiles == 1) {
+        return rc;
     }
-    return kv8 ? launch_decode_d<FP16, 64, true>(stream, p, a.batch, zdim, g)
-               : launch_decode_d<FP16, 64, false>(stream, p, a.batch, zdim, g);
+    XL_LAUNCH_CHECK();
+    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, max_tiles);
 }
 
 }  // namespace xlite

@@ -1,22 +1,23 @@
 // GQA flash-decode on the matrix cores, split along the KV axis.
 //
-// Workgroup = 8 wavefronts = one (sequence, KV tile). Every wave streams the positions of its KV
-// range for ONE kv head (waves loop over kv heads when there are more than 8; when there are fewer,
-// the spare waves take sub-ranges of the tile) and never synchronises with the other waves while
-// streaming:
-//   global -> registers : 1 KiB of consecutive cache bytes per wave-wide load, 16 bytes per lane
-//   registers -> LDS    : rows stored 16-bit, row major, 16-byte chunks XOR-swizzled so that both
-//                         read patterns below are bank-conflict free
+// Workgroup = 8 wavefronts = one (sequence, KV tile). The tile is walked in steps of 16 positions.
+// All 512 threads fetch a step's cache bytes in address order (HBM streams best when every
+// wave-wide load covers 1 KiB of consecutive memory; 256-byte rows at a 2 KiB stride reach only
+// ~60 % of that), then every wave computes ONE kv head of the step (passes over groups of 8 kv
+// heads when there are more; when there are fewer, the spare waves take sub ranges of the tile):
+//   global -> registers : 16 bytes per lane; two steps are always in flight (a single batch per
+//                         wave leaves HBM idle for one round trip between batches)
+//   registers -> LDS    : two stages (one barrier per step); rows stored 16-bit, row major, 16-byte
+//                         chunks XOR-swizzled so that both read patterns below are conflict free
 //   S^T[token][head]  = K . Q^T    v_mfma_f32_16x16x32 (A = K rows via ds_read_b128, B = Q regs)
-//   O^T[d][head]     += V^T . P^T  v_mfma_f32_16x16x32 (A = V^T via ds_read_b64_tr_b16, B = P regs)
+//   O^T[d][head]     += V^T . P^T  v_mfma_f32_16x16x16 (A = V^T via ds_read_b64_tr_b16, B = P regs)
 // The query heads that share the kv head are the 16 MFMA columns (unused columns carry zeros), so
-// one lane column owns one head: the online softmax needs two cross-lane exchanges per 32
-// positions, and P leaves the first product in the register layout the second one consumes.
+// one lane column owns one head: the online softmax needs two cross-lane exchanges per step, and P leaves the first product in the register layout the second one consumes.
 // int8 caches are widened to 16 bit (exactly) on their way into LDS; their per-position scales are
 // applied to the scores (K) and to the probabilities (V).
 //
-// Each wave leaves an fp32 partial (max, sum, O) per query head in the workspace; the last
-// workgroup of a query row to finish (ticket counter) merges all partials of the row.
+// Each wave leaves an fp32 partial (max, sum, O) per query head in the workspace; a small second
+// kernel merges the partials of every query row (merge.hip).
 //
 // Replaces the split-KV path of the reference (xlite/csrc/kernels/flash_attention.h:323-628) for
 // batches in which every sequence contributes one query row.
@@ -28,7 +29,7 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kWaves = 8;
-constexpr int kStep = 32;  // positions per inner step (one k=32 PV product)
+constexpr int kStep = 16;  // positions per inner step
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 
@@ -41,6 +42,11 @@ struct Mfma16<BF16> {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                        __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
+    // k = 16: four 16-bit elements per lane
+    static __device__ __forceinline__ f32x4_t run16(const s16x4_t &a, const uint2 &b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    }
 };
 template <>
 struct Mfma16<FP16> {
@@ -48,6 +54,12 @@ struct Mfma16<FP16> {
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
                                                       __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t run16(const s16x4_t &a, const uint2 &b, f32x4_t c)
+    {
+        typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 f16x4_t;
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+                                                     __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
     }
 };
 
@@ -62,7 +74,7 @@ struct DecodeMfmaParams {
     const int32_t *lens;
     const int32_t *cached_lens;
     const int32_t *block_tables;
-    int32_t *counters;
+    int32_t *part_cnt; // [token][head] number of partial slots (0: final value stored directly)
     float *part_acc;   // [token][head][slot][D]
     float *part_ml;    // [token][head][slot][2]
     uint32_t q_row_stride;
@@ -93,18 +105,30 @@ __device__ __forceinline__ uint4 widen(const uint2 &raw)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-template <typename T, int D, bool KV8>
+// XOR pattern applied to the 16-byte chunk index of LDS row `row`. One pattern serves both read
+// shapes: 16 lanes reading the same chunk of 16 consecutive rows (K as MFMA A operand) land in 16
+// different chunk slots, and 8 consecutive rows read as 32-byte pieces (transposing V read) land
+// in 8 different 32-byte slots of the 256-byte bank window.
+template <int D>
+__device__ __forceinline__ uint32_t swizzle(uint32_t row)
+{
+    constexpr uint32_t CH = D / 8, R256 = 256 / (D * 2);
+    const uint32_t rr = row / R256;
+    return ((rr & (CH / 2 - 1)) << 1) | ((rr / (CH / 2)) & 1);
+}
+
+template <typename T, int D, bool KV8, bool MULTI_SUB>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_mfma_kernel(const DecodeMfmaParams p)
 {
     constexpr int CH = D / 8;            // 16-byte chunks per LDS row
     constexpr int ROWB = D * 2;          // LDS bytes per row
-    constexpr int R256 = 256 / ROWB;     // rows per 256-byte bank window (1 or 2)
-    constexpr int RPI = 64 / CH;         // cache rows fetched by one wave-wide load
-    constexpr int NLD = kStep / RPI;     // loads per tile and tensor
     constexpr int KS = D / 32;           // k-steps of the QK product
     constexpr int MT = D / 16;           // 16-row tiles of O^T
     constexpr int TILE_BYTES = kStep * ROWB;
+    constexpr int NT = kWaves * 64;
+    constexpr int NV = kWaves * kStep * CH / NT;  // 16-byte vectors per thread, step and tensor
+    constexpr int STAGE_BYTES = kWaves * 2 * TILE_BYTES;
     typedef typename std::conditional<KV8, uint2, uint4>::type gvec_t;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -113,28 +137,23 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t tile = blockIdx.x;
     const uint32_t seq = blockIdx.y;
-    unsigned char *k_lds = smem + wave * 2 * TILE_BYTES;
-    unsigned char *v_lds = k_lds + TILE_BYTES;
+    // LDS: two stages; in a stage one region per (kv head, sub range) pair of the pass = per
+    // computing wave, K tile then V tile. int8 caches: behind the stages, the scales of the two
+    // stages [stage][K | V][region][16 positions]
+    const uint32_t my_lds = wave * 2 * TILE_BYTES;
+    float *sc_lds = reinterpret_cast<float *>(smem + 2 * STAGE_BYTES);
+    // block-table entries of the tile, copied once per query row: a lookup inside the streaming
+    // loop must not be a vector memory load, whose completion can only be awaited together with
+    // every cache load issued before it (that would drain the prefetch pipeline at every step)
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE_BYTES + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0));
 
-    // ---- lane roles ------------------------------------------------------------------------------
+    // ---- compute roles -------------------------------------------------------------------------------
     const uint32_t col = lane & 15;       // MFMA column = query head inside the group
     const uint32_t jq = lane >> 4;        // 16-lane group
-    // loader: row lr (+ RPI per load), 16-byte chunk lc
-    const uint32_t lr = lane / CH, lc = lane % CH;
-
-    // LDS write offsets of the loader (K and V swizzles differ), one per load of the tile
-    uint32_t kw_off[NLD], vw_off[NLD];
-#pragma unroll
-    for (int i = 0; i < NLD; i++) {
-        const uint32_t row = i * RPI + lr;
-        kw_off[i] = row * ROWB + ((lc ^ ((row / R256) % CH)) << 4);
-        vw_off[i] = row * ROWB + ((lc ^ (2 * ((row / R256) % (CH / 2)))) << 4);
-    }
-    // LDS read offsets: K rows as the A operand of the QK product (sub tile 1 is +16 rows)
-    uint32_t kr_off[KS];
+    uint32_t kr_off[KS];                  // K rows as the A operand of the QK product
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-        kr_off[ks] = col * ROWB + (((4 * ks + jq) ^ ((col / R256) % CH)) << 4);
+        kr_off[ks] = my_lds + col * ROWB + (((4 * ks + jq) ^ swizzle<D>(col)) << 4);
     }
     // V^T through the transposing read: inside a 16-lane group lane 4*j' + q points at the four
     // elements [16*mt + 4q, +4) of position 4*jq + j'; it receives positions 4*jq .. 4*jq + 3 of
@@ -145,10 +164,33 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         const uint32_t q4 = lane & 3;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            const uint32_t chunk = 2 * mt + (q4 >> 1);
-            vr_off[mt] = pos * ROWB + ((chunk ^ (2 * ((pos / R256) % (CH / 2)))) << 4) + ((q4 & 1) << 3);
+            vr_off[mt] = my_lds + TILE_BYTES + pos * ROWB + (((2 * mt + (q4 >> 1)) ^ swizzle<D>(pos)) << 4) + ((q4 & 1) << 3);
         }
     }
+
+    // ---- loader roles: the 512 threads fetch the step's cache bytes in address order, so that every
+    // wave-wide load covers 1 KiB of consecutive memory. Vector v = tid + 512 i of a step:
+    // chunk = v % CH, kv head (inside the pass) = (v / CH) % KVW, position = (v / (CH KVW)) % 16,
+    // sub range = v / (CH KVW 16). KVW = kv heads per pass (a power of two), KVW * n_sub = 8.
+    const uint32_t kvw = kWaves / p.n_sub;
+    const uint32_t kvw_shift = __builtin_ctz(kvw);
+    const uint32_t lc = threadIdx.x % CH;
+    auto vec_kvl = [&](int i) { return ((threadIdx.x + NT * i) / CH) & (kvw - 1); };
+    auto vec_pos = [&](int i) { return ((threadIdx.x + NT * i) / CH >> kvw_shift) & (kStep - 1); };
+    auto vec_sub = [&](int i) { return MULTI_SUB ? ((threadIdx.x + NT * i) / (CH * kStep)) >> kvw_shift : 0u; };
+    uint32_t w_off[NV];   // LDS offset of the K vector; its V twin sits TILE_BYTES further
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const uint32_t region = vec_sub(i) * kvw + vec_kvl(i);   // the wave that consumes this vector
+        w_off[i] = region * 2 * TILE_BYTES + vec_pos(i) * ROWB + ((lc ^ swizzle<D>(vec_pos(i))) << 4);
+    }
+    // scale loader (int8 caches): threads 0..127 fetch the K scales of the step, 128..255 the V scales
+    const uint32_t sj = threadIdx.x & 127;
+    const bool s_active = KV8 && threadIdx.x < 256;
+    const uint32_t s_kvl = sj & (kvw - 1), s_pos = (sj >> kvw_shift) & (kStep - 1);
+    const uint32_t s_sub = MULTI_SUB ? sj >> (kvw_shift + 4) : 0u;
+    const float *s_src = threadIdx.x < 128 ? p.k_scale : p.v_scale;
+    const uint32_t s_dst = (threadIdx.x < 128 ? 0 : kWaves * kStep) + (s_sub * kvw + s_kvl) * kStep + s_pos;
 
     const int32_t qlen = p.lens[seq];
     const int32_t clen = p.cached_lens[seq];
@@ -156,9 +198,9 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const gvec_t *kc = static_cast<const gvec_t *>(p.k_cache);
     const gvec_t *vc = static_cast<const gvec_t *>(p.v_cache);
-    const uint32_t row_vecs = static_cast<uint32_t>(CH);  // gvec_t per (position, kv head) row
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t sub_len = p.tile_tokens / p.n_sub;
+    const uint32_t my_kvl = wave & (kvw - 1), my_sub = wave >> kvw_shift;
 
     for (int32_t r = 0; r < qlen; r++) {
         const uint32_t tok = static_cast<uint32_t>(qstart + r);
@@ -170,13 +212,23 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         const uint32_t t0 = tile * p.tile_tokens;
         const uint32_t t1 = min(limit, t0 + p.tile_tokens);
         const bool single = n_tiles == 1 && p.n_sub == 1;
+        // every sub range runs the same number of steps (the first one is never shorter than the others)
+        const uint32_t n_steps = ceil_div(min(t1 - t0, sub_len), kStep);
+        const uint32_t ta = min(t1, t0 + my_sub * sub_len);   // this wave's range
+        const uint32_t tb = min(t1, ta + sub_len);
+        const uint32_t blk0 = t0 / p.block_size;
+        {
+            const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
+            for (uint32_t i = threadIdx.x; i < nblk; i += NT) {
+                tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
+            }
+            __syncthreads();
+        }
 
-        // (kv head, sub range) passes of this wave
-        for (uint32_t pass = wave; pass < p.n_kv_heads * p.n_sub; pass += kWaves) {
-            const uint32_t kvh = pass % p.n_kv_heads;
-            const uint32_t sub = pass / p.n_kv_heads;
-            const uint32_t ta = min(t1, t0 + sub * sub_len);
-            const uint32_t tb = min(t1, ta + sub_len);
+        // passes over groups of `kvw` kv heads
+        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += kvw) {
+            const uint32_t kvh = kv0 + my_kvl;
+            const bool kv_ok = kvh < p.n_kv_heads;
             const uint32_t head0 = kvh * p.group;
 
             // ---- Q^T as the B operand: column = head, 8 consecutive elements per k group ----------
@@ -185,8 +237,15 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride + static_cast<uint64_t>(head0 + col) * D;
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8)
-                                             : make_uint4(0, 0, 0, 0);
+                    qreg[ks] = (kv_ok && col < g_valid) ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8)
+                                                        : make_uint4(0, 0, 0, 0);
+                }
+                // Consume the query registers here, before any cache load is issued: their first real
+                // use is inside the streaming loop, where waiting for them would mean waiting for
+                // every prefetched cache load issued since (memory loads complete in order).
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
                 }
             }
             f32x4_t O[MT];
@@ -196,98 +255,143 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             }
             float m_run = -INFINITY, l_run = 0.f;
 
-            // ---- stream [ta, tb) in steps of 32 positions; ta is a multiple of 32 -------------------
-            gvec_t kreg[NLD], vreg[NLD];
-            float ksc[2][4], vsc[2][4];
-            // all 32 positions of a step lie in one block (block_size is a multiple of 32); the block
-            // index and the offset inside it advance with the steps, no division in the loop
-            uint32_t nxt_blk = ta / p.block_size, nxt_off = ta % p.block_size;
-            auto issue = [&]() {
-                const uint64_t phys = static_cast<uint32_t>(table[nxt_blk]);
-                const uint64_t row0 = (phys * p.block_size + nxt_off) * p.n_kv_heads + kvh;
+            // byte offset of this thread's i-th vector from the first cache row of its sub range's
+            // step; kv heads past the last one (a pass may be ragged) re-read the last head.
+            // Positions at or beyond the end of a range (last step only) re-read the last valid
+            // position instead: their probabilities are forced to zero, and a finite value times
+            // zero cannot poison the products the way stale cache bytes (NaN) could.
+            constexpr uint32_t VB = sizeof(gvec_t);
+            const uint32_t row_bytes = p.n_kv_heads * CH * VB;
+            uint32_t g_off[NV];
 #pragma unroll
-                for (int i = 0; i < NLD; i++) {
-                    const uint64_t row = row0 + static_cast<uint64_t>(i * RPI + lr) * p.n_kv_heads;
-                    kreg[i] = kc[row * row_vecs + lc];
-                    vreg[i] = vc[row * row_vecs + lc];
-                }
-                if constexpr (KV8) {
-                    // scales of the positions this lane will hold after the QK product
+            for (int i = 0; i < NV; i++) {
+                g_off[i] = vec_pos(i) * row_bytes + (min(kv0 + vec_kvl(i), p.n_kv_heads - 1) * CH + lc) * VB;
+            }
+            const uint32_t s_off = s_pos * p.n_kv_heads + min(kv0 + s_kvl, p.n_kv_heads - 1);
+
+            // two register sets: two steps are in flight at any time, so that the memory system always
+            // has queued work when a step's data has arrived
+            gvec_t kreg[2][NV], vreg[2][NV];
+            float sreg[2] = {0.f, 0.f};
+            // first position of a step of sub range `sub`: its 16 positions share one block
+            // (block_size % 16 == 0 and every range starts at a multiple of 16)
+            auto step_start = [&](uint32_t sub, uint32_t step) -> uint32_t {
+                const uint32_t t = t0 + sub * sub_len + step * kStep;
+                return t < t1 ? t : t0;   // exhausted sub range: any valid rows, nobody consumes them
+            };
+            auto row_of = [&](uint32_t t) -> uint64_t {
+                const uint32_t blk = t / p.block_size, off = t % p.block_size;
+                return (static_cast<uint64_t>(tbl_lds[blk - blk0]) * p.block_size + off) * p.n_kv_heads;
+            };
+            auto sub_end = [&](uint32_t sub) { return min(t1, t0 + (sub + 1) * sub_len); };
+            auto issue = [&](uint32_t step, auto slot_tag) {
+                constexpr int SL = decltype(slot_tag)::value;
+                const bool last_step = step + 1 == n_steps;
+                if constexpr (!MULTI_SUB) {
+                    const uint32_t ts = step_start(0, step);
+                    const uint64_t row0 = row_of(ts);   // uniform: scalar address arithmetic
+                    const char *kb = reinterpret_cast<const char *>(kc) + row0 * CH * VB;
+                    const char *vb = reinterpret_cast<const char *>(vc) + row0 * CH * VB;
+                    if (!last_step) {
 #pragma unroll
-                    for (int s = 0; s < 2; s++) {
+                        for (int i = 0; i < NV; i++) {
+                            kreg[SL][i] = *reinterpret_cast<const gvec_t *>(kb + g_off[i]);
+                            vreg[SL][i] = *reinterpret_cast<const gvec_t *>(vb + g_off[i]);
+                        }
+                        if constexpr (KV8) {
+                            if (s_active) {
+                                sreg[SL] = s_src[row0 + s_off];
+                            }
+                        }
+                    } else {
+                        const uint32_t last_pos = t1 - 1 - ts;   // >= 0: the first range is never empty
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const uint64_t row = row0 + static_cast<uint64_t>(16 * s + 4 * jq + e) * p.n_kv_heads;
-                            ksc[s][e] = p.k_scale[row];
-                            vsc[s][e] = p.v_scale[row];
+                        for (int i = 0; i < NV; i++) {
+                            const uint32_t back = vec_pos(i) > last_pos ? (vec_pos(i) - last_pos) * row_bytes : 0u;
+                            kreg[SL][i] = *reinterpret_cast<const gvec_t *>(kb + (g_off[i] - back));
+                            vreg[SL][i] = *reinterpret_cast<const gvec_t *>(vb + (g_off[i] - back));
+                        }
+                        if constexpr (KV8) {
+                            if (s_active) {
+                                const uint32_t back = s_pos > last_pos ? (s_pos - last_pos) * p.n_kv_heads : 0u;
+                                sreg[SL] = s_src[row0 + s_off - back];
+                            }
                         }
                     }
-                }
-                nxt_off += kStep;
-                if (nxt_off >= p.block_size) {
-                    nxt_off = 0;
-                    nxt_blk++;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NV; i++) {
+                        const uint32_t ts = step_start(vec_sub(i), step);
+                        const uint32_t end = max(sub_end(vec_sub(i)), ts + 1);
+                        const uint32_t last_pos = min(end - 1 - ts, static_cast<uint32_t>(kStep - 1));
+                        const uint32_t back = vec_pos(i) > last_pos ? (vec_pos(i) - last_pos) * row_bytes : 0u;
+                        const uint64_t row0 = row_of(ts);
+                        kreg[SL][i] = *reinterpret_cast<const gvec_t *>(reinterpret_cast<const char *>(kc) + row0 * CH * VB + (g_off[i] - back));
+                        vreg[SL][i] = *reinterpret_cast<const gvec_t *>(reinterpret_cast<const char *>(vc) + row0 * CH * VB + (g_off[i] - back));
+                    }
+                    if constexpr (KV8) {
+                        if (s_active) {
+                            const uint32_t ts = step_start(s_sub, step);
+                            const uint32_t end = max(sub_end(s_sub), ts + 1);
+                            const uint32_t last_pos = min(end - 1 - ts, static_cast<uint32_t>(kStep - 1));
+                            const uint32_t back = s_pos > last_pos ? (s_pos - last_pos) * p.n_kv_heads : 0u;
+                            sreg[SL] = s_src[row_of(ts) + s_off - back];
+                        }
+                    }
                 }
             };
-
-            if (ta < tb) {
-                issue();
-            }
-            for (uint32_t t = ta; t < tb; t += kStep) {
-                // ---- registers -> LDS (rows beyond the end of the range become zeros) ----------------
-                const bool partial = t + kStep > tb;
+            // registers of set SL -> LDS stage SL (step s uses set and stage s % 2)
+            auto stage_write = [&](auto slot_tag) {
+                constexpr int SL = decltype(slot_tag)::value;
 #pragma unroll
-                for (int i = 0; i < NLD; i++) {
-                    uint4 kv = widen<T>(kreg[i]);
-                    uint4 vv = widen<T>(vreg[i]);
-                    if (partial && t + i * RPI + lr >= tb) {
-                        kv = make_uint4(0, 0, 0, 0);
-                        vv = make_uint4(0, 0, 0, 0);
-                    }
-                    *reinterpret_cast<uint4 *>(k_lds + kw_off[i]) = kv;
-                    *reinterpret_cast<uint4 *>(v_lds + vw_off[i]) = vv;
+                for (int i = 0; i < NV; i++) {
+                    *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i]) = widen<T>(kreg[SL][i]);
+                    *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i] + TILE_BYTES) = widen<T>(vreg[SL][i]);
                 }
-                float kscale[2][4], vscale[2][4];
                 if constexpr (KV8) {
-#pragma unroll
-                    for (int s = 0; s < 2; s++) {
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            kscale[s][e] = ksc[s][e];
-                            vscale[s][e] = vsc[s][e];
-                        }
+                    if (s_active) {
+                        sc_lds[SL * 2 * kWaves * kStep + s_dst] = sreg[SL];
                     }
                 }
-                if (t + kStep < tb) {
-                    issue();
+            };
+            auto compute = [&](uint32_t step, auto slot_tag) {
+                constexpr int SL = decltype(slot_tag)::value;
+                const uint32_t t = ta + step * kStep;
+                if (t >= tb) {
+                    return;
                 }
-
-                // ---- S^T = K . Q^T for the two 16-position sub tiles ----------------------------------
-                f32x4_t S[2];
+                const unsigned char *stage = smem + SL * STAGE_BYTES;
+                // ---- S^T = K . Q^T: 16 positions x 16 heads ---------------------------------------------------
+                f32x4_t S = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
-                    S[s] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int ks = 0; ks < KS; ks++) {
-                        const uint4 a = *reinterpret_cast<const uint4 *>(k_lds + kr_off[ks] + s * 16 * ROWB);
-                        S[s] = Mfma16<T>::run(a, qreg[ks], S[s]);
-                    }
+                for (int ks = 0; ks < KS; ks++) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(stage + kr_off[ks]);
+                    S = Mfma16<T>::run(a, qreg[ks], S);
                 }
-
-                // ---- online softmax; lane holds positions t + 16 s + 4 jq + e of head `col` -------------
+                // V^T operands do not depend on the softmax: fetch them now
+                s16x4_t vt[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+                    vt[mt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(const_cast<unsigned char *>(stage) + vr_off[mt]));
+                }
+                float4 kscale, vscale;
+                if constexpr (KV8) {
+                    const float *sc = sc_lds + SL * 2 * kWaves * kStep;
+                    kscale = *reinterpret_cast<const float4 *>(sc + wave * kStep + 4 * jq);
+                    vscale = *reinterpret_cast<const float4 *>(sc + (kWaves + wave) * kStep + 4 * jq);
+                }
+                // ---- online softmax; lane holds positions t + 4 jq + e of head `col` ----------------------------
                 float mx = -INFINITY;
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        float v = S[s][e] * kLog2e;
-                        if constexpr (KV8) {
-                            v *= kscale[s][e];
-                        }
-                        v = (t + 16 * s + 4 * jq + e) < tb ? v : -INFINITY;  // also drops NaN of padding rows
-                        S[s][e] = v;
-                        mx = fmaxf(mx, v);
+                for (int e = 0; e < 4; e++) {
+                    float v = S[e] * kLog2e;
+                    if constexpr (KV8) {
+                        v *= reinterpret_cast<const float *>(&kscale)[e];
                     }
+                    v = (t + 4 * jq + e) < tb ? v : -INFINITY;   // padding positions (also drops their NaN)
+                    S[e] = v;
+                    mx = fmaxf(mx, v);
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16));
                 mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -295,51 +399,65 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 const float m_safe = m_new == -INFINITY ? 0.f : m_new;
                 const float alpha = fast_exp2(m_run - m_safe);
                 m_run = m_new;
-                float pe[2][4];
+                float pe[4];
                 float psum = 0.f;
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const float x = fast_exp2(S[s][e] - m_safe);
-                        psum += x;
-                        if constexpr (KV8) {
-                            // the scale of a padding row may be anything (even NaN): keep p at 0 there
-                            pe[s][e] = (t + 16 * s + 4 * jq + e) < tb ? x * vscale[s][e] : 0.f;
-                        } else {
-                            pe[s][e] = x;
-                        }
+                for (int e = 0; e < 4; e++) {
+                    const float x = fast_exp2(S[e] - m_safe);
+                    psum += x;
+                    if constexpr (KV8) {
+                        pe[e] = (t + 4 * jq + e) < tb ? x * reinterpret_cast<const float *>(&vscale)[e] : 0.f;
+                    } else {
+                        pe[e] = x;
                     }
                 }
                 l_run = l_run * alpha + psum;
-                const uint4 pb = make_uint4(T::pack(pe[0][0], pe[0][1]), T::pack(pe[0][2], pe[0][3]),
-                                            T::pack(pe[1][0], pe[1][1]), T::pack(pe[1][2], pe[1][3]));
+                const uint2 pb = make_uint2(T::pack(pe[0], pe[1]), T::pack(pe[2], pe[3]));
+                // the running maximum rarely moves after the first steps: skip the rescale then
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        O[mt][0] *= alpha;
+                        O[mt][1] *= alpha;
+                        O[mt][2] *= alpha;
+                        O[mt][3] *= alpha;
+                    }
+                }
+                // ---- O^T += V^T . P^T (k = the 16 positions) ------------------------------------------------------
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
-                    O[mt][0] *= alpha;
-                    O[mt][1] *= alpha;
-                    O[mt][2] *= alpha;
-                    O[mt][3] *= alpha;
+                    O[mt] = Mfma16<T>::run16(vt[mt], pb, O[mt]);
                 }
+            };
 
-                // ---- O^T += V^T . P^T ---------------------------------------------------------------------
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
-                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (lds_tr_ptr)(v_lds + vr_off[mt]));
-                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (lds_tr_ptr)(v_lds + vr_off[mt] + 16 * ROWB));
-                    const uint2 lo2 = __builtin_bit_cast(uint2, lo);
-                    const uint2 hi2 = __builtin_bit_cast(uint2, hi);
-                    O[mt] = Mfma16<T>::run(make_uint4(lo2.x, lo2.y, hi2.x, hi2.y), pb, O[mt]);
-                }
+            using S0 = std::integral_constant<int, 0>;
+            using S1 = std::integral_constant<int, 1>;
+            // Software pipeline: registers hold steps n+1 and n+2 while step n is computed from LDS.
+            // Every load and LDS write below is unconditional (steps past the end re-read the last
+            // step and land in a stage nobody consumes): a conditional prefetch would force the
+            // wait for the older batch to assume that the newer one was never issued, i.e. to wait
+            // for everything in flight.
+            const uint32_t last = n_steps - 1;   // n_steps >= 1: the tile is not empty
+            issue(0, S0{});
+            issue(min(1u, last), S1{});
+            stage_write(S0{});
+            issue(min(2u, last), S0{});
+            __syncthreads();
+            for (uint32_t step = 0; step < n_steps; step += 2) {
+                compute(step, S0{});
+                stage_write(S1{});
+                issue(min(step + 3, last), S1{});
+                __syncthreads();
+                compute(step + 1, S1{});
+                stage_write(S0{});
+                issue(min(step + 4, last), S0{});
+                __syncthreads();
             }
 
             // ---- this wave's result for (kv head, sub range) -----------------------------------------------
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
-            if (col < g_valid) {
+            if (kv_ok && col < g_valid) {
                 // O^T lane layout: column = head `col`, rows 16 mt + 4 jq + e
                 if (single) {
                     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -352,7 +470,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<uint2 *>(dst + mt * 16 + jq * 4) = o;
                     }
                 } else {
-                    const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * p.max_slots + tile * p.n_sub + sub;
+                    const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * p.max_slots + tile * p.n_sub + my_sub;
                     float *dst = p.part_acc + slot * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
@@ -362,73 +480,27 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
                     }
                 }
+                // every workgroup of the row stores the same count: no ordering needed
+                if (jq == 0 && tile == 0 && my_sub == 0 && p.part_cnt != nullptr) {
+                    p.part_cnt[static_cast<uint64_t>(tok) * p.n_heads + head0 + col] = single ? 0 : static_cast<int32_t>(n_tiles * p.n_sub);
+                }
             }
         }
-        if (single) {
-            continue;
-        }
-
-        // ---- publish, take a ticket; the last workgroup of the row merges all partials ---------------------
-        __threadfence();
-        __syncthreads();
-        int32_t *flag = reinterpret_cast<int32_t *>(smem);
-        int32_t *counter = p.counters + tok;
-        if (threadIdx.x == 0) {
-            *flag = atomicAdd(counter, 1);
-        }
-        __syncthreads();
-        const bool last = *flag == static_cast<int32_t>(n_tiles) - 1;
-        __syncthreads();
-        if (!last) {
-            continue;
-        }
-        __threadfence();
-        const uint32_t n_slots = n_tiles * p.n_sub;
-        constexpr int C4 = D / 4;
-        for (uint32_t it = threadIdx.x; it < p.n_heads * C4; it += kWaves * 64) {
-            const uint32_t head = it / C4, c = it % C4;
-            const uint64_t base = (static_cast<uint64_t>(tok) * p.n_heads + head) * p.max_slots;
-            float mm = -INFINITY;
-            for (uint32_t s = 0; s < n_slots; s++) {
-                mm = fmaxf(mm, p.part_ml[(base + s) * 2]);
-            }
-            const float ms = mm == -INFINITY ? 0.f : mm;
-            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-            float lsum = 0.f;
-            for (uint32_t s = 0; s < n_slots; s++) {
-                const float2 ml = *reinterpret_cast<const float2 *>(p.part_ml + (base + s) * 2);
-                const float w = fast_exp2(ml.x - ms);
-                lsum += ml.y * w;
-                const float4 x = *reinterpret_cast<const float4 *>(p.part_acc + (base + s) * D + c * 4);
-                acc.x += x.x * w;
-                acc.y += x.y * w;
-                acc.z += x.z * w;
-                acc.w += x.w * w;
-            }
-            const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-            uint2 o;
-            o.x = T::pack(acc.x * inv, acc.y * inv);
-            o.y = T::pack(acc.z * inv, acc.w * inv);
-            *reinterpret_cast<uint2 *>(p.out + (static_cast<uint64_t>(tok) * p.n_heads + head) * D + c * 4) = o;
-        }
-        if (threadIdx.x == 0) {
-            *counter = 0;
-        }
-        __syncthreads();
     }
 }
 
-template <typename T, int D, bool KV8>
-int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
+template <typename T, int D, bool KV8, bool MULTI_SUB>
+int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
 {
-    constexpr size_t lds = static_cast<size_t>(kWaves) * 2 * kStep * D * 2;
-    auto kernel = decode_mfma_kernel<T, D, KV8>;
+    const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
+                       (p.tile_tokens / kStep + 2) * sizeof(uint32_t);
+    auto kernel = decode_mfma_kernel<T, D, KV8, MULTI_SUB>;
     if (lds > 64 * 1024) {
-        static bool configured = false;
-        if (!configured) {
+        static size_t configured = 0;
+        if (configured < lds) {
             XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            configured = true;
+            configured = lds;
         }
     }
     dim3 grid(ceil_div(p.max_slots, p.n_sub), batch, 1);
@@ -437,14 +509,21 @@ int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
     return XLITE_HIP_OK;
 }
 
+template <typename T, int D, bool KV8>
+int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
+{
+    return p.n_sub > 1 ? launch_inst<T, D, KV8, true>(stream, p, batch)
+                       : launch_inst<T, D, KV8, false>(stream, p, batch);
+}
+
 }  // namespace
 
 bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
                            uint32_t total_tokens)
 {
     const uint32_t group = n_heads / n_kv_heads;
-    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16 &&
-           static_cast<size_t>(total_tokens) * sizeof(int32_t) <= XLITE_HIP_WS_COUNTER_BYTES;
+    (void)total_tokens;
+    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16;
 }
 
 void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, uint32_t max_num_block,
@@ -466,8 +545,7 @@ void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, 
 
 size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim, uint32_t max_slots)
 {
-    return XLITE_HIP_WS_COUNTER_BYTES +
-           static_cast<size_t>(total_tokens) * n_heads * max_slots * (head_dim + 2) * sizeof(float);
+    return max_slots > 1 ? partial_bytes(total_tokens, n_heads, head_dim, max_slots) : 0;
 }
 
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
@@ -479,6 +557,8 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
         return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
                                                     " bytes, have " + std::to_string(a.workspace_bytes));
     }
+    const PartialBuffers pb = max_slots > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_slots)
+                                            : PartialBuffers{};
     DecodeMfmaParams p{};
     p.q = static_cast<const uint16_t *>(a.qkv);
     p.k_cache = a.k_cache;
@@ -490,10 +570,9 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     p.lens = a.lens;
     p.cached_lens = a.cached_lens;
     p.block_tables = a.block_tables;
-    char *ws = static_cast<char *>(a.workspace);
-    p.counters = reinterpret_cast<int32_t *>(ws);
-    p.part_acc = ws ? reinterpret_cast<float *>(ws + XLITE_HIP_WS_COUNTER_BYTES) : nullptr;
-    p.part_ml = ws ? p.part_acc + static_cast<size_t>(a.total_tokens) * a.n_heads * max_slots * a.head_dim : nullptr;
+    p.part_cnt = pb.cnt;
+    p.part_acc = pb.acc;
+    p.part_ml = pb.ml;
     p.q_row_stride = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
     p.n_heads = a.n_heads;
     p.n_kv_heads = a.n_kv_heads;
@@ -506,16 +585,22 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
 
     const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
     const bool bf = a.dtype == XLITE_HIP_BF16;
+    int rc;
     if (a.head_dim == 128) {
         if (bf) {
-            return kv8 ? launch_one<BF16, 128, true>(stream, p, a.batch) : launch_one<BF16, 128, false>(stream, p, a.batch);
+            rc = kv8 ? launch_one<BF16, 128, true>(stream, p, a.batch) : launch_one<BF16, 128, false>(stream, p, a.batch);
+        } else {
+            rc = kv8 ? launch_one<FP16, 128, true>(stream, p, a.batch) : launch_one<FP16, 128, false>(stream, p, a.batch);
         }
-        return kv8 ? launch_one<FP16, 128, true>(stream, p, a.batch) : launch_one<FP16, 128, false>(stream, p, a.batch);
+    } else if (bf) {
+        rc = kv8 ? launch_one<BF16, 64, true>(stream, p, a.batch) : launch_one<BF16, 64, false>(stream, p, a.batch);
+    } else {
+        rc = kv8 ? launch_one<FP16, 64, true>(stream, p, a.batch) : launch_one<FP16, 64, false>(stream, p, a.batch);
     }
-    if (bf) {
-        return kv8 ? launch_one<BF16, 64, true>(stream, p, a.batch) : launch_one<BF16, 64, false>(stream, p, a.batch);
+    if (rc != XLITE_HIP_OK || max_slots == 1) {
+        return rc;
     }
-    return kv8 ? launch_one<FP16, 64, true>(stream, p, a.batch) : launch_one<FP16, 64, false>(stream, p, a.batch);
+    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, max_slots);
 }
 
 }  // namespace xlite

@@ -1,0 +1,91 @@
+// Merge of split-KV partial results: out[row][head] = sum_s w_s O_s / sum_s w_s l_s with
+// w_s = 2^(m_s - max_s m_s) (maxima are kept in the log2 domain). A separate launch instead of a
+// "last workgroup to finish merges" scheme: the device-scope fences the latter needs write back
+// and invalidate the L2 of every XCD once per workgroup, which costs far more than this kernel.
+// The algebra is the online-softmax update of the reference
+// (xlite/csrc/kernels/softmax_attn_aiv.h:595-647), applied once over fp32 partials.
+#include "attention_common.h"
+
+namespace xlite {
+
+namespace {
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
+             const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t n_heads,
+             uint32_t dv, uint32_t max_slots)
+{
+    const uint32_t row = blockIdx.x;
+    const uint32_t c4 = dv / 4;
+    for (uint32_t it = threadIdx.x; it < n_heads * c4; it += blockDim.x) {
+        const uint32_t head = it / c4, c = it % c4;
+        const uint64_t rh = static_cast<uint64_t>(row) * n_heads + head;
+        const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
+        if (n == 0) {
+            continue;  // the producer wrote the final value itself
+        }
+        const uint64_t base = rh * max_slots;
+        float mm = -INFINITY;
+        for (uint32_t s = 0; s < n; s++) {
+            mm = fmaxf(mm, part_ml[(base + s) * 2]);
+        }
+        const float ms = mm == -INFINITY ? 0.f : mm;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float lsum = 0.f;
+        for (uint32_t s = 0; s < n; s++) {
+            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + (base + s) * 2);
+            const float w = fast_exp2(ml.x - ms);
+            lsum += ml.y * w;
+            const float4 x = *reinterpret_cast<const float4 *>(part_acc + (base + s) * dv + c * 4);
+            acc.x += x.x * w;
+            acc.y += x.y * w;
+            acc.z += x.z * w;
+            acc.w += x.w * w;
+        }
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+        uint2 o;
+        o.x = T::pack(acc.x * inv, acc.y * inv);
+        o.y = T::pack(acc.z * inv, acc.w * inv);
+        *reinterpret_cast<uint2 *>(out + rh * dv + c * 4) = o;
+    }
+}
+
+}  // namespace
+
+size_t partial_bytes(uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots)
+{
+    const size_t rh = static_cast<size_t>(rows) * n_heads;
+    return ((rh * sizeof(int32_t) + 255) / 256) * 256 + rh * max_slots * (dv + 2) * sizeof(float);
+}
+
+PartialBuffers carve_partials(void *workspace, uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots)
+{
+    PartialBuffers b{};
+    if (workspace == nullptr) {
+        return b;
+    }
+    const size_t rh = static_cast<size_t>(rows) * n_heads;
+    char *ws = static_cast<char *>(workspace);
+    b.cnt = reinterpret_cast<int32_t *>(ws);
+    b.acc = reinterpret_cast<float *>(ws + ((rh * sizeof(int32_t) + 255) / 256) * 256);
+    b.ml = b.acc + rh * max_slots * dv;
+    return b;
+}
+
+int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
+                 uint32_t n_heads, uint32_t dv, uint32_t max_slots)
+{
+    if (rows == 0) {
+        return XLITE_HIP_OK;
+    }
+    if (dtype == XLITE_HIP_BF16) {
+        merge_kernel<BF16><<<rows, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+    } else {
+        merge_kernel<FP16><<<rows, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+}  // namespace xlite

@@ -13,8 +13,8 @@
 // permuted identically on the V^T side). Scores and outputs accumulate in fp32; P is rounded to
 // the 16-bit storage type before the second product, as in the reference (softmax_attn_aiv.h:904-908).
 //
-// The KV range of an M tile can be split across workgroups (grid.x); partial (max, sum, O) are
-// merged by the last workgroup to finish.
+// The KV range of an M tile can be split across workgroups (grid.x); their partial (max, sum, O)
+// are merged by a second small kernel (merge.hip).
 //
 // Replaces attention.h / flash_attention.h for batches with multi-token queries
 // (xlite/csrc/kernels/attention.h:308-492) and mla_v2.h / flash_mla_v2.h / mla_v3.h.
@@ -59,7 +59,7 @@ struct MfmaParams {
     const int32_t *lens;
     const int32_t *cached_lens;
     const int32_t *block_tables;  // nullptr: dense cache of dense_len rows per sequence, no causality
-    int32_t *counters;
+    int32_t *part_cnt;   // [token][head] number of partial splits (0: final value stored directly)
     float *part_acc;
     float *part_ml;
     uint32_t q0_tok_stride, q0_head_stride, q1_tok_stride, q1_head_stride;
@@ -102,7 +102,6 @@ mfma_attention_kernel(const MfmaParams p)
     uint16_t *Ks = reinterpret_cast<uint16_t *>(smem_raw);
     uint16_t *Vt = Ks + BN * KSTRIDE;
     uint64_t *rowidx = reinterpret_cast<uint64_t *>(Vt + DV * VSTRIDE);
-    int32_t *flag = reinterpret_cast<int32_t *>(rowidx + BN);
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
@@ -312,8 +311,9 @@ mfma_attention_kernel(const MfmaParams p)
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
 
-    if (n_splits == 1) {
-        if (m_valid) {
+    if (m_valid) {
+        const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head;
+        if (n_splits == 1) {
             const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
             uint16_t *dst = p.out + static_cast<uint64_t>(tok) * p.out_tok_stride + static_cast<uint64_t>(head) * DV;
 #pragma unroll
@@ -326,77 +326,32 @@ mfma_attention_kernel(const MfmaParams p)
                     *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
                 }
             }
-        }
-        return;
-    }
-
-    // ---- partial result, ticket, merge by the last split to finish ------------------------------------------
-    if (m_valid) {
-        const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head) * p.max_splits + split;
-        float *dst = p.part_acc + slot * DV;
+        } else {
+            // partial result of this split; a second kernel merges the splits of every row (merge.hip)
+            const uint64_t slot = rh * p.max_splits + split;
+            float *dst = p.part_acc + slot * DV;
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
+            for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
-            for (int kg = 0; kg < 4; kg++) {
-                *reinterpret_cast<float4 *>(dst + dt * 32 + kg * 8 + half * 4) =
-                    make_float4(O[dt][kg * 4], O[dt][kg * 4 + 1], O[dt][kg * 4 + 2], O[dt][kg * 4 + 3]);
+                for (int kg = 0; kg < 4; kg++) {
+                    *reinterpret_cast<float4 *>(dst + dt * 32 + kg * 8 + half * 4) =
+                        make_float4(O[dt][kg * 4], O[dt][kg * 4 + 1], O[dt][kg * 4 + 2], O[dt][kg * 4 + 3]);
+                }
+            }
+            if (half == 0) {
+                *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
             }
         }
-        if (half == 0) {
-            *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+        if (half == 0 && split == 0 && p.part_cnt != nullptr) {
+            p.part_cnt[rh] = n_splits == 1 ? 0 : static_cast<int32_t>(n_splits);
         }
-    }
-    __threadfence();
-    __syncthreads();
-    int32_t *counter = p.counters + static_cast<uint64_t>(blockIdx.z) * gridDim.y + blockIdx.y;
-    if (threadIdx.x == 0) {
-        *flag = atomicAdd(counter, 1);
-    }
-    __syncthreads();
-    if (*flag != static_cast<int32_t>(n_splits) - 1) {
-        return;
-    }
-    __threadfence();
-
-    constexpr int CH = DV / 4;  // float4 chunks per row
-    const uint32_t rows = m_last - m_first + 1;
-    for (uint32_t it = threadIdx.x; it < rows * CH; it += kThreads) {
-        const uint32_t mm = m_first + it / CH, c = it % CH;
-        const uint32_t t2 = static_cast<uint32_t>(qstart) + mm / G;
-        const uint32_t h2 = kvh * G + mm % G;
-        const uint64_t base = (static_cast<uint64_t>(t2) * p.n_heads + h2) * p.max_splits;
-        float mxx = -INFINITY;
-        for (uint32_t s = 0; s < n_splits; s++) {
-            mxx = fmaxf(mxx, p.part_ml[(base + s) * 2]);
-        }
-        const float ms = mxx == -INFINITY ? 0.f : mxx;
-        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        float lsum = 0.f;
-        for (uint32_t s = 0; s < n_splits; s++) {
-            const float2 ml = *reinterpret_cast<const float2 *>(p.part_ml + (base + s) * 2);
-            const float w = fast_exp2(ml.x - ms);
-            lsum += ml.y * w;
-            const float4 x = *reinterpret_cast<const float4 *>(p.part_acc + (base + s) * DV + c * 4);
-            acc.x += x.x * w;
-            acc.y += x.y * w;
-            acc.z += x.z * w;
-            acc.w += x.w * w;
-        }
-        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-        uint2 o;
-        o.x = T::pack(acc.x * inv, acc.y * inv);
-        o.y = T::pack(acc.z * inv, acc.w * inv);
-        *reinterpret_cast<uint2 *>(p.out + static_cast<uint64_t>(t2) * p.out_tok_stride + static_cast<uint64_t>(h2) * DV + c * 4) = o;
-    }
-    if (threadIdx.x == 0) {
-        *counter = 0;
     }
 }
 
 template <int DQK, int DV, int BN>
 constexpr size_t lds_bytes()
 {
-    return static_cast<size_t>(BN) * (DQK + 8) * 2 + static_cast<size_t>(DV) * (BN + 8) * 2 + BN * 8 + 16;
+    return static_cast<size_t>(BN) * (DQK + 8) * 2 + static_cast<size_t>(DV) * (BN + 8) * 2 + BN * 8;
 }
 
 template <typename T, int DQ0, int DQ1, int DV, int BN, bool SEPARATE_V>
@@ -417,13 +372,11 @@ int launch_kernel(hipStream_t stream, const MfmaParams &p, dim3 grid)
     return XLITE_HIP_OK;
 }
 
-void fill_common(MfmaParams &p, void *workspace, uint32_t total_tokens, uint32_t n_heads, uint32_t dv,
-                 uint32_t max_splits)
+void fill_common(MfmaParams &p, const PartialBuffers &pb)
 {
-    char *ws = static_cast<char *>(workspace);
-    p.counters = reinterpret_cast<int32_t *>(ws);
-    p.part_acc = ws ? reinterpret_cast<float *>(ws + XLITE_HIP_WS_COUNTER_BYTES) : nullptr;
-    p.part_ml = ws ? p.part_acc + static_cast<size_t>(total_tokens) * n_heads * max_splits * dv : nullptr;
+    p.part_cnt = pb.cnt;
+    p.part_acc = pb.acc;
+    p.part_ml = pb.ml;
 }
 
 }  // namespace
@@ -432,11 +385,7 @@ bool mfma_gqa_supported(uint32_t head_dim) { return head_dim == 64 || head_dim =
 
 size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits)
 {
-    if (splits <= 1) {
-        return XLITE_HIP_WS_COUNTER_BYTES;
-    }
-    return XLITE_HIP_WS_COUNTER_BYTES +
-           static_cast<size_t>(total_tokens) * n_heads * splits * (dv + 2) * sizeof(float);
+    return splits <= 1 ? 0 : partial_bytes(total_tokens, n_heads, dv, splits);
 }
 
 // Number of KV splits so that about two workgroups per compute unit exist; the split length is a
@@ -465,9 +414,8 @@ int launch_mfma_gqa(hipStream_t stream, const AttentionArgs &a)
     const uint32_t max_ctx = a.max_num_block * a.block_size;
     uint32_t splits = mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, max_ctx, BN);
     const uint32_t m_tiles = ceil_div(a.total_tokens * G, kMTile) + a.batch;
-    if (static_cast<size_t>(m_tiles) * a.n_kv_heads * sizeof(int32_t) > XLITE_HIP_WS_COUNTER_BYTES ||
-        a.workspace == nullptr ||
-        a.workspace_bytes < mfma_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, splits)) {
+    if (a.workspace == nullptr ||
+        a.workspace_bytes < mfma_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, splits + 1)) {
         splits = 1;  // no scratch: every M tile walks its whole KV range
     }
     uint32_t split_len = ceil_div(ceil_div(max_ctx, splits), BN) * BN;
@@ -500,16 +448,24 @@ int launch_mfma_gqa(hipStream_t stream, const AttentionArgs &a)
     p.split_len = split_len;
     p.max_splits = max_splits;
     p.scale_log2e = kLog2e;
-    fill_common(p, a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_splits);
+    const PartialBuffers pb = max_splits > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_splits)
+                                             : PartialBuffers{};
+    fill_common(p, pb);
 
     dim3 grid(max_splits, m_tiles, a.n_kv_heads);
     const bool bf = a.dtype == XLITE_HIP_BF16;
+    int rc;
     if (a.head_dim == 128) {
-        return bf ? launch_kernel<BF16, 128, 0, 128, BN, true>(stream, p, grid)
-                  : launch_kernel<FP16, 128, 0, 128, BN, true>(stream, p, grid);
+        rc = bf ? launch_kernel<BF16, 128, 0, 128, BN, true>(stream, p, grid)
+                : launch_kernel<FP16, 128, 0, 128, BN, true>(stream, p, grid);
+    } else {
+        rc = bf ? launch_kernel<BF16, 64, 0, 64, BN, true>(stream, p, grid)
+                : launch_kernel<FP16, 64, 0, 64, BN, true>(stream, p, grid);
     }
-    return bf ? launch_kernel<BF16, 64, 0, 64, BN, true>(stream, p, grid)
-              : launch_kernel<FP16, 64, 0, 64, BN, true>(stream, p, grid);
+    if (rc != XLITE_HIP_OK || max_splits == 1) {
+        return rc;
+    }
+    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, max_splits);
 }
 
 int launch_mfma_mla(hipStream_t stream, const MlaArgs &a)
@@ -519,8 +475,8 @@ int launch_mfma_mla(hipStream_t stream, const MlaArgs &a)
     const uint32_t max_ctx = dense ? a.dense_len : a.max_num_blocks * a.block_size;
     uint32_t splits = mfma_pick_splits(a.total_tokens, a.n_heads, a.batch, 1, max_ctx, BN);
     const uint32_t m_tiles = ceil_div(a.total_tokens * a.n_heads, kMTile) + a.batch;
-    if (static_cast<size_t>(m_tiles) * sizeof(int32_t) > XLITE_HIP_WS_COUNTER_BYTES || a.workspace == nullptr ||
-        a.workspace_bytes < mfma_workspace_bytes(a.total_tokens, a.n_heads, a.kv_lora_rank, splits)) {
+    if (a.workspace == nullptr ||
+        a.workspace_bytes < mfma_workspace_bytes(a.total_tokens, a.n_heads, a.kv_lora_rank, splits + 1)) {
         splits = 1;
     }
     uint32_t split_len = ceil_div(ceil_div(max_ctx, splits), BN) * BN;
@@ -557,11 +513,17 @@ int launch_mfma_mla(hipStream_t stream, const MlaArgs &a)
     p.split_len = split_len;
     p.max_splits = max_splits;
     p.scale_log2e = a.scale * kLog2e;
-    fill_common(p, a.workspace, a.total_tokens, a.n_heads, a.kv_lora_rank, max_splits);
+    const PartialBuffers pb = max_splits > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, a.kv_lora_rank, max_splits)
+                                             : PartialBuffers{};
+    fill_common(p, pb);
 
     dim3 grid(max_splits, m_tiles, 1);
     if (a.kv_lora_rank == 512 && a.rope_head_dim == 64) {
-        return launch_kernel<BF16, 512, 64, 512, BN, false>(stream, p, grid);
+        const int rc = launch_kernel<BF16, 512, 64, 512, BN, false>(stream, p, grid);
+        if (rc != XLITE_HIP_OK || max_splits == 1) {
+            return rc;
+        }
+        return launch_merge(stream, a.dtype, a.o_absorb, pb, a.total_tokens, a.n_heads, a.kv_lora_rank, max_splits);
     }
     return fail(XLITE_HIP_EINVAL, __func__,
                 "only kv_lora_rank 512 with rope_head_dim 64 is built for the matrix-core path");

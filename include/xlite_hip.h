@@ -77,11 +77,11 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  * Row r of sequence i attends to cache positions 0 .. cached_lens[i] + r.
  * No softmax scale is applied here (q arrives pre-scaled).
  *
- * workspace   device scratch of at least xlite_hip_attention_workspace_bytes();
- *             its first XLITE_HIP_WS_COUNTER_BYTES must be zero before the first
- *             call and are left zero by every call.
+ * workspace   device scratch of at least xlite_hip_attention_workspace_bytes()
+ *             (split-KV partial results; contents need no initialisation and
+ *             are not preserved). With a smaller or NULL workspace the call
+ *             still works but splits the KV axis less, or not at all.
  * ---------------------------------------------------------------------- */
-#define XLITE_HIP_WS_COUNTER_BYTES 65536
 
 size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
                                            uint32_t n_kv_heads, uint32_t head_dim,
