@@ -17,7 +17,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 # packed fp32 ops are switched off on purpose (device code only); the host pass of hipcc does
 # not know the feature and says so, which is harmless
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-ffp-contract=off"]
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-inline-asm", "-ffp-contract=off"]
 
 
 def sources():

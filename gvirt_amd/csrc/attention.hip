@@ -101,7 +101,27 @@ extern "C" size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t 
 {
     const uint32_t max_ctx = max_num_blocks * block_size;
     const uint32_t splits = mfma_pick_splits(total_tokens, n_heads, batch, 1, max_ctx, 32);
-    return mfma_workspace_bytes(total_tokens, n_heads, kv_lora_rank, splits + 1);
+    size_t need = mfma_workspace_bytes(total_tokens, n_heads, kv_lora_rank, splits + 1);
+    if (total_tokens == batch && block_size > 0) {
+        // the decode kernel plans its own tiles; block_size == 1 describes a dense cache of
+        // max_num_blocks rows per sequence
+        MlaArgs a{};
+        a.total_tokens = total_tokens;
+        a.batch = batch;
+        a.n_heads = n_heads;
+        a.kv_lora_rank = kv_lora_rank;
+        a.block_size = block_size;
+        a.max_num_blocks = max_num_blocks;
+        a.dense_len = max_num_blocks * block_size;
+        static const int32_t dummy = 0;
+        a.block_tables = &dummy;
+        const size_t d = mla_decode_workspace_bytes(a);
+        need = d > need ? d : need;
+        a.block_tables = nullptr;
+        const size_t d2 = mla_decode_workspace_bytes(a);
+        need = d2 > need ? d2 : need;
+    }
+    return need;
 }
 
 extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const void *qr,
@@ -132,6 +152,9 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
     MlaArgs a{q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks,
               0, scale, topk_indices, top_k, dtype, workspace, workspace_bytes};
+    if (mla_decode_supported(a)) {
+        return launch_mla_decode(as_stream(stream), a);
+    }
     return launch_mfma_mla(as_stream(stream), a);
 }
 
@@ -156,5 +179,8 @@ extern "C" int xlite_hip_mla_v3(void *stream, const void *q_absorb, const void *
     MlaArgs a{q_absorb, qr, k_dense, pe_dense, o_absorb, query_start_loc, lens, cached_lens, nullptr,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, 1, batch, index_topk,
               index_topk, scale, nullptr, 0, dtype, workspace, workspace_bytes};
+    if (mla_decode_supported(a)) {
+        return launch_mla_decode(as_stream(stream), a);
+    }
     return launch_mfma_mla(as_stream(stream), a);
 }

@@ -74,6 +74,11 @@ void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, 
 size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim, uint32_t max_slots);
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
 
+// mla_decode.hip
+bool mla_decode_supported(const MlaArgs &a);
+size_t mla_decode_workspace_bytes(const MlaArgs &a);
+int launch_mla_decode(hipStream_t stream, const MlaArgs &a);
+
 // mfma_attention.hip
 bool mfma_gqa_supported(uint32_t head_dim);
 size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits);

@@ -18,7 +18,7 @@ merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
 {
     const uint32_t row = blockIdx.x;
     const uint32_t c4 = dv / 4;
-    for (uint32_t it = threadIdx.x; it < n_heads * c4; it += blockDim.x) {
+    for (uint32_t it = blockIdx.y * blockDim.x + threadIdx.x; it < n_heads * c4; it += gridDim.y * blockDim.x) {
         const uint32_t head = it / c4, c = it % c4;
         const uint64_t rh = static_cast<uint64_t>(row) * n_heads + head;
         const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
@@ -79,10 +79,12 @@ int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers 
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
+    // one thread per (row, head, four output columns)
+    const dim3 grid(rows, min(ceil_div(n_heads * (dv / 4), 256u), 65535u), 1);
     if (dtype == XLITE_HIP_BF16) {
-        merge_kernel<BF16><<<rows, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+        merge_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
     } else {
-        merge_kernel<FP16><<<rows, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+        merge_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

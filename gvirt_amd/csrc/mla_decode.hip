@@ -1,0 +1,448 @@
+// DeepSeek-style absorbed MLA decode on the matrix cores, split along the KV axis.
+//
+// One latent "kv head" is shared by all query heads, so the heads are the MFMA columns: a
+// workgroup of 4 wavefronts (one per SIMD, each with the full 512-register budget) covers up to
+// 128 heads, 32 per wave, of one (sequence, KV tile). The tile is walked in steps of 32 positions:
+//   S^T[pos][head]  = [kc | pe][pos][:] . [q_absorb | qr][head][:]   36 x v_mfma_f32_32x32x16_bf16
+//   O^T[c][head]   += kc^T[c][pos] . P^T[pos][head]                   32 x v_mfma_f32_32x32x16_bf16
+// Register plan per lane: Q (B operand of the first product) 144, O^T accumulators 256, the rest
+// for S, P and operands in flight. The cache never passes through registers: every wave copies its
+// share of a step straight from global memory into LDS (global_load_lds_dwordx4, 1 KiB of
+// consecutive cache bytes per instruction) into a ring of four 36 KiB stages, three steps in
+// flight while the fourth is consumed, one barrier per step. K rows are read from LDS as MFMA A
+// operands with ds_read_b128; the latent is read again, transposed, with ds_read_b64_tr_b16, so the
+// same LDS bytes serve both products. The 16-byte chunks of a row are XOR-swizzled (by choosing
+// which global chunk a lane copies) so that both read shapes are bank-conflict free.
+// Every workgroup leaves fp32 partials (max, sum, O) that a second kernel merges (merge.hip).
+//
+// Replaces mla_v2.h / flash_mla_v2.h (paged cache, xlite/csrc/kernels/flash_mla_v2.h:537-847) and
+// mla_v3.h (dense per-sequence cache) of the reference for batches with one query row per sequence.
+#include "attention_common.h"
+
+namespace xlite {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kRescaleSlack = 8.0f;
+constexpr int kWaves = 4;
+constexpr int kNT = kWaves * 64;
+constexpr int kStep = 32;
+constexpr int kStages = 4;
+constexpr int C = 512;                 // kv_lora_rank
+constexpr int R = 64;                  // rope_head_dim
+constexpr int KS_C = C / 16;           // k-steps over the latent part
+constexpr int KS_R = R / 16;           // k-steps over the rotary part
+constexpr int DT = C / 32;             // 32-row tiles of O^T
+constexpr int KC_ROWB = C * 2;         // 1024: LDS bytes of a latent row
+constexpr int PE_ROWB = R * 2;         // 128
+constexpr int KC_BYTES = kStep * KC_ROWB;             // 32 KiB
+constexpr int STAGE_BYTES = KC_BYTES + kStep * PE_ROWB;  // 36 KiB: latent rows, then rotary rows
+constexpr int DMA_PER_WAVE = (kStep + kStep * PE_ROWB / 1024) / kWaves;  // 8 latent rows + 1 rotary block
+
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+
+struct MlaDecodeParams {
+    const uint16_t *q_absorb;
+    const uint16_t *qr;
+    const uint16_t *k_cache;
+    const uint16_t *pe_cache;
+    uint16_t *out;
+    const int32_t *query_start_loc;
+    const int32_t *lens;
+    const int32_t *cached_lens;
+    const int32_t *block_tables;   // nullptr: dense cache, dense_len rows per sequence, no causality
+    int32_t *part_cnt;
+    float *part_acc;
+    float *part_ml;
+    uint32_t n_heads;
+    uint32_t block_size;
+    uint32_t max_num_blocks;
+    uint32_t dense_len;
+    uint32_t tile_tokens;
+    uint32_t max_slots;
+    float scale_log2e;
+};
+
+// XOR patterns for the 16-byte chunk index inside a row.
+// Latent rows (1024 bytes, every row starts at bank 0): low four chunk bits. The 16 rows that one
+// ds_read_b128 pass touches get 16 different chunk slots, and the 4 rows that one transposing pass
+// touches get 4 different 64-byte groups.
+__device__ __forceinline__ uint32_t swz_kc(uint32_t row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// Rotary rows (128 bytes, two per bank window): low three chunk bits; rows of equal parity differ.
+__device__ __forceinline__ uint32_t swz_pe(uint32_t row) { return (row >> 1) & 7; }
+
+// One wave-wide copy of 1 KiB from global memory into LDS at `lds_addr` + 16 * lane. The compiler
+// does not see the LDS write nor the vmcnt increment: completion is awaited with dma_wait below.
+__device__ __forceinline__ void dma_1k(uint32_t lds_addr, uint32_t voff, const void *base)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                 :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+__global__ void __launch_bounds__(kNT)
+mla_decode_kernel(const MlaDecodeParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE_BYTES);
+    const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
+        static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t tile = blockIdx.x;
+    const uint32_t seq = blockIdx.y;
+    const uint32_t col = lane & 31;
+    const uint32_t half = lane >> 5;
+    const bool dense = p.block_tables == nullptr;
+
+    // ---- copy roles: wave w moves latent rows w, w+4, .. (lane = chunk slot) and rotary rows
+    // 8w .. 8w+7 (lane / 8 = row, lane % 8 = chunk slot); a slot holds chunk (slot ^ pattern(row))
+    uint32_t kc_voff[kStep / kWaves];
+#pragma unroll
+    for (int i = 0; i < kStep / kWaves; i++) {
+        const uint32_t row = wave + kWaves * i;
+        kc_voff[i] = row * KC_ROWB + (((lane & ~15u) | ((lane & 15u) ^ swz_kc(row))) << 4);
+    }
+    const uint32_t pe_row = wave * 8 + (lane >> 3);
+    const uint32_t pe_chunk = (lane & 7u) ^ swz_pe(pe_row);
+
+    // ---- read roles --------------------------------------------------------------------------------
+    // K rows as the A operand: row = position `col`, chunk 2 ks + half; chunk' = 2 ks ^ x
+    const uint32_t kx = (half ^ swz_kc(col)) << 4;                    // latent part, low 8 address bits
+    const uint32_t px = (half ^ swz_pe(col)) << 4;                    // rotary part, low 7 address bits
+    const uint32_t k_row = col * KC_ROWB;
+    const uint32_t p_row = KC_BYTES + col * PE_ROWB;
+    // transposed latent: 16-lane group g = lane / 16 covers columns 16 (g % 2) .. +16 of a 32-column
+    // tile for the positions of half g / 2; lane 4 j' + q points at elements [4 q, +4) of position
+    // 4 half + j' (+8 for the second read, +16 for the second k-step)
+    uint32_t vr_off[4][2];
+    {
+        const uint32_t g = lane >> 4, jp = (lane & 15) >> 2, q = lane & 3;
+        const uint32_t y = 2 * (g & 1) + (q >> 1);
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+#pragma unroll
+            for (int rd = 0; rd < 2; rd++) {
+                const uint32_t pos = 4 * (g >> 1) + jp + 8 * rd;
+                vr_off[a][rd] = pos * KC_ROWB + ((((4 * a + y) & 15u) ^ swz_kc(pos)) << 4) + ((q & 1) << 3);
+            }
+        }
+    }
+
+    const int32_t qlen = p.lens[seq];
+    const int32_t clen = p.cached_lens[seq];
+    const int32_t qstart = p.query_start_loc[seq];
+    const int32_t *table = dense ? nullptr : p.block_tables + static_cast<uint64_t>(seq) * p.max_num_blocks;
+
+    for (int32_t r = 0; r < qlen; r++) {
+        const uint32_t tok = static_cast<uint32_t>(qstart + r);
+        const uint32_t limit = dense ? min(static_cast<uint32_t>(clen + qlen), p.dense_len)
+                                     : static_cast<uint32_t>(clen + r + 1);
+        const uint32_t n_tiles = ceil_div(limit, p.tile_tokens);
+        if (tile >= n_tiles) {
+            continue;
+        }
+        const uint32_t t0 = tile * p.tile_tokens;
+        const uint32_t t1 = min(limit, t0 + p.tile_tokens);
+        const uint32_t n_steps = ceil_div(t1 - t0, kStep);
+        const bool single = n_tiles == 1;
+        const uint32_t blk0 = dense ? 0 : t0 / p.block_size;
+        if (!dense) {
+            // block-table entries of the tile (lookups in the loop then cost an LDS read only)
+            const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
+            for (uint32_t i = threadIdx.x; i < nblk; i += kNT) {
+                tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
+            }
+        }
+        __syncthreads();
+
+        // passes over groups of 128 heads
+        for (uint32_t h0 = 0; h0 < p.n_heads; h0 += 32 * kWaves) {
+            const uint32_t head = h0 + wave * 32 + col;
+            const bool h_ok = head < p.n_heads;
+
+            // ---- [q_absorb | qr] as the B operand: column = head, 8 consecutive elements per half
+            uint4 qreg[KS_C + KS_R];
+            {
+                const uint16_t *qa = p.q_absorb + (static_cast<uint64_t>(tok) * p.n_heads + head) * C;
+                const uint16_t *qq = p.qr + (static_cast<uint64_t>(tok) * p.n_heads + head) * R;
+#pragma unroll
+                for (int ks = 0; ks < KS_C + KS_R; ks++) {
+                    const int e0 = ks * 16 + half * 8;
+                    qreg[ks] = !h_ok ? make_uint4(0, 0, 0, 0)
+                               : (ks < KS_C ? *reinterpret_cast<const uint4 *>(qa + e0)
+                                            : *reinterpret_cast<const uint4 *>(qq + (e0 - C)));
+                }
+                // consume the registers now: all memory loads the compiler knows of are then complete,
+                // and it never waits on vmcnt inside the streaming loop (where the copies are in flight)
+#pragma unroll
+                for (int ks = 0; ks < KS_C + KS_R; ks++) {
+                    asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+                }
+            }
+            f32x16_t O[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    O[dt][k] = 0.f;
+                }
+            }
+            float m_run = -INFINITY, l_run = 0.f;
+
+            // first cache row of a step: its 32 positions share one block (block_size % 32 == 0)
+            auto issue = [&](uint32_t step) {
+                const uint32_t ts = t0 + step * kStep;
+                uint64_t row0;
+                if (dense) {
+                    row0 = static_cast<uint64_t>(seq) * p.dense_len + ts;
+                } else {
+                    const uint32_t blk = ts / p.block_size, off = ts % p.block_size;
+                    const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
+                    row0 = static_cast<uint64_t>(phys) * p.block_size + off;
+                }
+                // positions at or beyond the end re-read the last valid one: finite values whose
+                // probabilities are forced to zero
+                const uint32_t last_pos = min(t1 - 1 - ts, static_cast<uint32_t>(kStep - 1));
+                const uint32_t stage = smem_addr + (step % kStages) * STAGE_BYTES;
+                const char *kb = reinterpret_cast<const char *>(p.k_cache) + row0 * KC_ROWB;
+                const char *pb = reinterpret_cast<const char *>(p.pe_cache) + row0 * PE_ROWB;
+#pragma unroll
+                for (int i = 0; i < kStep / kWaves; i++) {
+                    const uint32_t row = wave + kWaves * i;
+                    const uint32_t back = row > last_pos ? (row - last_pos) * KC_ROWB : 0u;   // uniform
+                    dma_1k(stage + row * KC_ROWB, kc_voff[i], kb - back);
+                }
+                const uint32_t prow = min(pe_row, last_pos);
+                dma_1k(stage + KC_BYTES + wave * 1024, prow * PE_ROWB + (pe_chunk << 4), pb);
+            };
+
+            auto compute = [&](uint32_t step) {
+                const uint32_t t = t0 + step * kStep;
+                const unsigned char *stage = smem + (step % kStages) * STAGE_BYTES;
+                // ---- S^T = K . Q^T: 32 positions x 32 heads, -----------------------------------------
+                f32x16_t Sa;
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    Sa[k] = 0.f;
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS_C; ks++) {
+                    const uint32_t off = k_row + ((ks >> 3) << 8) + ((((2 * ks) & 15) << 4) ^ kx);
+                    const uint4 a = *reinterpret_cast<const uint4 *>(stage + off);
+                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                                 __builtin_bit_cast(bf16x8_t, qreg[ks]), Sa, 0, 0, 0);
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS_R; ks++) {
+                    const uint32_t off = p_row + ((((2 * ks) & 7) << 4) ^ px);
+                    const uint4 a = *reinterpret_cast<const uint4 *>(stage + off);
+                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                                 __builtin_bit_cast(bf16x8_t, qreg[KS_C + ks]), Sa, 0, 0, 0);
+                }
+                // ---- online softmax; register k holds position t + 8 (k / 4) + 4 half + k % 4 ---------------
+                float mx = -INFINITY;
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    const uint32_t pos = t + (k / 4) * 8 + half * 4 + (k % 4);
+                    const float v = pos < t1 ? Sa[k] * p.scale_log2e : -INFINITY;
+                    Sa[k] = v;
+                    mx = fmaxf(mx, v);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                // the reference maximum only moves when the step maximum exceeds it by more than 2^8:
+                // probabilities then stay below 2^8 (exact in bf16 to the same relative precision, and the
+                // normaliser shares the reference), and the accumulators are rescaled rarely
+                const float m_new = mx > m_run + kRescaleSlack ? mx : m_run;
+                const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = fast_exp2(m_run - m_safe);
+                m_run = m_new;
+                uint32_t pw[8];
+                float psum = 0.f;
+#pragma unroll
+                for (int k = 0; k < 16; k += 2) {
+                    const float e0 = fast_exp2(Sa[k] - m_safe);
+                    const float e1 = fast_exp2(Sa[k + 1] - m_safe);
+                    psum += e0 + e1;
+                    pw[k / 2] = BF16::pack(e0, e1);
+                }
+                l_run = l_run * alpha + psum;
+                if (__any(alpha != 1.0f)) {
+                    // the accumulators live in the accumulation registers, which the vector ALU cannot
+                    // multiply in place: one element at a time through a temporary. The waits cover the
+                    // distance the hardware wants between a matrix instruction and a read of its result
+                    // (and between the write-back and the next matrix instruction).
+                    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                        for (int k = 0; k < 16; k++) {
+                            float tmp;
+                            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                                         : "+a"(O[dt][k]), "=&v"(tmp) : "v"(alpha));
+                        }
+                    }
+                    asm volatile("s_nop 7" ::: "memory");
+                }
+                // ---- O^T += kc^T . P^T: 16 tiles of 32 latent columns, two k-steps of 16 positions ---------
+                const uint4 pb0 = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+                const uint4 pb1 = make_uint4(pw[4], pw[5], pw[6], pw[7]);
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) {
+                    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+                    unsigned char *base = const_cast<unsigned char *>(stage) + ((dt >> 2) << 8);
+                    const s16x4_t a00 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + vr_off[dt & 3][0]));
+                    const s16x4_t a01 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + vr_off[dt & 3][1]));
+                    const s16x4_t a10 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + 16 * KC_ROWB + vr_off[dt & 3][0]));
+                    const s16x4_t a11 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + 16 * KC_ROWB + vr_off[dt & 3][1]));
+                    const uint2 x00 = __builtin_bit_cast(uint2, a00), x01 = __builtin_bit_cast(uint2, a01);
+                    const uint2 x10 = __builtin_bit_cast(uint2, a10), x11 = __builtin_bit_cast(uint2, a11);
+                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8_t, make_uint4(x00.x, x00.y, x01.x, x01.y)),
+                        __builtin_bit_cast(bf16x8_t, pb0), O[dt], 0, 0, 0);
+                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8_t, make_uint4(x10.x, x10.y, x11.x, x11.y)),
+                        __builtin_bit_cast(bf16x8_t, pb1), O[dt], 0, 0, 0);
+                }
+            };
+
+            // ---- pipeline: three steps in flight; every copy is unconditional (steps past the end copy
+            // the last step again into a stage nobody consumes), so the wait counts below are exact
+            const uint32_t last = n_steps - 1;
+            issue(0);
+            issue(min(1u, last));
+            issue(min(2u, last));
+            for (uint32_t step = 0; step < n_steps; step++) {
+                dma_wait<2 * DMA_PER_WAVE>();   // this wave's share of `step` has landed
+                __syncthreads();                // ... and everybody else's; stage (step - 1) % 4 is free
+                issue(min(step + 3, last));
+                compute(step);
+            }
+            dma_wait<0>();
+            __syncthreads();   // nothing in flight, nobody reading: the ring can be reused
+
+            const float l_tot = l_run + __shfl_xor(l_run, 32);
+            if (h_ok) {
+                // O^T lane layout: column = head, register k of tile dt = latent 32 dt + 8 (k / 4) + 4 half + k % 4
+                const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head;
+                if (single) {
+                    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+                    uint16_t *dst = p.out + rh * C;
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                        for (int kg = 0; kg < 4; kg++) {
+                            uint2 o;
+                            o.x = BF16::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
+                            o.y = BF16::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
+                            *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
+                        }
+                    }
+                } else {
+                    const uint64_t slot = rh * p.max_slots + tile;
+                    float *dst = p.part_acc + slot * C;
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                        for (int kg = 0; kg < 4; kg++) {
+                            *reinterpret_cast<float4 *>(dst + dt * 32 + kg * 8 + half * 4) =
+                                make_float4(O[dt][kg * 4], O[dt][kg * 4 + 1], O[dt][kg * 4 + 2], O[dt][kg * 4 + 3]);
+                        }
+                    }
+                    if (half == 0) {
+                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+                    }
+                }
+                if (half == 0 && tile == 0 && p.part_cnt != nullptr) {
+                    p.part_cnt[rh] = single ? 0 : static_cast<int32_t>(n_tiles);
+                }
+            }
+        }
+        __syncthreads();  // tbl_lds is rewritten for the next query row
+    }
+}
+
+}  // namespace
+
+bool mla_decode_supported(const MlaArgs &a)
+{
+    const bool dense = a.block_tables == nullptr;
+    return a.total_tokens == a.batch && a.kv_lora_rank == C && a.rope_head_dim == R && a.top_k == 0 &&
+           (dense || a.block_size % kStep == 0);
+}
+
+void mla_decode_plan(const MlaArgs &a, uint32_t *tile_tokens, uint32_t *max_slots)
+{
+    const bool dense = a.block_tables == nullptr;
+    const uint64_t max_ctx = dense ? a.dense_len : static_cast<uint64_t>(a.max_num_blocks) * a.block_size;
+    // about one workgroup per compute unit if every sequence were as long as allowed; tiles between
+    // 256 and 1024 positions
+    uint64_t tile = max_ctx * a.batch / 256;
+    tile = tile > 1024 ? 1024 : (tile < 256 ? 256 : tile);
+    tile = (tile + kStep - 1) / kStep * kStep;
+    *tile_tokens = static_cast<uint32_t>(tile);
+    *max_slots = static_cast<uint32_t>((max_ctx + tile - 1) / tile);
+}
+
+size_t mla_decode_workspace_bytes(const MlaArgs &a)
+{
+    uint32_t tile, max_slots;
+    mla_decode_plan(a, &tile, &max_slots);
+    return max_slots > 1 ? partial_bytes(a.total_tokens, a.n_heads, C, max_slots) : 0;
+}
+
+int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
+{
+    uint32_t tile, max_slots;
+    mla_decode_plan(a, &tile, &max_slots);
+    const size_t need = mla_decode_workspace_bytes(a);
+    if (max_slots > 1 && (a.workspace == nullptr || a.workspace_bytes < need)) {
+        return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
+                                                    " bytes, have " + std::to_string(a.workspace_bytes));
+    }
+    const PartialBuffers pb = max_slots > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, C, max_slots)
+                                            : PartialBuffers{};
+    MlaDecodeParams p{};
+    p.q_absorb = static_cast<const uint16_t *>(a.q_absorb);
+    p.qr = static_cast<const uint16_t *>(a.qr);
+    p.k_cache = static_cast<const uint16_t *>(a.k_cache);
+    p.pe_cache = static_cast<const uint16_t *>(a.pe_cache);
+    p.out = static_cast<uint16_t *>(a.o_absorb);
+    p.query_start_loc = a.query_start_loc;
+    p.lens = a.lens;
+    p.cached_lens = a.cached_lens;
+    p.block_tables = a.block_tables;
+    p.part_cnt = pb.cnt;
+    p.part_acc = pb.acc;
+    p.part_ml = pb.ml;
+    p.n_heads = a.n_heads;
+    p.block_size = a.block_size;
+    p.max_num_blocks = a.max_num_blocks;
+    p.dense_len = a.dense_len;
+    p.tile_tokens = tile;
+    p.max_slots = max_slots;
+    p.scale_log2e = a.scale * kLog2e;
+
+    const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + (tile / 16 + 2) * sizeof(uint32_t);
+    static bool configured = false;
+    if (!configured) {
+        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mla_decode_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        configured = true;
+    }
+    dim3 grid(max_slots, a.batch, 1);
+    mla_decode_kernel<<<grid, kNT, lds, stream>>>(p);
+    XL_LAUNCH_CHECK();
+    if (max_slots == 1) {
+        return XLITE_HIP_OK;
+    }
+    return launch_merge(stream, a.dtype, a.o_absorb, pb, a.total_tokens, a.n_heads, C, max_slots);
+}
+
+}  // namespace xlite
