@@ -22,6 +22,10 @@ import time
 
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
+# script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
+# where no counter run has been taken.
+MEASURED_TRAFFIC_BYTES = {"c2": 1080422086, "c4": 335656121}
 
 
 def _events(torch):
@@ -154,8 +158,9 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
-        "roofline": {"bound": "hbm", "kernel": "decode_kernel", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "decode_mfma_kernel (+ merge_kernel)", "achieved": round(achieved, 2),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name.split()[0]),
                      "algorithmic_bytes_per_launch": int(alg_bytes)},
         "cpu_baseline": cpu,
     }
@@ -227,8 +232,8 @@ def bench_mla(args, torch, rt):
             "config": {"workload": "c4 deepseek-r1 MLA absorbed decode", "batch": 32, "n_heads": 128, "ctx_total": int(sum(ctx)),
                        "kv_bytes_per_step": int(w["kv_bytes"]), "flops_per_step": int(w["flops"])},
             "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1),
-            "roofline": {"bound": "hbm", "kernel": "mfma_attention_kernel", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c4"),
                          "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
             "cpu_baseline": None}
 
@@ -240,6 +245,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB device-to-device copy kernel: under a counter run its "
+                         "FETCH_SIZE / WRITE_SIZE readings give the scale of those counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's share only (no collectives, no sharding); run with --gpus 1",
@@ -252,6 +260,13 @@ def main():
     from gvirt_amd import workloads as W
     from gvirt_amd._C import Runtime
     rt = Runtime(0, 64)
+
+    if args.calibrate_copy:
+        src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        dst.copy_(src)   # one elementwise copy kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     todo = ["c2", "c1", "c5", "c3", "c4"] if args.config == "all" else [args.config]
     for c in todo:
