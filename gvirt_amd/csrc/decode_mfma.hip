@@ -489,6 +489,265 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same computation for the common shape (head_dim 128, 16-bit cache, kv heads a multiple of 8)
+// with the cache copied straight from global memory into LDS (global_load_lds_dwordx4): no staging
+// registers, no LDS store instructions, and a deeper queue of outstanding memory requests. A copy
+// instruction moves 1 KiB of consecutive cache bytes (one position, four kv heads) to 1 KiB of
+// consecutive LDS, so a stage is position major: [K | V][16 positions][8 kv heads][256 bytes]. The
+// 16-byte chunks of a row are XOR-swizzled by the position (the lane picks which global chunk lands
+// in its LDS slot), which keeps both read shapes conflict free exactly as in the kernel above.
+// Two stages of 64 KiB; a step's copies are issued as soon as every wave has finished with the stage.
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void dma_1k(uint32_t lds_addr, uint32_t voff, const void *base)
+{
+    // the compiler sees neither the LDS write nor the memory counter: completion is awaited by dma_wait
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                 :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kWaves * 64)
+decode_dma_kernel(const DecodeMfmaParams p)
+{
+    constexpr int D = 128;
+    constexpr int KS = D / 32, MT = D / 16;
+    constexpr int HEADB = D * 2;                 // bytes of one (position, kv head) row
+    constexpr int POSB = kWaves * HEADB;         // LDS bytes of one position: the 8 kv heads of the pass
+    constexpr int KBYTES = kStep * POSB;         // 32 KiB: the K half of a stage
+    constexpr int STAGE = 2 * KBYTES;
+    constexpr int PER_WAVE = 8;                  // copies per wave and step
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE);
+    const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
+        static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t tile = blockIdx.x;
+    const uint32_t seq = blockIdx.y;
+    const uint32_t col = lane & 15;
+    const uint32_t jq = lane >> 4;
+
+    // read roles (this wave's kv head = `wave` inside the pass)
+    uint32_t kr_off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        kr_off[ks] = col * POSB + wave * HEADB + (((4 * ks + jq) ^ swizzle<D>(col)) << 4);
+    }
+    uint32_t vr_off[MT];
+    {
+        const uint32_t pos = 4 * jq + (col >> 2);
+        const uint32_t q4 = lane & 3;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            vr_off[mt] = KBYTES + pos * POSB + wave * HEADB + (((2 * mt + (q4 >> 1)) ^ swizzle<D>(pos)) << 4) + ((q4 & 1) << 3);
+        }
+    }
+    // copy roles: wave w moves positions 2w and 2w+1, each as two copies of four kv heads, for K and V.
+    // Lane = (kv head inside the four) * 16 + chunk slot; the slot receives chunk slot ^ pattern(position).
+    uint32_t c_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        c_voff[i] = (lane >> 4) * HEADB + (((lane & 15u) ^ swizzle<D>(2 * wave + i)) << 4);
+    }
+
+    const int32_t qlen = p.lens[seq];
+    const int32_t clen = p.cached_lens[seq];
+    const int32_t qstart = p.query_start_loc[seq];
+    const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
+    const uint32_t g_valid = p.group < 16 ? p.group : 16;
+    const uint32_t row_bytes = p.n_kv_heads * HEADB;
+
+    for (int32_t r = 0; r < qlen; r++) {
+        const uint32_t tok = static_cast<uint32_t>(qstart + r);
+        const uint32_t limit = static_cast<uint32_t>(clen + r + 1);
+        const uint32_t n_tiles = ceil_div(limit, p.tile_tokens);
+        if (tile >= n_tiles) {
+            continue;
+        }
+        const uint32_t t0 = tile * p.tile_tokens;
+        const uint32_t t1 = min(limit, t0 + p.tile_tokens);
+        const bool single = n_tiles == 1;
+        const uint32_t n_steps = ceil_div(t1 - t0, kStep);
+        const uint32_t blk0 = t0 / p.block_size;
+        {
+            const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
+            for (uint32_t i = threadIdx.x; i < nblk; i += kWaves * 64) {
+                tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
+            }
+            __syncthreads();
+        }
+
+        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += kWaves) {
+            const uint32_t kvh = kv0 + wave;
+            const uint32_t head0 = kvh * p.group;
+
+            uint4 qreg[KS];
+            {
+                const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride + static_cast<uint64_t>(head0 + col) * D;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8) : make_uint4(0, 0, 0, 0);
+                }
+                // complete these loads before any copy is issued: memory operations finish in order
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+                }
+            }
+            f32x4_t O[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                O[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            }
+            float m_run = -INFINITY, l_run = 0.f;
+
+            // copies of one step into stage step % 2. The 16 positions of a step share one block
+            // (block_size % 16 == 0). Positions at or beyond the end re-read the last valid one.
+            auto issue = [&](uint32_t step) {
+                const uint32_t ts = t0 + step * kStep;
+                const uint32_t blk = ts / p.block_size, off = ts % p.block_size;
+                const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
+                const uint64_t row0 = static_cast<uint64_t>(phys) * p.block_size + off;
+                const uint32_t last_pos = min(t1 - 1 - ts, static_cast<uint32_t>(kStep - 1));
+                const uint32_t st = smem_addr + (step & 1) * STAGE;
+                const char *kb = static_cast<const char *>(p.k_cache) + row0 * row_bytes + kv0 * HEADB;
+                const char *vb = static_cast<const char *>(p.v_cache) + row0 * row_bytes + kv0 * HEADB;
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const uint32_t pos = 2 * wave + i;
+                    const uint32_t src = min(pos, last_pos) * row_bytes;   // uniform
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        dma_1k(st + pos * POSB + j * 1024, c_voff[i], kb + src + j * 1024);
+                        dma_1k(st + KBYTES + pos * POSB + j * 1024, c_voff[i], vb + src + j * 1024);
+                    }
+                }
+            };
+            auto compute = [&](uint32_t step) {
+                const uint32_t t = t0 + step * kStep;
+                const unsigned char *stage = smem + (step & 1) * STAGE;
+                f32x4_t S = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(stage + kr_off[ks]);
+                    S = Mfma16<T>::run(a, qreg[ks], S);
+                }
+                s16x4_t vt[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+                    vt[mt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(const_cast<unsigned char *>(stage) + vr_off[mt]));
+                }
+                float mx = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float v = S[e] * kLog2e;
+                    v = (t + 4 * jq + e) < t1 ? v : -INFINITY;
+                    S[e] = v;
+                    mx = fmaxf(mx, v);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                const float m_new = fmaxf(m_run, mx);
+                const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = fast_exp2(m_run - m_safe);
+                m_run = m_new;
+                float pe[4];
+                float psum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    pe[e] = fast_exp2(S[e] - m_safe);
+                    psum += pe[e];
+                }
+                l_run = l_run * alpha + psum;
+                const uint2 pb = make_uint2(T::pack(pe[0], pe[1]), T::pack(pe[2], pe[3]));
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        O[mt][0] *= alpha;
+                        O[mt][1] *= alpha;
+                        O[mt][2] *= alpha;
+                        O[mt][3] *= alpha;
+                    }
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    O[mt] = Mfma16<T>::run16(vt[mt], pb, O[mt]);
+                }
+            };
+
+            // every copy is unconditional (steps past the end copy the last step again, into the stage
+            // nobody reads any more), so the wait counts are exact
+            const uint32_t last = n_steps - 1;
+            issue(0);
+            issue(min(1u, last));
+            for (uint32_t step = 0; step < n_steps; step++) {
+                dma_wait<PER_WAVE>();   // this wave's share of `step` has landed
+                __syncthreads();        // ... and everybody else's
+                compute(step);
+                __syncthreads();        // the stage is free again
+                issue(min(step + 2, last));
+            }
+            dma_wait<0>();
+            __syncthreads();
+
+            float l_tot = l_run + __shfl_xor(l_run, 16);
+            l_tot += __shfl_xor(l_tot, 32);
+            if (col < g_valid) {
+                if (single) {
+                    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+                    uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        uint2 o;
+                        o.x = T::pack(O[mt][0] * inv, O[mt][1] * inv);
+                        o.y = T::pack(O[mt][2] * inv, O[mt][3] * inv);
+                        *reinterpret_cast<uint2 *>(dst + mt * 16 + jq * 4) = o;
+                    }
+                } else {
+                    const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * p.max_slots + tile;
+                    float *dst = p.part_acc + slot * D;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
+                    }
+                    if (jq == 0) {
+                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+                    }
+                }
+                if (jq == 0 && tile == 0 && p.part_cnt != nullptr) {
+                    p.part_cnt[static_cast<uint64_t>(tok) * p.n_heads + head0 + col] = single ? 0 : static_cast<int32_t>(n_tiles);
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
+{
+    const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) + (p.tile_tokens / kStep + 2) * sizeof(uint32_t);
+    auto kernel = decode_dma_kernel<T>;
+    static size_t configured = 0;
+    if (configured < lds) {
+        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        configured = lds;
+    }
+    dim3 grid(p.max_slots, batch, 1);
+    kernel<<<grid, kWaves * 64, lds, stream>>>(p);
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
 template <typename T, int D, bool KV8, bool MULTI_SUB>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
 {
@@ -586,7 +845,9 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
     const bool bf = a.dtype == XLITE_HIP_BF16;
     int rc;
-    if (a.head_dim == 128) {
+    if (a.head_dim == 128 && !kv8 && a.n_kv_heads % kWaves == 0) {
+        rc = bf ? launch_dma<BF16>(stream, p, a.batch) : launch_dma<FP16>(stream, p, a.batch);
+    } else if (a.head_dim == 128) {
         if (bf) {
             rc = kv8 ? launch_one<BF16, 128, true>(stream, p, a.batch) : launch_one<BF16, 128, false>(stream, p, a.batch);
         } else {
