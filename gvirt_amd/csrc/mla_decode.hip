@@ -29,6 +29,7 @@ constexpr int kWaves = 4;
 constexpr int kNT = kWaves * 64;
 constexpr int kStep = 32;
 constexpr int kStages = 4;
+constexpr int kAhead = 2;               // operand fetches in flight ahead of the matrix instruction using them
 constexpr int C = 512;                 // kv_lora_rank
 constexpr int R = 64;                  // rope_head_dim
 constexpr int KS_C = C / 16;           // k-steps over the latent part
@@ -103,36 +104,28 @@ mla_decode_kernel(const MlaDecodeParams p)
 
     // ---- copy roles: wave w moves latent rows w, w+4, .. (lane = chunk slot) and rotary rows
     // 8w .. 8w+7 (lane / 8 = row, lane % 8 = chunk slot); a slot holds chunk (slot ^ pattern(row))
-    uint32_t kc_voff[kStep / kWaves];
-#pragma unroll
-    for (int i = 0; i < kStep / kWaves; i++) {
-        const uint32_t row = wave + kWaves * i;
-        kc_voff[i] = row * KC_ROWB + (((lane & ~15u) | ((lane & 15u) ^ swz_kc(row))) << 4);
-    }
+    // (row = wave + 4 i has pattern 4 wave | i % 4: one lane offset, XORed with 16 (i % 4) per copy)
+    uint32_t kc_voff = ((lane & ~15u) | ((lane & 15u) ^ (wave << 2))) << 4;
     const uint32_t pe_row = wave * 8 + (lane >> 3);
     const uint32_t pe_chunk = (lane & 7u) ^ swz_pe(pe_row);
 
     // ---- read roles --------------------------------------------------------------------------------
     // K rows as the A operand: row = position `col`, chunk 2 ks + half; chunk' = 2 ks ^ x
-    const uint32_t kx = (half ^ swz_kc(col)) << 4;                    // latent part, low 8 address bits
-    const uint32_t px = (half ^ swz_pe(col)) << 4;                    // rotary part, low 7 address bits
+    uint32_t kx = (half ^ swz_kc(col)) << 4;                    // latent part, low 8 address bits
+    uint32_t px = (half ^ swz_pe(col)) << 4;                    // rotary part, low 7 address bits
     const uint32_t k_row = col * KC_ROWB;
     const uint32_t p_row = KC_BYTES + col * PE_ROWB;
     // transposed latent: 16-lane group g = lane / 16 covers columns 16 (g % 2) .. +16 of a 32-column
     // tile for the positions of half g / 2; lane 4 j' + q points at elements [4 q, +4) of position
     // 4 half + j' (+8 for the second read, +16 for the second k-step)
-    uint32_t vr_off[4][2];
+    // The offsets of tile a = dt % 4 and of the second read differ from vr_off by XOR constants
+    // (64 a, and 32 plus 8 rows); a tile's 256-byte group and the second k-step are immediates.
+    uint32_t vr_off;
     {
         const uint32_t g = lane >> 4, jp = (lane & 15) >> 2, q = lane & 3;
         const uint32_t y = 2 * (g & 1) + (q >> 1);
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-#pragma unroll
-            for (int rd = 0; rd < 2; rd++) {
-                const uint32_t pos = 4 * (g >> 1) + jp + 8 * rd;
-                vr_off[a][rd] = pos * KC_ROWB + ((((4 * a + y) & 15u) ^ swz_kc(pos)) << 4) + ((q & 1) << 3);
-            }
-        }
+        const uint32_t pos = 4 * (g >> 1) + jp;
+        vr_off = pos * KC_ROWB + ((y ^ swz_kc(pos)) << 4) + ((q & 1) << 3);
     }
 
     const int32_t qlen = p.lens[seq];
@@ -166,24 +159,36 @@ mla_decode_kernel(const MlaDecodeParams p)
         for (uint32_t h0 = 0; h0 < p.n_heads; h0 += 32 * kWaves) {
             const uint32_t head = h0 + wave * 32 + col;
             const bool h_ok = head < p.n_heads;
+            unsigned char *my_stage = smem + wave * STAGE_BYTES;   // private to the wave outside the loop
 
-            // ---- [q_absorb | qr] as the B operand: column = head, 8 consecutive elements per half
+            // ---- [q_absorb | qr] of this wave's 32 heads: copied into the wave's stage with the layout of
+            // a cache step (head = row), then read as the B operand (column = head, 8 elements per half).
+            // Heads past the end repeat the last one; their results are never stored.
             uint4 qreg[KS_C + KS_R];
             {
-                const uint16_t *qa = p.q_absorb + (static_cast<uint64_t>(tok) * p.n_heads + head) * C;
-                const uint16_t *qq = p.qr + (static_cast<uint64_t>(tok) * p.n_heads + head) * R;
+                const uint32_t st = smem_addr + wave * STAGE_BYTES;
+                const uint32_t h_last = p.n_heads - 1;
+                const char *qa = reinterpret_cast<const char *>(p.q_absorb) + static_cast<uint64_t>(tok) * p.n_heads * KC_ROWB;
+                const char *qq = reinterpret_cast<const char *>(p.qr) + static_cast<uint64_t>(tok) * p.n_heads * PE_ROWB;
 #pragma unroll
-                for (int ks = 0; ks < KS_C + KS_R; ks++) {
-                    const int e0 = ks * 16 + half * 8;
-                    qreg[ks] = !h_ok ? make_uint4(0, 0, 0, 0)
-                               : (ks < KS_C ? *reinterpret_cast<const uint4 *>(qa + e0)
-                                            : *reinterpret_cast<const uint4 *>(qq + (e0 - C)));
+                for (int row = 0; row < 32; row++) {
+                    const uint32_t hr = min(h0 + wave * 32 + row, h_last);
+                    dma_1k(st + row * KC_ROWB, ((lane & ~15u) | ((lane & 15u) ^ swz_kc(row))) << 4, qa + static_cast<uint64_t>(hr) * KC_ROWB);
                 }
-                // consume the registers now: all memory loads the compiler knows of are then complete,
-                // and it never waits on vmcnt inside the streaming loop (where the copies are in flight)
 #pragma unroll
-                for (int ks = 0; ks < KS_C + KS_R; ks++) {
-                    asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t row = i * 8 + (lane >> 3);
+                    const uint32_t hr = min(h0 + wave * 32 + row, h_last);
+                    dma_1k(st + KC_BYTES + i * 1024, hr * PE_ROWB + (((lane & 7u) ^ swz_pe(row)) << 4), qq);
+                }
+                dma_wait<0>();
+#pragma unroll
+                for (int ks = 0; ks < KS_C; ks++) {
+                    qreg[ks] = *reinterpret_cast<const uint4 *>(my_stage + k_row + ((ks >> 3) << 8) + ((((2 * ks) & 15) << 4) ^ kx));
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS_R; ks++) {
+                    qreg[KS_C + ks] = *reinterpret_cast<const uint4 *>(my_stage + p_row + ((((2 * ks) & 7) << 4) ^ px));
                 }
             }
             f32x16_t O[DT];
@@ -195,11 +200,16 @@ mla_decode_kernel(const MlaDecodeParams p)
                 }
             }
             float m_run = -INFINITY, l_run = 0.f;
+            __syncthreads();   // every wave holds its Q: the stages may be overwritten
 
-            // first cache row of a step: its 32 positions share one block (block_size % 32 == 0)
-            auto issue = [&](uint32_t step) {
+            // ---- cache copies of one step: scalars first, then nine 1 KiB copies per wave ----------------
+            struct StepCopy {
+                const char *kb, *pb;
+                uint32_t stage, last_pos;
+            };
+            auto plan = [&](uint32_t step) {
                 const uint32_t ts = t0 + step * kStep;
-                uint64_t row0;
+                uint64_t row0;   // first cache row: the 32 positions share one block (block_size % 32 == 0)
                 if (dense) {
                     row0 = static_cast<uint64_t>(seq) * p.dense_len + ts;
                 } else {
@@ -207,58 +217,98 @@ mla_decode_kernel(const MlaDecodeParams p)
                     const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
                     row0 = static_cast<uint64_t>(phys) * p.block_size + off;
                 }
+                StepCopy c;
                 // positions at or beyond the end re-read the last valid one: finite values whose
                 // probabilities are forced to zero
-                const uint32_t last_pos = min(t1 - 1 - ts, static_cast<uint32_t>(kStep - 1));
-                const uint32_t stage = smem_addr + (step % kStages) * STAGE_BYTES;
-                const char *kb = reinterpret_cast<const char *>(p.k_cache) + row0 * KC_ROWB;
-                const char *pb = reinterpret_cast<const char *>(p.pe_cache) + row0 * PE_ROWB;
-#pragma unroll
-                for (int i = 0; i < kStep / kWaves; i++) {
+                c.last_pos = min(t1 - 1 - ts, static_cast<uint32_t>(kStep - 1));
+                c.stage = smem_addr + (step % kStages) * STAGE_BYTES;
+                c.kb = reinterpret_cast<const char *>(p.k_cache) + row0 * KC_ROWB;
+                c.pb = reinterpret_cast<const char *>(p.pe_cache) + row0 * PE_ROWB;
+                return c;
+            };
+            auto copy_piece = [&](const StepCopy &c, int i) {
+                if (i < kStep / kWaves) {
                     const uint32_t row = wave + kWaves * i;
-                    const uint32_t back = row > last_pos ? (row - last_pos) * KC_ROWB : 0u;   // uniform
-                    dma_1k(stage + row * KC_ROWB, kc_voff[i], kb - back);
+                    const uint32_t back = row > c.last_pos ? (row - c.last_pos) * KC_ROWB : 0u;   // uniform
+                    dma_1k(c.stage + row * KC_ROWB, kc_voff ^ ((i & 3) << 4), c.kb + row * KC_ROWB - back);
+                } else {
+                    const uint32_t prow = min(pe_row, c.last_pos);
+                    dma_1k(c.stage + KC_BYTES + wave * 1024, prow * PE_ROWB + (pe_chunk << 4), c.pb);
                 }
-                const uint32_t prow = min(pe_row, last_pos);
-                dma_1k(stage + KC_BYTES + wave * 1024, prow * PE_ROWB + (pe_chunk << 4), pb);
+            };
+            auto issue = [&](uint32_t step) {
+                const StepCopy c = plan(step);
+#pragma unroll
+                for (int i = 0; i < DMA_PER_WAVE; i++) {
+                    copy_piece(c, i);
+                }
             };
 
-            auto compute = [&](uint32_t step) {
-                const uint32_t t = t0 + step * kStep;
+            // ---- S^T = K . Q^T of one step: 32 positions x 32 heads; operands are fetched three ahead -----
+            auto rd_k = [&](const unsigned char *stage, int ks) {
+                return ks < KS_C
+                    ? *reinterpret_cast<const uint4 *>(stage + k_row + ((ks >> 3) << 8) + ((((2 * ks) & 15) << 4) ^ kx))
+                    : *reinterpret_cast<const uint4 *>(stage + p_row + ((((2 * (ks - KS_C)) & 7) << 4) ^ px));
+            };
+            // `between(ks)` is vector-ALU work placed behind the ks-th matrix instruction, which it does not
+            // depend on: it runs while the matrix pipe is busy. The fences keep that order.
+            auto qk = [&](uint32_t step, auto &&between) {
                 const unsigned char *stage = smem + (step % kStages) * STAGE_BYTES;
-                // ---- S^T = K . Q^T: 32 positions x 32 heads, -----------------------------------------
-                f32x16_t Sa;
+                f32x16_t S;
 #pragma unroll
                 for (int k = 0; k < 16; k++) {
-                    Sa[k] = 0.f;
+                    S[k] = 0.f;
+                }
+                uint4 a[kAhead];
+#pragma unroll
+                for (int i = 0; i < kAhead; i++) {
+                    a[i] = rd_k(stage, i);
                 }
 #pragma unroll
-                for (int ks = 0; ks < KS_C; ks++) {
-                    const uint32_t off = k_row + ((ks >> 3) << 8) + ((((2 * ks) & 15) << 4) ^ kx);
-                    const uint4 a = *reinterpret_cast<const uint4 *>(stage + off);
-                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                                 __builtin_bit_cast(bf16x8_t, qreg[ks]), Sa, 0, 0, 0);
+                for (int ks = 0; ks < KS_C + KS_R; ks++) {
+                    S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[ks % kAhead]),
+                                                                __builtin_bit_cast(bf16x8_t, qreg[ks]), S, 0, 0, 0);
+                    if (ks + kAhead < KS_C + KS_R) {
+                        a[ks % kAhead] = rd_k(stage, ks + kAhead);
+                    }
+                    between(ks);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-#pragma unroll
-                for (int ks = 0; ks < KS_R; ks++) {
-                    const uint32_t off = p_row + ((((2 * ks) & 7) << 4) ^ px);
-                    const uint4 a = *reinterpret_cast<const uint4 *>(stage + off);
-                    Sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                                 __builtin_bit_cast(bf16x8_t, qreg[KS_C + ks]), Sa, 0, 0, 0);
-                }
-                // ---- online softmax; register k holds position t + 8 (k / 4) + 4 half + k % 4 ---------------
+                return S;
+            };
+
+            // ---- pipeline: copies run three steps ahead of the step being consumed. Every copy is
+            // unconditional (steps past the end copy the last step again, same bytes to the same place), so
+            // the wait counts are exact.
+            const uint32_t last = n_steps - 1;
+            issue(0);
+            issue(min(1u, last));
+            issue(min(2u, last));
+            for (uint32_t step = 0; step < n_steps; step++) {
+                const uint32_t t = t0 + step * kStep;
+                // keep the offsets derived from these out of loop-invariant registers: there are none to spare
+                asm volatile("" : "+v"(kx), "+v"(px), "+v"(vr_off), "+v"(kc_voff));
+                dma_wait<2 * DMA_PER_WAVE>();   // this wave's share of `step` has landed
+                __syncthreads();            // ... and everybody else's; stage (step - 1) % 4 is free
+
+                // ---- scores, then the online softmax. Register k holds position t + 8 (k / 4) + 4 half +
+                // k % 4. The reference maximum only moves when the step maximum exceeds it by more than
+                // 2^8: probabilities then stay below 2^8 (the same relative precision in bf16, and the
+                // normaliser shares the reference), and the accumulators are rescaled rarely.
+                f32x16_t S = qk(step, [](int) {});
+                const uint32_t lane_pos = t + half * 4;
                 float mx = -INFINITY;
 #pragma unroll
                 for (int k = 0; k < 16; k++) {
-                    const uint32_t pos = t + (k / 4) * 8 + half * 4 + (k % 4);
-                    const float v = pos < t1 ? Sa[k] * p.scale_log2e : -INFINITY;
-                    Sa[k] = v;
+                    const uint32_t pos = lane_pos + (k / 4) * 8 + (k % 4);
+                    const float v = pos < t1 ? S[k] * p.scale_log2e : -INFINITY;
+                    S[k] = v;
                     mx = fmaxf(mx, v);
                 }
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-                // the reference maximum only moves when the step maximum exceeds it by more than 2^8:
-                // probabilities then stay below 2^8 (exact in bf16 to the same relative precision, and the
-                // normaliser shares the reference), and the accumulators are rescaled rarely
+                {
+                    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+                    mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                }
                 const float m_new = mx > m_run + kRescaleSlack ? mx : m_run;
                 const float m_safe = m_new == -INFINITY ? 0.f : m_new;
                 const float alpha = fast_exp2(m_run - m_safe);
@@ -267,12 +317,13 @@ mla_decode_kernel(const MlaDecodeParams p)
                 float psum = 0.f;
 #pragma unroll
                 for (int k = 0; k < 16; k += 2) {
-                    const float e0 = fast_exp2(Sa[k] - m_safe);
-                    const float e1 = fast_exp2(Sa[k + 1] - m_safe);
+                    const float e0 = fast_exp2(S[k] - m_safe);
+                    const float e1 = fast_exp2(S[k + 1] - m_safe);
                     psum += e0 + e1;
                     pw[k / 2] = BF16::pack(e0, e1);
                 }
                 l_run = l_run * alpha + psum;
+
                 if (__any(alpha != 1.0f)) {
                     // the accumulators live in the accumulation registers, which the vector ALU cannot
                     // multiply in place: one element at a time through a temporary. The waits cover the
@@ -290,81 +341,96 @@ mla_decode_kernel(const MlaDecodeParams p)
                     }
                     asm volatile("s_nop 7" ::: "memory");
                 }
-                // ---- O^T += kc^T . P^T: 16 tiles of 32 latent columns, two k-steps of 16 positions ---------
-                const uint4 pb0 = make_uint4(pw[0], pw[1], pw[2], pw[3]);
-                const uint4 pb1 = make_uint4(pw[4], pw[5], pw[6], pw[7]);
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++) {
-                    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
-                    unsigned char *base = const_cast<unsigned char *>(stage) + ((dt >> 2) << 8);
-                    const s16x4_t a00 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + vr_off[dt & 3][0]));
-                    const s16x4_t a01 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + vr_off[dt & 3][1]));
-                    const s16x4_t a10 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + 16 * KC_ROWB + vr_off[dt & 3][0]));
-                    const s16x4_t a11 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + 16 * KC_ROWB + vr_off[dt & 3][1]));
-                    const uint2 x00 = __builtin_bit_cast(uint2, a00), x01 = __builtin_bit_cast(uint2, a01);
-                    const uint2 x10 = __builtin_bit_cast(uint2, a10), x11 = __builtin_bit_cast(uint2, a11);
-                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8_t, make_uint4(x00.x, x00.y, x01.x, x01.y)),
-                        __builtin_bit_cast(bf16x8_t, pb0), O[dt], 0, 0, 0);
-                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8_t, make_uint4(x10.x, x10.y, x11.x, x11.y)),
-                        __builtin_bit_cast(bf16x8_t, pb1), O[dt], 0, 0, 0);
-                }
-            };
 
-            // ---- pipeline: three steps in flight; every copy is unconditional (steps past the end copy
-            // the last step again into a stage nobody consumes), so the wait counts below are exact
-            const uint32_t last = n_steps - 1;
-            issue(0);
-            issue(min(1u, last));
-            issue(min(2u, last));
-            for (uint32_t step = 0; step < n_steps; step++) {
-                dma_wait<2 * DMA_PER_WAVE>();   // this wave's share of `step` has landed
-                __syncthreads();                // ... and everybody else's; stage (step - 1) % 4 is free
-                issue(min(step + 3, last));
-                compute(step);
+                // ---- O^T += kc^T . P^T: 16 tiles of 32 latent columns, two k-steps of 16 positions; the
+                // transposed operands of the next tile are fetched before this tile's products, and the
+                // copies of step + 3 are issued in between
+                {
+                    const StepCopy c = plan(min(step + 3, last));
+                    unsigned char *stage = smem + (step % kStages) * STAGE_BYTES;
+                    const uint4 pb0 = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+                    const uint4 pb1 = make_uint4(pw[4], pw[5], pw[6], pw[7]);
+                    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+                    auto rd_v = [&](int dt, int kk, int rd) {
+                        unsigned char *ptr = stage + ((dt >> 2) << 8) + kk * 16 * KC_ROWB + rd * 8 * KC_ROWB +
+                                             (vr_off ^ (((dt & 3) << 6) | (rd << 5)));
+                        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
+                    };
+                    uint2 v[2][4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        v[0][j] = rd_v(0, j >> 1, j & 1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+                        if (dt + 1 < DT) {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                v[(dt + 1) & 1][j] = rd_v(dt + 1, j >> 1, j & 1);
+                            }
+                        }
+                        const uint2 *x = v[dt & 1];
+                        O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8_t, make_uint4(x[0].x, x[0].y, x[1].x, x[1].y)),
+                            __builtin_bit_cast(bf16x8_t, pb0), O[dt], 0, 0, 0);
+                        O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8_t, make_uint4(x[2].x, x[2].y, x[3].x, x[3].y)),
+                            __builtin_bit_cast(bf16x8_t, pb1), O[dt], 0, 0, 0);
+                        if (dt < DMA_PER_WAVE) {
+                            copy_piece(c, dt);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
             }
             dma_wait<0>();
             __syncthreads();   // nothing in flight, nobody reading: the ring can be reused
 
+            // ---- results: O^T lane layout is column = head, register k of tile dt = latent
+            // 32 dt + 8 (k / 4) + 4 half + k % 4. Transposed through the wave's stage, 256 latent columns at a
+            // time, so that every store instruction writes one head's contiguous row segment.
             const float l_tot = l_run + __shfl_xor(l_run, 32);
-            if (h_ok) {
-                // O^T lane layout: column = head, register k of tile dt = latent 32 dt + 8 (k / 4) + 4 half + k % 4
-                const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head;
-                if (single) {
-                    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-                    uint16_t *dst = p.out + rh * C;
+            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            constexpr int TR_ROWB = 256 * 4 + 16;
+            const uint32_t heads_here = min(32u, p.n_heads > h0 + wave * 32 ? p.n_heads - (h0 + wave * 32) : 0u);
+            const uint64_t rh0 = static_cast<uint64_t>(tok) * p.n_heads + h0 + wave * 32;
 #pragma unroll
-                    for (int dt = 0; dt < DT; dt++) {
+            for (int ch = 0; ch < 2; ch++) {
 #pragma unroll
-                        for (int kg = 0; kg < 4; kg++) {
-                            uint2 o;
-                            o.x = BF16::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
-                            o.y = BF16::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
-                            *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
-                        }
-                    }
-                } else {
-                    const uint64_t slot = rh * p.max_slots + tile;
-                    float *dst = p.part_acc + slot * C;
+                for (int d8 = 0; d8 < 8; d8++) {
+                    const int dt = ch * 8 + d8;
 #pragma unroll
-                    for (int dt = 0; dt < DT; dt++) {
-#pragma unroll
-                        for (int kg = 0; kg < 4; kg++) {
-                            *reinterpret_cast<float4 *>(dst + dt * 32 + kg * 8 + half * 4) =
-                                make_float4(O[dt][kg * 4], O[dt][kg * 4 + 1], O[dt][kg * 4 + 2], O[dt][kg * 4 + 3]);
-                        }
-                    }
-                    if (half == 0) {
-                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+                    for (int kg = 0; kg < 4; kg++) {
+                        const float sc = single ? inv : 1.0f;
+                        *reinterpret_cast<float4 *>(my_stage + col * TR_ROWB + (d8 * 32 + kg * 8 + half * 4) * 4) =
+                            make_float4(O[dt][kg * 4] * sc, O[dt][kg * 4 + 1] * sc, O[dt][kg * 4 + 2] * sc, O[dt][kg * 4 + 3] * sc);
                     }
                 }
-                if (half == 0 && tile == 0 && p.part_cnt != nullptr) {
+                // wave-private region: the LDS counter wait the compiler inserts is all the ordering needed
+                for (uint32_t hr = 0; hr < heads_here; hr++) {
+                    const float4 x = *reinterpret_cast<const float4 *>(my_stage + hr * TR_ROWB + lane * 16);
+                    if (single) {
+                        uint2 o;
+                        o.x = BF16::pack(x.x, x.y);
+                        o.y = BF16::pack(x.z, x.w);
+                        *reinterpret_cast<uint2 *>(p.out + (rh0 + hr) * C + ch * 256 + lane * 4) = o;
+                    } else {
+                        *reinterpret_cast<float4 *>(p.part_acc + ((rh0 + hr) * p.max_slots + tile) * C + ch * 256 + lane * 4) = x;
+                    }
+                }
+            }
+            if (h_ok && half == 0) {
+                const uint64_t rh = rh0 + col;
+                if (!single) {
+                    *reinterpret_cast<float2 *>(p.part_ml + (rh * p.max_slots + tile) * 2) = make_float2(m_run, l_tot);
+                }
+                if (tile == 0 && p.part_cnt != nullptr) {
                     p.part_cnt[rh] = single ? 0 : static_cast<int32_t>(n_tiles);
                 }
             }
+            __syncthreads();   // the stages are reused by the next pass
         }
-        __syncthreads();  // tbl_lds is rewritten for the next query row
     }
 }
 
