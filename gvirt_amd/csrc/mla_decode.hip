@@ -80,6 +80,18 @@ __device__ __forceinline__ void dma_1k(uint32_t lds_addr, uint32_t voff, const v
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
                  :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
+// Four copies whose LDS and global addresses advance by 1 KiB each: the instruction's immediate offset is
+// added to both, so one M0 value and one base serve the four.
+__device__ __forceinline__ void dma_4x1k(uint32_t lds_addr, uint32_t v0, uint32_t v1, uint32_t v2, uint32_t v3,
+                                         const void *base)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %5\n\t"
+                 "global_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\t"
+                 "global_load_lds_dwordx4 %4, %5 offset:3072\n\t"
+                 :: "s"(lds_addr), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(base) : "memory", "m0");
+}
 template <int N>
 __device__ __forceinline__ void dma_wait()
 {
@@ -102,31 +114,34 @@ mla_decode_kernel(const MlaDecodeParams p)
     const uint32_t half = lane >> 5;
     const bool dense = p.block_tables == nullptr;
 
-    // ---- copy roles: wave w moves latent rows w, w+4, .. (lane = chunk slot) and rotary rows
-    // 8w .. 8w+7 (lane / 8 = row, lane % 8 = chunk slot); a slot holds chunk (slot ^ pattern(row))
-    // (row = wave + 4 i has pattern 4 wave | i % 4: one lane offset, XORed with 16 (i % 4) per copy)
-    uint32_t kc_voff = ((lane & ~15u) | ((lane & 15u) ^ (wave << 2))) << 4;
-    const uint32_t pe_row = wave * 8 + (lane >> 3);
-    const uint32_t pe_chunk = (lane & 7u) ^ swz_pe(pe_row);
-
-    // ---- read roles --------------------------------------------------------------------------------
-    // K rows as the A operand: row = position `col`, chunk 2 ks + half; chunk' = 2 ks ^ x
-    uint32_t kx = (half ^ swz_kc(col)) << 4;                    // latent part, low 8 address bits
-    uint32_t px = (half ^ swz_pe(col)) << 4;                    // rotary part, low 7 address bits
-    const uint32_t k_row = col * KC_ROWB;
-    const uint32_t p_row = KC_BYTES + col * PE_ROWB;
-    // transposed latent: 16-lane group g = lane / 16 covers columns 16 (g % 2) .. +16 of a 32-column
-    // tile for the positions of half g / 2; lane 4 j' + q points at elements [4 q, +4) of position
-    // 4 half + j' (+8 for the second read, +16 for the second k-step)
-    // The offsets of tile a = dt % 4 and of the second read differ from vr_off by XOR constants
-    // (64 a, and 32 plus 8 rows); a tile's 256-byte group and the second k-step are immediates.
-    uint32_t vr_off;
-    {
-        const uint32_t g = lane >> 4, jp = (lane & 15) >> 2, q = lane & 3;
+    // ---- per-lane address roles. They are recomputed from the lane index at every step (a dozen vector
+    // instructions) instead of living in a dozen registers for the whole kernel: there are none to spare.
+    // Copy roles: wave w moves latent rows 8w .. 8w+7 (lane = chunk slot) and rotary rows 8w .. 8w+7
+    // (lane / 8 = row, lane % 8 = chunk slot); a slot holds chunk (slot ^ pattern(row)). The pattern of row
+    // 8w + i is 4 (i % 4) | (2w % 4 + i / 4): one lane offset, XORed with a constant per copy.
+    // Read roles: K rows as the A operand (row = position `col`, chunk 2 ks + half, chunk' = 2 ks ^ x);
+    // transposed latent: 16-lane group g = lane / 16 covers columns 16 (g % 2) .. +16 of a 32-column tile
+    // for the positions of half g / 2; lane 4 j' + q points at elements [4 q, +4) of position 4 half + j'
+    // (+8 for the second read, +16 for the second k-step). The offsets of tile a = dt % 4 and of the second
+    // read differ from vr_off by XOR constants (64 a, and 32 plus 8 rows); a tile's 256-byte group and the
+    // second k-step are immediates.
+    uint32_t kc_voff, pe_voff, pe_row, kx, px, k_row, p_row, vr_off, half4;
+    auto set_roles = [&](uint32_t ln) {
+        const uint32_t c5 = ln & 31, hf = ln >> 5;
+        half4 = hf * 4;
+        kc_voff = ((ln & ~15u) | ((ln & 15u) ^ ((2 * wave) & 3))) << 4;
+        pe_row = wave * 8 + (ln >> 3);
+        pe_voff = ((ln & 7u) ^ swz_pe(pe_row)) << 4;
+        kx = (hf ^ swz_kc(c5)) << 4;
+        px = (hf ^ swz_pe(c5)) << 4;
+        k_row = c5 * KC_ROWB;
+        p_row = KC_BYTES + c5 * PE_ROWB;
+        const uint32_t g = ln >> 4, jp = (ln & 15) >> 2, q = ln & 3;
         const uint32_t y = 2 * (g & 1) + (q >> 1);
         const uint32_t pos = 4 * (g >> 1) + jp;
         vr_off = pos * KC_ROWB + ((y ^ swz_kc(pos)) << 4) + ((q & 1) << 3);
-    }
+    };
+    set_roles(lane);
 
     const int32_t qlen = p.lens[seq];
     const int32_t clen = p.cached_lens[seq];
@@ -170,16 +185,31 @@ mla_decode_kernel(const MlaDecodeParams p)
                 const uint32_t h_last = p.n_heads - 1;
                 const char *qa = reinterpret_cast<const char *>(p.q_absorb) + static_cast<uint64_t>(tok) * p.n_heads * KC_ROWB;
                 const char *qq = reinterpret_cast<const char *>(p.qr) + static_cast<uint64_t>(tok) * p.n_heads * PE_ROWB;
+                const uint32_t hw = h0 + wave * 32;
+                if (hw + 32 <= p.n_heads) {
+                    // 32 consecutive heads: 32 KiB and 4 KiB of consecutive memory, four copies per M0 value
+                    const uint32_t lv = lane << 4;
 #pragma unroll
-                for (int row = 0; row < 32; row++) {
-                    const uint32_t hr = min(h0 + wave * 32 + row, h_last);
-                    dma_1k(st + row * KC_ROWB, ((lane & ~15u) | ((lane & 15u) ^ swz_kc(row))) << 4, qa + static_cast<uint64_t>(hr) * KC_ROWB);
-                }
+                    for (int g = 0; g < 8; g++) {
+                        dma_4x1k(st + g * 4 * KC_ROWB, lv ^ (swz_kc(4 * g) << 4), lv ^ (swz_kc(4 * g + 1) << 4),
+                                 lv ^ (swz_kc(4 * g + 2) << 4), lv ^ (swz_kc(4 * g + 3) << 4),
+                                 qa + static_cast<uint64_t>(hw + 4 * g) * KC_ROWB);
+                    }
+                    // rotary rows 8 i + lane / 8: pattern (4 i + lane / 16) % 8, i.e. the lane's own XOR 4 (i % 2)
+                    const uint32_t pv = ((lane >> 3) * PE_ROWB) + (((lane & 7u) ^ ((lane >> 4) & 7u)) << 4);
+                    dma_4x1k(st + KC_BYTES, pv, pv ^ (4u << 4), pv, pv ^ (4u << 4), qq + static_cast<uint64_t>(hw) * PE_ROWB);
+                } else {
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint32_t row = i * 8 + (lane >> 3);
-                    const uint32_t hr = min(h0 + wave * 32 + row, h_last);
-                    dma_1k(st + KC_BYTES + i * 1024, hr * PE_ROWB + (((lane & 7u) ^ swz_pe(row)) << 4), qq);
+                    for (uint32_t row = 0; row < 32; row++) {
+                        const uint32_t hr = min(hw + row, h_last);
+                        dma_1k(st + row * KC_ROWB, ((lane & ~15u) | ((lane & 15u) ^ swz_kc(row))) << 4, qa + static_cast<uint64_t>(hr) * KC_ROWB);
+                    }
+#pragma unroll
+                    for (uint32_t i = 0; i < 4; i++) {
+                        const uint32_t row = i * 8 + (lane >> 3);
+                        const uint32_t hr = min(hw + row, h_last);
+                        dma_1k(st + KC_BYTES + i * 1024, hr * PE_ROWB + (((lane & 7u) ^ swz_pe(row)) << 4), qq);
+                    }
                 }
                 dma_wait<0>();
 #pragma unroll
@@ -226,34 +256,58 @@ mla_decode_kernel(const MlaDecodeParams p)
                 c.pb = reinterpret_cast<const char *>(p.pe_cache) + row0 * PE_ROWB;
                 return c;
             };
-            auto copy_piece = [&](const StepCopy &c, int i) {
-                if (i < kStep / kWaves) {
-                    const uint32_t row = wave + kWaves * i;
-                    const uint32_t back = row > c.last_pos ? (row - c.last_pos) * KC_ROWB : 0u;   // uniform
-                    dma_1k(c.stage + row * KC_ROWB, kc_voff ^ ((i & 3) << 4), c.kb + row * KC_ROWB - back);
-                } else {
+            auto row_xor = [](int i) { return static_cast<uint32_t>(((i & 3) << 6) | ((i >> 2) << 4)); };
+            // piece 0, 1: four latent rows each; piece 2: the rotary rows. A step that ends inside the
+            // tile's last positions takes the general path (piece 0 issues all nine copies).
+            auto copy_piece = [&](const StepCopy &c, int piece) {
+                const bool full = c.last_pos == kStep - 1;
+                if (full) {
+                    if (piece < 2) {
+                        const uint32_t r0 = 8 * wave + 4 * piece;
+                        dma_4x1k(c.stage + r0 * KC_ROWB, kc_voff ^ row_xor(4 * piece), kc_voff ^ row_xor(4 * piece + 1),
+                                 kc_voff ^ row_xor(4 * piece + 2), kc_voff ^ row_xor(4 * piece + 3), c.kb + r0 * KC_ROWB);
+                    } else {
+                        dma_1k(c.stage + KC_BYTES + wave * 1024, pe_row * PE_ROWB + pe_voff, c.pb);
+                    }
+                } else if (piece == 0) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const uint32_t row = 8 * wave + i;
+                        const uint32_t src = min(row, c.last_pos);   // uniform
+                        dma_1k(c.stage + row * KC_ROWB, kc_voff ^ row_xor(i), c.kb + src * KC_ROWB);
+                    }
                     const uint32_t prow = min(pe_row, c.last_pos);
-                    dma_1k(c.stage + KC_BYTES + wave * 1024, prow * PE_ROWB + (pe_chunk << 4), c.pb);
+                    dma_1k(c.stage + KC_BYTES + wave * 1024, prow * PE_ROWB + pe_voff, c.pb);
                 }
             };
             auto issue = [&](uint32_t step) {
                 const StepCopy c = plan(step);
 #pragma unroll
-                for (int i = 0; i < DMA_PER_WAVE; i++) {
+                for (int i = 0; i < 3; i++) {
                     copy_piece(c, i);
                 }
             };
 
             // ---- S^T = K . Q^T of one step: 32 positions x 32 heads; operands are fetched three ahead -----
-            auto rd_k = [&](const unsigned char *stage, int ks) {
-                return ks < KS_C
-                    ? *reinterpret_cast<const uint4 *>(stage + k_row + ((ks >> 3) << 8) + ((((2 * ks) & 15) << 4) ^ kx))
-                    : *reinterpret_cast<const uint4 *>(stage + p_row + ((((2 * (ks - KS_C)) & 7) << 4) ^ px));
-            };
-            // `between(ks)` is vector-ALU work placed behind the ks-th matrix instruction, which it does not
-            // depend on: it runs while the matrix pipe is busy. The fences keep that order.
-            auto qk = [&](uint32_t step, auto &&between) {
-                const unsigned char *stage = smem + (step % kStages) * STAGE_BYTES;
+            // One accumulation chain (a product that accumulates onto the previous result issues every ~44
+            // cycles instead of 32) with the operand fetches kAhead products ahead: kAhead x 44 cycles cover
+            // the LDS latency, and a second accumulator would cost 16 registers that are not there.
+            // ---- S^T = K . Q^T of one step: 32 positions x 32 heads. One accumulation chain (a product that
+            // accumulates onto the previous result issues every ~44 cycles instead of 32) with the operand
+            // fetches kAhead products ahead.
+            auto qk = [&](uint32_t step) {
+                // addresses of the latent part: 8 registers (the chunk index of k-step ks is 2 ks ^ x; its low
+                // bits select the register, the rest is an immediate)
+                const uint32_t soff = (step % kStages) * STAGE_BYTES;
+                uint32_t xk[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    xk[j] = soff + k_row + ((j << 5) ^ kx);
+                }
+                auto rd_k = [&](int ks) {
+                    return ks < KS_C ? *reinterpret_cast<const uint4 *>(smem + xk[ks & 7] + ((ks >> 3) << 8))
+                                     : *reinterpret_cast<const uint4 *>(smem + soff + p_row + ((((ks - KS_C) & 3) << 5) ^ px));
+                };
                 f32x16_t S;
 #pragma unroll
                 for (int k = 0; k < 16; k++) {
@@ -262,16 +316,15 @@ mla_decode_kernel(const MlaDecodeParams p)
                 uint4 a[kAhead];
 #pragma unroll
                 for (int i = 0; i < kAhead; i++) {
-                    a[i] = rd_k(stage, i);
+                    a[i] = rd_k(i);
                 }
 #pragma unroll
                 for (int ks = 0; ks < KS_C + KS_R; ks++) {
                     S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[ks % kAhead]),
                                                                 __builtin_bit_cast(bf16x8_t, qreg[ks]), S, 0, 0, 0);
                     if (ks + kAhead < KS_C + KS_R) {
-                        a[ks % kAhead] = rd_k(stage, ks + kAhead);
+                        a[ks % kAhead] = rd_k(ks + kAhead);
                     }
-                    between(ks);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 return S;
@@ -286,8 +339,13 @@ mla_decode_kernel(const MlaDecodeParams p)
             issue(min(2u, last));
             for (uint32_t step = 0; step < n_steps; step++) {
                 const uint32_t t = t0 + step * kStep;
-                // keep the offsets derived from these out of loop-invariant registers: there are none to spare
-                asm volatile("" : "+v"(kx), "+v"(px), "+v"(vr_off), "+v"(kc_voff));
+                {
+                    // the lane index from the hardware, opaque to the compiler: nothing derived from it can be
+                    // hoisted out of the loop (and end up in a spill slot, whose reload would wait for every copy)
+                    uint32_t ln;
+                    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+                    set_roles(ln);
+                }
                 dma_wait<2 * DMA_PER_WAVE>();   // this wave's share of `step` has landed
                 __syncthreads();            // ... and everybody else's; stage (step - 1) % 4 is free
 
@@ -295,15 +353,23 @@ mla_decode_kernel(const MlaDecodeParams p)
                 // k % 4. The reference maximum only moves when the step maximum exceeds it by more than
                 // 2^8: probabilities then stay below 2^8 (the same relative precision in bf16, and the
                 // normaliser shares the reference), and the accumulators are rescaled rarely.
-                f32x16_t S = qk(step, [](int) {});
-                const uint32_t lane_pos = t + half * 4;
+                f32x16_t S = qk(step);
+                const uint32_t lane_pos = t + half4;
                 float mx = -INFINITY;
 #pragma unroll
                 for (int k = 0; k < 16; k++) {
-                    const uint32_t pos = lane_pos + (k / 4) * 8 + (k % 4);
-                    const float v = pos < t1 ? S[k] * p.scale_log2e : -INFINITY;
-                    S[k] = v;
-                    mx = fmaxf(mx, v);
+                    S[k] *= p.scale_log2e;
+                }
+                if (t + kStep > t1) {   // uniform: only a tile's last step has positions to mask
+#pragma unroll
+                    for (int k = 0; k < 16; k++) {
+                        const uint32_t pos = lane_pos + (k / 4) * 8 + (k % 4);
+                        S[k] = pos < t1 ? S[k] : -INFINITY;
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    mx = fmaxf(mx, S[k]);
                 }
                 {
                     const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
@@ -347,41 +413,62 @@ mla_decode_kernel(const MlaDecodeParams p)
                 // copies of step + 3 are issued in between
                 {
                     const StepCopy c = plan(min(step + 3, last));
-                    unsigned char *stage = smem + (step % kStages) * STAGE_BYTES;
                     const uint4 pb0 = make_uint4(pw[0], pw[1], pw[2], pw[3]);
                     const uint4 pb1 = make_uint4(pw[4], pw[5], pw[6], pw[7]);
                     typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
-                    auto rd_v = [&](int dt, int kk, int rd) {
-                        unsigned char *ptr = stage + ((dt >> 2) << 8) + kk * 16 * KC_ROWB + rd * 8 * KC_ROWB +
-                                             (vr_off ^ (((dt & 3) << 6) | (rd << 5)));
-                        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
-                    };
-                    uint2 v[2][4];
+                    uint32_t xv[4][2];
+                    {
+                        const uint32_t soff = (step % kStages) * STAGE_BYTES;
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        v[0][j] = rd_v(0, j >> 1, j & 1);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                        for (int a = 0; a < 4; a++) {
 #pragma unroll
-                    for (int dt = 0; dt < DT; dt++) {
-                        if (dt + 1 < DT) {
-#pragma unroll
-                            for (int j = 0; j < 4; j++) {
-                                v[(dt + 1) & 1][j] = rd_v(dt + 1, j >> 1, j & 1);
+                            for (int rd = 0; rd < 2; rd++) {
+                                xv[a][rd] = soff + (vr_off ^ ((a << 6) | (rd << 5)));
                             }
                         }
-                        const uint2 *x = v[dt & 1];
+                    }
+                    auto rd_v = [&](int dt, int kk, int rd) {
+                        unsigned char *ptr = smem + xv[dt & 3][rd] + ((dt >> 2) << 8) + kk * 16 * KC_ROWB + rd * 8 * KC_ROWB;
+                        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
+                    };
+                    constexpr int VB = 3;   // operand buffers: the fetches run two tiles ahead of the products
+                    uint2 v[VB][4];
+#pragma unroll
+                    for (int d = 0; d < VB - 1; d++) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            v[d][j] = rd_v(d, j >> 1, j & 1);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    uint2 carry[2];
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+                        if (dt + VB - 1 < DT) {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                v[(dt + VB - 1) % VB][j] = rd_v(dt + VB - 1, j >> 1, j & 1);
+                            }
+                        }
+                        const uint2 *x = v[dt % VB];
                         O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                             __builtin_bit_cast(bf16x8_t, make_uint4(x[0].x, x[0].y, x[1].x, x[1].y)),
                             __builtin_bit_cast(bf16x8_t, pb0), O[dt], 0, 0, 0);
-                        O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8_t, make_uint4(x[2].x, x[2].y, x[3].x, x[3].y)),
-                            __builtin_bit_cast(bf16x8_t, pb1), O[dt], 0, 0, 0);
-                        if (dt < DMA_PER_WAVE) {
-                            copy_piece(c, dt);
+                        if (dt > 0) {
+                            O[dt - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(bf16x8_t, make_uint4(carry[0].x, carry[0].y, carry[1].x, carry[1].y)),
+                                __builtin_bit_cast(bf16x8_t, pb1), O[dt - 1], 0, 0, 0);
+                        }
+                        carry[0] = x[2];
+                        carry[1] = x[3];
+                        if (dt % 5 == 0 && dt < 15) {
+                            copy_piece(c, dt / 5);
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     }
+                    O[DT - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8_t, make_uint4(carry[0].x, carry[0].y, carry[1].x, carry[1].y)),
+                        __builtin_bit_cast(bf16x8_t, pb1), O[DT - 1], 0, 0, 0);
                 }
             }
             dma_wait<0>();
