@@ -79,6 +79,10 @@ bool mla_decode_supported(const MlaArgs &a);
 size_t mla_decode_workspace_bytes(const MlaArgs &a);
 int launch_mla_decode(hipStream_t stream, const MlaArgs &a);
 
+// prefill_mfma.hip
+bool prefill_mfma_supported(const AttentionArgs &a);
+int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a);
+
 // mfma_attention.hip
 bool mfma_gqa_supported(uint32_t head_dim);
 size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits);

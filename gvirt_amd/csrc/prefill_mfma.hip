@@ -1,0 +1,408 @@
+// Chunked causal prefill over the paged GQA cache on the matrix cores (head_dim 128, 16-bit cache).
+//
+// Workgroup = 8 wavefronts (two per SIMD: while one waits for LDS or does its softmax on the vector
+// ALU, the other keeps the matrix pipe busy) = 256 "M rows" of one kv head, an M row being one
+// (query position, query head of the group) pair. Each wave owns 32 M rows and keeps their query
+// vectors in registers as the B operand; the visible KV positions are walked in tiles of 64:
+//     S^T[pos][m]  = K[pos][:] . Q[m][:]           16 x v_mfma_f32_32x32x16 (A = K rows, ds_read_b128)
+//     O^T[d][m]   += V^T[d][pos] . P^T[pos][m]     16 x v_mfma_f32_32x32x16 (A = V^T, ds_read_b64_tr_b16)
+// K and V tiles are copied straight from the cache into LDS (global_load_lds_dwordx4, one instruction
+// = four consecutive positions of the kv head = 1 KiB of LDS) into a ring of three 32 KiB stages; V
+// stays row major and is transposed on the way out of LDS, so no transposing stores are needed. The
+// 16-byte chunks of a row are XOR-swizzled by the position (the lane chooses which global chunk lands
+// in its LDS slot) so that both read shapes are bank-conflict free.
+// M tiles are numbered sequence by sequence and launched last-first: the tiles with the longest
+// visible range start first.
+//
+// Replaces attention.h / flash_attention.h for batches with multi-token queries
+// (xlite/csrc/kernels/attention.h:308-492, causal rule softmax_attn_aiv.h:739-741).
+#include "attention_common.h"
+
+namespace xlite {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * 64;
+constexpr int kMTile = kWaves * 32;
+constexpr int D = 128;
+constexpr int BN = 64;                    // positions per KV tile
+constexpr int ROWB = D * 2;               // 256: bytes of one (position, kv head) row
+constexpr int KBYTES = BN * ROWB;         // 16 KiB
+constexpr int STAGE = 2 * KBYTES;         // K tile, then V tile
+constexpr int kStages = 3;
+constexpr int KS = D / 16;                // k-steps of the QK product
+constexpr int NT = BN / 32;               // 32-position sub tiles
+constexpr int DT = D / 32;                // 32-row tiles of O^T
+constexpr int PER_WAVE = 2 * BN / 4 / kWaves;   // copies per wave and tile (4)
+
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+
+template <typename T>
+struct Mfma32;
+template <>
+struct Mfma32<BF16> {
+    static __device__ __forceinline__ f32x16_t run(const uint4 &a, const uint4 &b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma32<FP16> {
+    static __device__ __forceinline__ f32x16_t run(const uint4 &a, const uint4 &b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+};
+
+struct PrefillParams {
+    const uint16_t *q;
+    const uint16_t *k_cache;
+    const uint16_t *v_cache;
+    uint16_t *out;
+    const int32_t *query_start_loc;
+    const int32_t *lens;
+    const int32_t *cached_lens;
+    const int32_t *block_tables;
+    uint32_t q_tok_stride;     // elements
+    uint32_t out_tok_stride;
+    uint32_t group;            // query heads per kv head
+    uint32_t n_kv_heads;
+    uint32_t batch;
+    uint32_t block_size;
+    uint32_t max_num_block;
+    uint32_t n_mtiles;         // grid.x
+};
+
+// XOR pattern of the 16-byte chunk index of LDS row `row` (rows are 256 bytes = one bank window). The
+// 16 rows that one ds_read_b128 pass touches get 16 different chunk slots, and the 4 rows that one
+// transposing pass touches get 4 different 64-byte groups.
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+// One wave-wide copy of 1 KiB from global memory into LDS at `lds_addr` + 16 * lane. The compiler sees
+// neither the LDS write nor the memory counter: completion is awaited with dma_wait.
+__device__ __forceinline__ void dma_1k(uint32_t lds_addr, uint32_t voff, const void *base)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                 :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads, 1)
+prefill_kernel(const PrefillParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
+        static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t col = lane & 31;
+    const uint32_t half = lane >> 5;
+    const uint32_t kvh = blockIdx.y;
+    const uint32_t G = p.group;
+
+    // ---- locate the M tile: tiles are numbered sequence by sequence; the grid runs them backwards ----
+    uint32_t seq = 0, mt = p.n_mtiles - 1 - blockIdx.x;
+    int32_t qlen = 0;
+    for (; seq < p.batch; seq++) {
+        qlen = p.lens[seq];
+        const uint32_t tiles = ceil_div(static_cast<uint32_t>(qlen > 0 ? qlen : 0) * G, static_cast<uint32_t>(kMTile));
+        if (mt < tiles) {
+            break;
+        }
+        mt -= tiles;
+    }
+    if (seq >= p.batch) {
+        return;
+    }
+    const int32_t clen = p.cached_lens[seq];
+    const int32_t qstart = p.query_start_loc[seq];
+    const uint32_t m_rows = static_cast<uint32_t>(qlen) * G;
+    const uint32_t m_first = mt * kMTile;
+    const uint32_t m_last = min(m_rows, m_first + kMTile) - 1;
+    // keys visible to at least one row of the tile
+    const uint32_t range_end = static_cast<uint32_t>(clen) + m_last / G + 1;
+    const uint32_t n_tiles = ceil_div(range_end, static_cast<uint32_t>(BN));
+    const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
+    const uint32_t row_bytes = p.n_kv_heads * ROWB;
+
+    // ---- this lane's M row ---------------------------------------------------------------------------
+    const uint32_t m = m_first + wave * 32 + col;
+    const bool m_valid = m < m_rows;
+    const uint32_t qpos = m_valid ? m / G : 0;
+    const uint32_t head = kvh * G + (m_valid ? m % G : 0);
+    const uint32_t tok = static_cast<uint32_t>(qstart) + qpos;
+    const uint32_t vis = m_valid ? static_cast<uint32_t>(clen) + qpos + 1 : 0u;   // causal: keys [0, vis)
+    // tiles wholly below every row's limit need no mask; first tile that does (uniform per wave)
+    const uint32_t wave_min_vis = static_cast<uint32_t>(clen) + min(m_first + wave * 32, m_rows - 1) / G + 1;
+
+    uint4 qreg[KS];
+    {
+        const uint16_t *src = p.q + static_cast<uint64_t>(tok) * p.q_tok_stride + static_cast<uint64_t>(head) * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            qreg[ks] = m_valid ? *reinterpret_cast<const uint4 *>(src + ks * 16 + half * 8) : make_uint4(0, 0, 0, 0);
+        }
+        // complete these loads before any copy is issued: memory operations finish in order, and their
+        // first use is inside the streaming loop
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+        }
+    }
+
+    f32x16_t O[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            O[dt][k] = 0.f;
+        }
+    }
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // ---- read roles ------------------------------------------------------------------------------------
+    // K rows as the A operand: row = position nt * 32 + col, chunk 2 ks + half
+    const uint32_t kx = (half ^ swz(col)) << 4;           // swz(col + 32) == swz(col)
+    const uint32_t k_row = col * ROWB;
+    // transposed V: 16-lane group g covers columns 16 (g % 2) .. +16 of a 32-column tile for the
+    // positions of half g / 2; lane 4 j' + q points at elements [4 q, +4) of position 4 half + j' (+8 for
+    // the second read of a 16-position k-step)
+    uint32_t vr_off;
+    {
+        const uint32_t g = lane >> 4, jp = (lane & 15) >> 2, q = lane & 3;
+        const uint32_t y = 2 * (g & 1) + (q >> 1);
+        const uint32_t pos = 4 * (g >> 1) + jp;
+        vr_off = KBYTES + pos * ROWB + ((y ^ swz(pos)) << 4) + ((q & 1) << 3);
+    }
+    // ---- copy role: wave w moves positions 8w .. 8w+7 of the tile, four per copy, for K and for V.
+    // Lane = (position inside the four) * 16 + chunk slot; the slot receives chunk slot ^ pattern(position).
+    uint32_t c_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t pos = 8 * wave + 4 * i + (lane >> 4);
+        c_voff[i] = (lane >> 4) * row_bytes + (((lane & 15u) ^ swz(pos)) << 4);
+    }
+
+    // copies of KV tile `tile` into stage tile % 3. Four consecutive positions share one block
+    // (block_size % 4 == 0). Positions at or beyond the end of the range re-read the last valid one
+    // (finite values; their probabilities are masked to zero).
+    auto issue = [&](uint32_t tile) {
+        const uint32_t st = smem_addr + (tile % kStages) * STAGE;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t pos = 8 * wave + 4 * i;
+            uint32_t t = tile * BN + pos;
+            uint32_t voff = c_voff[i];
+            if (t + 3 >= range_end) {   // uniform; only the last tile
+                const uint32_t lim = range_end - 1;
+                const uint32_t tl = min(t + (lane >> 4), lim);
+                t = min(t, lim) & ~3u;
+                voff = (tl - t) * row_bytes + (((lane & 15u) ^ swz(pos + (lane >> 4))) << 4);
+            }
+            const uint32_t blk = t / p.block_size, off = t % p.block_size;
+            // a scalar load: tracked apart from the copies in flight (a vector load is not: waiting for
+            // it would wait for every copy issued before it)
+            uint32_t phys;
+            asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(phys) : "s"(table + blk) : "memory");
+            const uint64_t row0 = static_cast<uint64_t>(phys) * p.block_size + off;
+            const char *kb = reinterpret_cast<const char *>(p.k_cache) + row0 * row_bytes + kvh * ROWB;
+            const char *vb = reinterpret_cast<const char *>(p.v_cache) + row0 * row_bytes + kvh * ROWB;
+            dma_1k(st + pos * ROWB, voff, kb);
+            dma_1k(st + KBYTES + pos * ROWB, voff, vb);
+        }
+    };
+
+    auto compute = [&](uint32_t tile) {
+        const uint32_t j0 = tile * BN;
+        const unsigned char *stage = smem + (tile % kStages) * STAGE;
+        // ---- S^T = K . Q^T: two sub tiles of 32 positions; independent accumulators alternate ---------
+        f32x16_t S[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                S[nt][k] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                const uint4 a = *reinterpret_cast<const uint4 *>(stage + nt * 32 * ROWB + k_row + ((ks >> 3) << 8) +
+                                                                 ((((2 * ks) & 15) << 4) ^ kx));
+                S[nt] = Mfma32<T>::run(a, qreg[ks], S[nt]);
+            }
+        }
+        // ---- online softmax; register k of sub tile nt holds position j0 + 32 nt + 8 (k / 4) + 4 half + k % 4.
+        // q arrives scaled by head_dim^-0.5 (rope_and_cache): no scale here.
+        float mx = -INFINITY;
+        if (j0 + BN > wave_min_vis) {   // uniform: the tile reaches past some row's causal limit
+            const uint32_t rem = vis > j0 + half * 4 ? vis - (j0 + half * 4) : 0u;
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    const uint32_t o = nt * 32 + (k / 4) * 8 + (k % 4);
+                    S[nt][k] = rem > o ? S[nt][k] * kLog2e : -INFINITY;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    S[nt][k] *= kLog2e;
+                }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                mx = fmaxf(mx, S[nt][k]);
+            }
+        }
+        {
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+        }
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        m_run = m_new;
+        uint4 pb[NT][2];
+        float psum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+            uint32_t w[8];
+#pragma unroll
+            for (int k = 0; k < 16; k += 2) {
+                const float e0 = fast_exp2(S[nt][k] - m_safe);
+                const float e1 = fast_exp2(S[nt][k + 1] - m_safe);
+                psum += e0 + e1;
+                w[k / 2] = T::pack(e0, e1);
+            }
+            pb[nt][0] = make_uint4(w[0], w[1], w[2], w[3]);
+            pb[nt][1] = make_uint4(w[4], w[5], w[6], w[7]);
+        }
+        l_run = l_run * alpha + psum;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    O[dt][k] *= alpha;
+                }
+            }
+        }
+        // ---- O^T += V^T . P^T: four tiles of 32 columns x four k-steps of 16 positions. The k-step order
+        // inside a lane's registers is positions 8 (e / 4) + 4 half + e % 4, on both operands.
+        typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+#pragma unroll
+        for (int kk = 0; kk < 2 * NT; kk++) {
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                unsigned char *ptr = const_cast<unsigned char *>(stage) + kk * 16 * ROWB + ((dt >> 2) << 8) +
+                                     (vr_off ^ ((dt & 3) << 6));
+                const uint2 x0 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
+                // second read: 8 positions further; the pattern of position p + 8 is that of p XOR 2
+                const uint2 x1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_tr_ptr)(const_cast<unsigned char *>(stage) + kk * 16 * ROWB + 8 * ROWB + ((dt >> 2) << 8) +
+                                 (vr_off ^ (((dt & 3) << 6) | (1 << 5))))));
+                O[dt] = Mfma32<T>::run(make_uint4(x0.x, x0.y, x1.x, x1.y), pb[kk / 2][kk % 2], O[dt]);
+            }
+        }
+    };
+
+    // ---- pipeline: two tiles in flight while the third is consumed; one barrier per tile. Every copy is
+    // unconditional (tiles past the end copy the last tile again into a stage nobody reads any more), so
+    // the wait counts are exact.
+    const uint32_t last = n_tiles - 1;
+    issue(0);
+    issue(min(1u, last));
+    for (uint32_t tile = 0; tile < n_tiles; tile++) {
+        dma_wait<PER_WAVE>();   // this wave's share of `tile` has landed
+        __syncthreads();        // ... and everybody else's; stage (tile - 1) % 3 is free
+        issue(min(tile + 2, last));
+        compute(tile);
+    }
+    dma_wait<0>();
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (m_valid) {
+        // O^T lane layout: column = M row, register k of tile dt = element 32 dt + 8 (k / 4) + 4 half + k % 4
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        uint16_t *dst = p.out + static_cast<uint64_t>(tok) * p.out_tok_stride + static_cast<uint64_t>(head) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+            for (int kg = 0; kg < 4; kg++) {
+                uint2 o;
+                o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
+                o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
+                *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+bool prefill_mfma_supported(const AttentionArgs &a)
+{
+    return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size % 4 == 0 && a.n_heads % a.n_kv_heads == 0;
+}
+
+int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
+{
+    const uint32_t G = a.n_heads / a.n_kv_heads;
+    PrefillParams p{};
+    p.q = static_cast<const uint16_t *>(a.qkv);
+    p.k_cache = static_cast<const uint16_t *>(a.k_cache);
+    p.v_cache = static_cast<const uint16_t *>(a.v_cache);
+    p.out = static_cast<uint16_t *>(a.output);
+    p.query_start_loc = a.query_start_loc;
+    p.lens = a.lens;
+    p.cached_lens = a.cached_lens;
+    p.block_tables = a.block_tables;
+    p.q_tok_stride = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
+    p.out_tok_stride = a.n_heads * a.head_dim;
+    p.group = G;
+    p.n_kv_heads = a.n_kv_heads;
+    p.batch = a.batch;
+    p.block_size = a.block_size;
+    p.max_num_block = a.max_num_block;
+    // upper bound on the number of M tiles: every sequence may end with a ragged one
+    p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
+
+    constexpr size_t lds = static_cast<size_t>(kStages) * STAGE;
+    const bool bf = a.dtype == XLITE_HIP_BF16;
+    static bool configured = false;
+    if (!configured) {
+        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_kernel<BF16>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_kernel<FP16>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        configured = true;
+    }
+    dim3 grid(p.n_mtiles, a.n_kv_heads, 1);
+    if (bf) {
+        prefill_kernel<BF16><<<grid, kThreads, lds, stream>>>(p);
+    } else {
+        prefill_kernel<FP16><<<grid, kThreads, lds, stream>>>(p);
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+}  // namespace xlite
