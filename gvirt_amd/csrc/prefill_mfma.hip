@@ -7,7 +7,7 @@
 //     S^T[pos][m]  = K[pos][:] . Q[m][:]           16 x v_mfma_f32_32x32x16 (A = K rows, ds_read_b128)
 //     O^T[d][m]   += V^T[d][pos] . P^T[pos][m]     16 x v_mfma_f32_32x32x16 (A = V^T, ds_read_b64_tr_b16)
 // K and V tiles are copied straight from the cache into LDS (global_load_lds_dwordx4, one instruction
-// = four consecutive positions of the kv head = 1 KiB of LDS) into a ring of three 32 KiB stages; V
+// = four consecutive positions of the kv head = 1 KiB of LDS) into a ring of four 32 KiB stages; V
 // stays row major and is transposed on the way out of LDS, so no transposing stores are needed. The
 // 16-byte chunks of a row are XOR-swizzled by the position (the lane chooses which global chunk lands
 // in its LDS slot) so that both read shapes are bank-conflict free.
@@ -24,6 +24,7 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kWaves = 8;
+constexpr int kXcds = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kMTile = kWaves * 32;
 constexpr int D = 128;
@@ -31,7 +32,7 @@ constexpr int BN = 64;                    // positions per KV tile
 constexpr int ROWB = D * 2;               // 256: bytes of one (position, kv head) row
 constexpr int KBYTES = BN * ROWB;         // 16 KiB
 constexpr int STAGE = 2 * KBYTES;         // K tile, then V tile
-constexpr int kStages = 3;
+constexpr int kStages = 4;
 constexpr int KS = D / 16;                // k-steps of the QK product
 constexpr int NT = BN / 32;               // 32-position sub tiles
 constexpr int DT = D / 32;                // 32-row tiles of O^T
@@ -72,7 +73,8 @@ struct PrefillParams {
     uint32_t group;            // query heads per kv head
     uint32_t n_kv_heads;
     uint32_t batch;
-    uint32_t block_size;
+    uint32_t block_size;       // a power of two
+    uint32_t block_shift;
     uint32_t max_num_block;
     uint32_t n_mtiles;         // grid.x
 };
@@ -107,11 +109,31 @@ prefill_kernel(const PrefillParams p)
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t col = lane & 31;
     const uint32_t half = lane >> 5;
-    const uint32_t kvh = blockIdx.y;
     const uint32_t G = p.group;
 
+    // ---- which (kv head, M tile). Workgroups are dealt round-robin to the 8 XCDs, each with its own L2;
+    // the M tiles of a kv head stream the same K/V, so a kv head's tiles are kept on one XCD (or on
+    // 8 / n_kv_heads of them, interleaved), where the tiles running at the same time share the L2 lines.
+    uint32_t kvh, mt_fwd;
+    {
+        const uint32_t xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+        if (p.n_kv_heads % kXcds == 0) {
+            kvh = (slot / p.n_mtiles) * kXcds + xcd;
+            mt_fwd = slot % p.n_mtiles;
+        } else if (kXcds % p.n_kv_heads == 0) {
+            const uint32_t r = kXcds / p.n_kv_heads;
+            kvh = xcd % p.n_kv_heads;
+            mt_fwd = slot * r + xcd / p.n_kv_heads;
+        } else {
+            kvh = blockIdx.x / p.n_mtiles;
+            mt_fwd = blockIdx.x % p.n_mtiles;
+        }
+        if (kvh >= p.n_kv_heads || mt_fwd >= p.n_mtiles) {
+            return;
+        }
+    }
     // ---- locate the M tile: tiles are numbered sequence by sequence; the grid runs them backwards ----
-    uint32_t seq = 0, mt = p.n_mtiles - 1 - blockIdx.x;
+    uint32_t seq = 0, mt = p.n_mtiles - 1 - mt_fwd;
     int32_t qlen = 0;
     for (; seq < p.batch; seq++) {
         qlen = p.lens[seq];
@@ -134,6 +156,11 @@ prefill_kernel(const PrefillParams p)
     const uint32_t n_tiles = ceil_div(range_end, static_cast<uint32_t>(BN));
     const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const uint32_t row_bytes = p.n_kv_heads * ROWB;
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE);
+    for (uint32_t i = threadIdx.x; i <= (range_end - 1) >> p.block_shift; i += kThreads) {
+        tbl_lds[i] = static_cast<uint32_t>(table[i]);
+    }
+    __syncthreads();
 
     // ---- this lane's M row ---------------------------------------------------------------------------
     const uint32_t m = m_first + wave * 32 + col;
@@ -209,12 +236,11 @@ prefill_kernel(const PrefillParams p)
                 t = min(t, lim) & ~3u;
                 voff = (tl - t) * row_bytes + (((lane & 15u) ^ swz(pos + (lane >> 4))) << 4);
             }
-            const uint32_t blk = t / p.block_size, off = t % p.block_size;
-            // a scalar load: tracked apart from the copies in flight (a vector load is not: waiting for
-            // it would wait for every copy issued before it)
-            uint32_t phys;
-            asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(phys) : "s"(table + blk) : "memory");
-            const uint64_t row0 = static_cast<uint64_t>(phys) * p.block_size + off;
+            // block-table entries come from LDS (copied there once): a vector load here would have to be
+            // awaited together with every copy issued before it
+            const uint32_t blk = t >> p.block_shift, off = t & (p.block_size - 1);
+            const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk]);
+            const uint64_t row0 = (static_cast<uint64_t>(phys) << p.block_shift) + off;
             const char *kb = reinterpret_cast<const char *>(p.k_cache) + row0 * row_bytes + kvh * ROWB;
             const char *vb = reinterpret_cast<const char *>(p.v_cache) + row0 * row_bytes + kvh * ROWB;
             dma_1k(st + pos * ROWB, voff, kb);
@@ -222,55 +248,67 @@ prefill_kernel(const PrefillParams p)
         }
     };
 
-    auto compute = [&](uint32_t tile) {
-        const uint32_t j0 = tile * BN;
-        const unsigned char *stage = smem + (tile % kStages) * STAGE;
-        // ---- S^T = K . Q^T: two sub tiles of 32 positions; independent accumulators alternate ---------
-        f32x16_t S[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-#pragma unroll
-            for (int k = 0; k < 16; k++) {
-                S[nt][k] = 0.f;
-            }
-        }
+    // The matrix pipe and the vector ALU of a SIMD do not run at the same time, so what can be hidden is
+    // LDS latency: a step's K operands are fetched during the previous step's second product, its V^T
+    // operands during its own softmax.
+    uint4 kop[KS];
+    auto fetch_k = [&](uint32_t stage_off, int h) {
+        const unsigned char *base = smem + stage_off + h * 32 * ROWB + k_row;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
+            kop[ks] = *reinterpret_cast<const uint4 *>(base + ((((2 * ks) & 15) << 4) ^ kx));
+        }
+    };
+
+    // ---- one step of 32 positions. Register k of S holds position j0 + 8 (k / 4) + 4 half + k % 4. The
+    // running maximum is kept in raw score units; q arrives scaled by head_dim^-0.5 (rope_and_cache), so the
+    // only factor is log2(e), folded into the exponent's multiply-add.
+    auto step = [&](uint32_t stage_off, int h, uint32_t j0, uint32_t next_stage_off, int next_h, auto mask_tag) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        // ---- S^T = K . Q^T: two accumulation chains, summed
+        f32x16_t S, S2;
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                const uint4 a = *reinterpret_cast<const uint4 *>(stage + nt * 32 * ROWB + k_row + ((ks >> 3) << 8) +
-                                                                 ((((2 * ks) & 15) << 4) ^ kx));
-                S[nt] = Mfma32<T>::run(a, qreg[ks], S[nt]);
+        for (int k = 0; k < 16; k++) {
+            S[k] = 0.f;
+            S2[k] = 0.f;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks += 2) {
+            S = Mfma32<T>::run(kop[ks], qreg[ks], S);
+            S2 = Mfma32<T>::run(kop[ks + 1], qreg[ks + 1], S2);
+        }
+        // V^T operands of this step: in flight during the softmax
+        typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+        unsigned char *vbase = smem + stage_off + h * 32 * ROWB;
+        uint2 vop[2][DT][2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                vop[kk][dt][0] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_tr_ptr)(vbase + kk * 16 * ROWB + (vr_off ^ ((dt & 3) << 6)))));
+                // second read: 8 positions further; the pattern of position p + 8 is that of p XOR 2
+                vop[kk][dt][1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_tr_ptr)(vbase + kk * 16 * ROWB + 8 * ROWB + (vr_off ^ (((dt & 3) << 6) | (1 << 5))))));
             }
         }
-        // ---- online softmax; register k of sub tile nt holds position j0 + 32 nt + 8 (k / 4) + 4 half + k % 4.
-        // q arrives scaled by head_dim^-0.5 (rope_and_cache): no scale here.
-        float mx = -INFINITY;
-        if (j0 + BN > wave_min_vis) {   // uniform: the tile reaches past some row's causal limit
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            S[k] += S2[k];
+        }
+        if constexpr (MASK) {
             const uint32_t rem = vis > j0 + half * 4 ? vis - (j0 + half * 4) : 0u;
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-#pragma unroll
-                for (int k = 0; k < 16; k++) {
-                    const uint32_t o = nt * 32 + (k / 4) * 8 + (k % 4);
-                    S[nt][k] = rem > o ? S[nt][k] * kLog2e : -INFINITY;
-                }
-            }
-        } else {
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-#pragma unroll
-                for (int k = 0; k < 16; k++) {
-                    S[nt][k] *= kLog2e;
-                }
+            for (int k = 0; k < 16; k++) {
+                const uint32_t o = (k / 4) * 8 + (k % 4);
+                S[k] = rem > o ? S[k] : -INFINITY;
             }
         }
+        float mx = -INFINITY;
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-#pragma unroll
-            for (int k = 0; k < 16; k++) {
-                mx = fmaxf(mx, S[nt][k]);
-            }
+        for (int k = 0; k < 16; k++) {
+            mx = fmaxf(mx, S[k]);
         }
         {
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
@@ -278,63 +316,78 @@ prefill_kernel(const PrefillParams p)
         }
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run - m_safe);
+        const float alpha = fast_exp2((m_run - m_safe) * kLog2e);
+        const float neg_m = -m_safe * kLog2e;
         m_run = m_new;
-        uint4 pb[NT][2];
+        uint32_t w[8];
         float psum = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-            uint32_t w[8];
-#pragma unroll
-            for (int k = 0; k < 16; k += 2) {
-                const float e0 = fast_exp2(S[nt][k] - m_safe);
-                const float e1 = fast_exp2(S[nt][k + 1] - m_safe);
-                psum += e0 + e1;
-                w[k / 2] = T::pack(e0, e1);
-            }
-            pb[nt][0] = make_uint4(w[0], w[1], w[2], w[3]);
-            pb[nt][1] = make_uint4(w[4], w[5], w[6], w[7]);
+        for (int k = 0; k < 16; k += 2) {
+            const float e0 = fast_exp2(__builtin_fmaf(S[k], kLog2e, neg_m));
+            const float e1 = fast_exp2(__builtin_fmaf(S[k + 1], kLog2e, neg_m));
+            psum += e0 + e1;
+            w[k / 2] = T::pack(e0, e1);
         }
+        const uint4 pb[2] = {make_uint4(w[0], w[1], w[2], w[3]), make_uint4(w[4], w[5], w[6], w[7])};
         l_run = l_run * alpha + psum;
         if (__any(alpha != 1.0f)) {
+            // in place (an opaque multiply keeps the accumulators in the same registers on both paths)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
                 for (int k = 0; k < 16; k++) {
-                    O[dt][k] *= alpha;
+                    asm volatile("v_mul_f32 %0, %1, %0" : "+v"(O[dt][k]) : "v"(alpha));
                 }
             }
         }
-        // ---- O^T += V^T . P^T: four tiles of 32 columns x four k-steps of 16 positions. The k-step order
+        __builtin_amdgcn_sched_barrier(0);
+        // K operands of the next step: in flight during the second product
+        fetch_k(next_stage_off, next_h);
+        // ---- O^T += V^T . P^T: four tiles of 32 columns x two k-steps of 16 positions. The k-step order
         // inside a lane's registers is positions 8 (e / 4) + 4 half + e % 4, on both operands.
-        typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
 #pragma unroll
-        for (int kk = 0; kk < 2 * NT; kk++) {
+        for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-                unsigned char *ptr = const_cast<unsigned char *>(stage) + kk * 16 * ROWB + ((dt >> 2) << 8) +
-                                     (vr_off ^ ((dt & 3) << 6));
-                const uint2 x0 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
-                // second read: 8 positions further; the pattern of position p + 8 is that of p XOR 2
-                const uint2 x1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (lds_tr_ptr)(const_cast<unsigned char *>(stage) + kk * 16 * ROWB + 8 * ROWB + ((dt >> 2) << 8) +
-                                 (vr_off ^ (((dt & 3) << 6) | (1 << 5))))));
-                O[dt] = Mfma32<T>::run(make_uint4(x0.x, x0.y, x1.x, x1.y), pb[kk / 2][kk % 2], O[dt]);
+                O[dt] = Mfma32<T>::run(make_uint4(vop[kk][dt][0].x, vop[kk][dt][0].y, vop[kk][dt][1].x, vop[kk][dt][1].y),
+                                       pb[kk], O[dt]);
             }
         }
     };
 
-    // ---- pipeline: two tiles in flight while the third is consumed; one barrier per tile. Every copy is
-    // unconditional (tiles past the end copy the last tile again into a stage nobody reads any more), so
-    // the wait counts are exact.
+    // ---- pipeline: copies run two tiles ahead of the tile being consumed (three right after they are
+    // issued); one barrier per tile of 64 positions, between its two steps, because the second step already
+    // fetches the next tile's first K operands. Every copy is unconditional (tiles past the end copy the last
+    // tile again into a stage nobody reads any more), so the wait counts are exact.
     const uint32_t last = n_tiles - 1;
     issue(0);
     issue(min(1u, last));
-    for (uint32_t tile = 0; tile < n_tiles; tile++) {
-        dma_wait<PER_WAVE>();   // this wave's share of `tile` has landed
-        __syncthreads();        // ... and everybody else's; stage (tile - 1) % 3 is free
-        issue(min(tile + 2, last));
-        compute(tile);
+    issue(min(2u, last));
+    dma_wait<2 * PER_WAVE>();
+    __syncthreads();
+    fetch_k(0, 0);
+    using MaskOn = std::integral_constant<bool, true>;
+    using MaskOff = std::integral_constant<bool, false>;
+    auto tile_iter = [&](uint32_t tile, auto mask_tag) {
+        const uint32_t so = (tile % kStages) * STAGE;
+        const uint32_t so_next = (min(tile + 1, last) % kStages) * STAGE;
+        const uint32_t j0 = tile * BN;
+        step(so, 0, j0, so, 1, mask_tag);
+        dma_wait<PER_WAVE>();   // this wave's share of tile + 1 has landed
+        __syncthreads();        // ... and everybody else's; stage (tile - 1) % 4 is free
+        issue(min(tile + 3, last));
+        step(so, 1, j0 + 32, so_next, 0, mask_tag);
+    };
+    // Tiles wholly below the causal limit of every row of the wave need no mask. Two loops rather than a
+    // branch in one: each loop body exists once, so the accumulators keep their registers. Every wave runs
+    // n_tiles iterations in total (one barrier each), wherever its own boundary between the loops lies.
+    const uint32_t first_masked = min(n_tiles, wave_min_vis / BN);
+    uint32_t tile = 0;
+    for (; tile < first_masked; tile++) {
+        tile_iter(tile, MaskOff{});
+    }
+    for (; tile < n_tiles; tile++) {
+        tile_iter(tile, MaskOn{});
     }
     dma_wait<0>();
 
@@ -360,7 +413,8 @@ prefill_kernel(const PrefillParams p)
 
 bool prefill_mfma_supported(const AttentionArgs &a)
 {
-    return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size % 4 == 0 && a.n_heads % a.n_kv_heads == 0;
+    return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size >= 4 &&
+           (a.block_size & (a.block_size - 1)) == 0 && a.n_heads % a.n_kv_heads == 0;
 }
 
 int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
@@ -381,21 +435,31 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.n_kv_heads = a.n_kv_heads;
     p.batch = a.batch;
     p.block_size = a.block_size;
+    p.block_shift = static_cast<uint32_t>(__builtin_ctz(a.block_size));
     p.max_num_block = a.max_num_block;
     // upper bound on the number of M tiles: every sequence may end with a ragged one
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
 
-    constexpr size_t lds = static_cast<size_t>(kStages) * STAGE;
+    const size_t lds = static_cast<size_t>(kStages) * STAGE + (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     const bool bf = a.dtype == XLITE_HIP_BF16;
-    static bool configured = false;
-    if (!configured) {
+    XL_REQUIRE(lds <= 160 * 1024, "block table too long for the prefill kernel");
+    static size_t configured = 0;
+    if (configured < lds) {
         XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_kernel<BF16>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
         XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_kernel<FP16>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        configured = true;
+        configured = lds;
     }
-    dim3 grid(p.n_mtiles, a.n_kv_heads, 1);
+    uint32_t n_wg;
+    if (a.n_kv_heads % kXcds == 0) {
+        n_wg = a.n_kv_heads * p.n_mtiles;
+    } else if (kXcds % a.n_kv_heads == 0) {
+        n_wg = kXcds * ceil_div(p.n_mtiles, kXcds / a.n_kv_heads);
+    } else {
+        n_wg = a.n_kv_heads * p.n_mtiles;
+    }
+    dim3 grid(n_wg, 1, 1);
     if (bf) {
         prefill_kernel<BF16><<<grid, kThreads, lds, stream>>>(p);
     } else {
