@@ -23,6 +23,7 @@ namespace xlite {
 namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kRescaleSlack = 2.0f / kLog2e;   // raw score units: a factor of 4
 constexpr int kWaves = 8;
 constexpr int kXcds = 8;
 constexpr int kThreads = kWaves * 64;
@@ -265,17 +266,17 @@ prefill_kernel(const PrefillParams p)
     // only factor is log2(e), folded into the exponent's multiply-add.
     auto step = [&](uint32_t stage_off, int h, uint32_t j0, uint32_t next_stage_off, int next_h, auto mask_tag) {
         constexpr bool MASK = decltype(mask_tag)::value;
-        // ---- S^T = K . Q^T: two accumulation chains, summed
-        f32x16_t S, S2;
+        // ---- S^T = K . Q^T (one accumulation chain: the SIMD's other wave fills the issue gaps between
+        // dependent products, and a second chain would cost 16 additions on the vector ALU, which the matrix
+        // pipe cannot overlap)
+        f32x16_t S;
 #pragma unroll
         for (int k = 0; k < 16; k++) {
             S[k] = 0.f;
-            S2[k] = 0.f;
         }
 #pragma unroll
-        for (int ks = 0; ks < KS; ks += 2) {
+        for (int ks = 0; ks < KS; ks++) {
             S = Mfma32<T>::run(kop[ks], qreg[ks], S);
-            S2 = Mfma32<T>::run(kop[ks + 1], qreg[ks + 1], S2);
         }
         // V^T operands of this step: in flight during the softmax
         typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
@@ -293,10 +294,6 @@ prefill_kernel(const PrefillParams p)
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int k = 0; k < 16; k++) {
-            S[k] += S2[k];
-        }
         if constexpr (MASK) {
             const uint32_t rem = vis > j0 + half * 4 ? vis - (j0 + half * 4) : 0u;
 #pragma unroll
@@ -314,7 +311,11 @@ prefill_kernel(const PrefillParams p)
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
             mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
         }
-        const float m_new = fmaxf(m_run, mx);
+        // The reference maximum only moves when the step maximum exceeds it by more than a factor of 4:
+        // probabilities then stay below 4, the normaliser shares the reference, and the accumulators are
+        // rescaled rarely. (A larger slack costs accuracy on peaked rows: with an exact reference the
+        // dominant probability is exactly 1, with a stale one it is rounded to 16 bits like the others.)
+        const float m_new = mx > m_run + kRescaleSlack ? mx : m_run;
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = fast_exp2((m_run - m_safe) * kLog2e);
         const float neg_m = -m_safe * kLog2e;
