@@ -25,7 +25,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
-MEASURED_TRAFFIC_BYTES = {"c2": 1080422086, "c4": 335656121}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080396025, "c4": 355209755}
 
 
 def _events(torch):
@@ -158,7 +158,7 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
-        "roofline": {"bound": "hbm", "kernel": "decode_mfma_kernel (+ merge_kernel)", "achieved": round(achieved, 2),
+        "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_mfma_kernel (+ merge_kernel)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name.split()[0]),
                      "algorithmic_bytes_per_launch": int(alg_bytes)},
@@ -201,7 +201,7 @@ def bench_prefill(args, torch, rt):
             "config": {"workload": "c3 qwen2.5-7b chunked causal prefill", "total_lens": lens, "chunk": 2048,
                        "calls_per_step": len(chunks)},
             "tokens_per_s": round(tokens / (ms * 1e-3), 1),
-            "roofline": {"bound": "mfma", "kernel": "mfma_attention_kernel", "achieved": round(tf, 2),
+            "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                          "traffic": None, "algorithmic_flops_per_step": int(flops)},
             "cpu_baseline": None}
