@@ -241,7 +241,7 @@ def mla_attention(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_cache
     if top_k:
         _dev("topk_indices", topk_indices, torch.int32)
         _req(topk_indices.numel() >= T * top_k, "mla: topk_indices too short")
-    need = rt._lib.xlite_hip_mla_workspace_bytes(T, n_heads, kv_lora_rank, block_size, batch, max_num_blocks)
+    need = rt._lib.xlite_hip_mla_workspace_bytes(T, n_heads, kv_lora_rank, rope_head_dim, block_size, batch, max_num_blocks, top_k)
     ws = rt.workspace(need)
     _lib.check(rt._lib.xlite_hip_mla_attention(
         rt.stream(), _ptr(q_absorb), _ptr(qr), _ptr(k_cache), _ptr(pe_cache), _ptr(o_absorb),
@@ -312,7 +312,7 @@ def mla_v3(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_dense_cache:
     T = q_absorb.shape[0]
     _req(k_dense_cache.numel() == batch * index_topk * kv_lora_rank, "mla_v3: k_dense shape mismatch")
     _req(pe_dense_cache.numel() == batch * index_topk * rope_head_dim, "mla_v3: pe_dense shape mismatch")
-    need = rt._lib.xlite_hip_mla_workspace_bytes(T, n_heads, kv_lora_rank, 1, batch, index_topk)
+    need = rt._lib.xlite_hip_mla_workspace_bytes(T, n_heads, kv_lora_rank, rope_head_dim, 1, batch, index_topk, 0)
     ws = rt.workspace(need)
     _lib.check(rt._lib.xlite_hip_mla_v3(
         rt.stream(), _ptr(q_absorb), _ptr(qr), _ptr(k_dense_cache), _ptr(pe_dense_cache), _ptr(o_absorb),

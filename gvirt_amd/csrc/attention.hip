@@ -105,9 +105,15 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
 }
 
 extern "C" size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
-                                                uint32_t kv_lora_rank, uint32_t block_size,
-                                                uint32_t batch, uint32_t max_num_blocks)
+                                                uint32_t kv_lora_rank, uint32_t rope_head_dim,
+                                                uint32_t block_size, uint32_t batch,
+                                                uint32_t max_num_blocks, uint32_t top_k)
 {
+    if (top_k > 0) {
+        // the gathered per-row caches, then the dense attention over them (every row a sequence)
+        return mla_topk_scratch_bytes(total_tokens, kv_lora_rank, rope_head_dim, top_k) +
+               xlite_hip_mla_workspace_bytes(total_tokens, n_heads, kv_lora_rank, rope_head_dim, 1, total_tokens, top_k, 0);
+    }
     const uint32_t max_ctx = max_num_blocks * block_size;
     const uint32_t splits = mfma_pick_splits(total_tokens, n_heads, batch, 1, max_ctx, 32);
     size_t need = mfma_workspace_bytes(total_tokens, n_heads, kv_lora_rank, splits + 1);
@@ -145,7 +151,6 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16, "qAbsorb/qr/kCache/peCache/oAbsorb dtype unsupported!");
     XL_REQUIRE(top_k <= 2048, "topK should be less than or equal to 2048");
-    XL_REQUIRE(top_k == 0, "top-k index masks are not built yet");
     if (batch == 0 || total_tokens == 0) {
         return XLITE_HIP_OK;
     }
@@ -154,13 +159,12 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
                "null tensor");
     XL_REQUIRE(n_heads > 0 && block_size > 0 && max_num_blocks > 0, "zero head count or block geometry");
     XL_REQUIRE(total_tokens >= batch, "fewer query tokens than sequences");
-    (void)topk_indices;
-    if (batch == 0 || total_tokens == 0) {
-        return XLITE_HIP_OK;
-    }
     MlaArgs a{q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks,
               0, scale, topk_indices, top_k, dtype, workspace, workspace_bytes};
+    if (top_k > 0) {
+        return launch_mla_topk(as_stream(stream), a);
+    }
     if (mla_decode_supported(a)) {
         return launch_mla_decode(as_stream(stream), a);
     }

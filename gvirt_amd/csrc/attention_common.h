@@ -83,6 +83,10 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a);
 bool prefill_mfma_supported(const AttentionArgs &a);
 int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a);
 
+// mla_topk.hip
+size_t mla_topk_scratch_bytes(uint32_t total_tokens, uint32_t kv_lora_rank, uint32_t rope_head_dim, uint32_t top_k);
+int launch_mla_topk(hipStream_t stream, const MlaArgs &a);
+
 // mfma_attention.hip
 bool mfma_gqa_supported(uint32_t head_dim);
 size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits);

@@ -108,11 +108,14 @@ int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, cons
  * o_absorb  [total_tokens, n_heads, kv_lora_rank]
  * scores = (q_absorb . k + qr . pe) * scale, causal as in attention.
  * topk_indices [total_tokens, top_k] int32 (top_k == 0: dense, pointer unused):
- * when top_k > 0 a row attends only to the listed positions that are also
- * inside its causal range. bf16 only (xlite/csrc/op.cpp:1014).
+ * when top_k > 0 a row whose causal range is longer than top_k attends only to the
+ * listed positions (ascending, inside the range); shorter rows see their whole range
+ * (xlite/csrc/kernels/mla_v2.h:697-699). The listed rows are gathered into the workspace
+ * first, so the workspace size depends on top_k. bf16 only (xlite/csrc/op.cpp:1014).
  * ---------------------------------------------------------------------- */
 size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t kv_lora_rank,
-                                     uint32_t block_size, uint32_t batch, uint32_t max_num_blocks);
+                                     uint32_t rope_head_dim, uint32_t block_size, uint32_t batch,
+                                     uint32_t max_num_blocks, uint32_t top_k);
 
 int xlite_hip_mla_attention(void *stream, const void *q_absorb, const void *qr,
                             const void *k_cache, const void *pe_cache, void *o_absorb,

@@ -175,7 +175,9 @@ void brute_mla(const uint16_t *qa, const uint16_t *qr, const uint16_t *kc, const
             int n = clens[i] + r + 1;
             double *s = (double *)malloc(sizeof(double) * (size_t)n);
             char *keep = (char *)malloc((size_t)n);
-            if (top_k > 0) {
+            /* the index list only applies to rows whose causal range is longer than top_k
+               (xlite/csrc/kernels/mla_v2.h:697-699) */
+            if (top_k > 0 && n > top_k) {
                 memset(keep, 0, (size_t)n);
                 for (int t = 0; t < top_k; t++) {
                     int idx = topk[(size_t)tok * top_k + t];

@@ -210,9 +210,16 @@ def mla_attention_ref(q_absorb, qr, k_cache, pe_cache, query_start_loc, lens, ca
         s = s + torch.einsum("qhr,nr->qhn", qrr[st:st + qlen].float(), pe)
         s = s * scale + causal_mask(qlen, clen).unsqueeze(1)
         if top_k > 0:
+            # the index list of a row applies only when its causal range is longer than top_k
+            # (xlite/csrc/kernels/mla_v2.h:697-699); indices outside the range are ignored
             idx = topk_indices.view(T, top_k)[st:st + qlen].long()
-            keep = torch.full((qlen, n), float("-inf"))
-            keep.scatter_(1, idx.clamp(max=n - 1), 0.0)
+            keep = torch.zeros(qlen, n)
+            for r in range(qlen):
+                limit = clen + r + 1
+                if limit > top_k:
+                    keep[r] = float("-inf")
+                    good = idx[r][(idx[r] >= 0) & (idx[r] < limit)]
+                    keep[r, good] = 0.0
             s = s + keep.unsqueeze(1)
         p = torch.softmax(s, dim=-1)
         p = torch.nan_to_num(p, nan=0.0)  # a row with no visible key yields zeros

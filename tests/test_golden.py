@@ -1,0 +1,118 @@
+"""Golden fixtures (tests/golden/*.npz, outputs of the fp64 C brute force) against the PyTorch oracle
+(CPU) and against the HIP kernels through the C ABI (GPU)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import xlite_oracle as O
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+GQA = ["gqa_decode_bf16.npz", "gqa_decode_fp16_d64.npz", "gqa_prefill_bf16.npz"]
+MLA = ["mla_decode.npz", "mla_prefill_topk.npz"]
+ROPE = ["rope_and_cache_bf16.npz", "rope_and_cache_fp16_partial.npz"]
+
+
+def _t16(bits, bf16):
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16 if bf16 else torch.float16)
+
+
+def _load(name):
+    return np.load(os.path.join(GOLD, name), allow_pickle=False)
+
+
+def _gqa_case(name, device="cpu"):
+    z = _load(name)
+    nH, nKV, d, bs, batch, maxblk, bf = [int(x) for x in z["dims"]]
+    t = lambda a: torch.from_numpy(a.copy()).to(device)
+    return dict(qkv=_t16(z["qkv"], bf).to(device), k_cache=_t16(z["k_cache"], bf).to(device), v_cache=_t16(z["v_cache"], bf).to(device),
+                block_tables=t(z["block_tables"]), query_start_loc=t(z["query_start_loc"]), lens=t(z["lens"]),
+                cached_lens=t(z["cached_lens"]), nH=nH, nKV=nKV, d=d, bs=bs, batch=batch, maxblk=maxblk, bf=bf,
+                expected=torch.from_numpy(z["expected"].copy()))
+
+
+def _mla_case(name, device="cpu"):
+    z = _load(name)
+    nH, R, C, bs, batch, maxblk, top_k = [int(x) for x in z["dims"]]
+    t = lambda a: torch.from_numpy(a.copy()).to(device)
+    return dict(q_absorb=_t16(z["q_absorb"], True).to(device), qr=_t16(z["qr"], True).to(device), k_cache=_t16(z["k_cache"], True).to(device),
+                pe_cache=_t16(z["pe_cache"], True).to(device), block_tables=t(z["block_tables"]), query_start_loc=t(z["query_start_loc"]),
+                lens=t(z["lens"]), cached_lens=t(z["cached_lens"]), nH=nH, R=R, C=C, bs=bs, batch=batch, maxblk=maxblk,
+                top_k=top_k, topk=t(z["topk"]) if top_k else None, scale=float(z["scale"]),
+                expected=torch.from_numpy(z["expected"].copy()))
+
+
+@pytest.mark.parametrize("name", GQA)
+def test_oracle_attention_matches_golden(name):
+    c = _gqa_case(name)
+    got = O.attention_ref(c["qkv"], c["k_cache"], c["v_cache"], c["query_start_loc"].tolist(), c["lens"].tolist(),
+                          c["cached_lens"].tolist(), c["block_tables"], c["nH"], c["nKV"], c["d"], c["bs"], c["batch"], c["maxblk"])
+    assert torch.allclose(got.float(), c["expected"], atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("name", MLA)
+def test_oracle_mla_matches_golden(name):
+    c = _mla_case(name)
+    got = O.mla_attention_ref(c["q_absorb"], c["qr"], c["k_cache"], c["pe_cache"], c["query_start_loc"].tolist(), c["lens"].tolist(),
+                              c["cached_lens"].tolist(), c["block_tables"], c["nH"], c["R"], c["C"], c["bs"], c["batch"], c["maxblk"],
+                              c["scale"], c["topk"], c["top_k"])
+    assert torch.allclose(got.float().view(c["expected"].shape), c["expected"], atol=3e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("name", ROPE)
+def test_oracle_rope_and_cache_matches_golden(name):
+    z = _load(name)
+    T, nH, nKV, d, rot, bs, NB, bf = [int(x) for x in z["dims"]]
+    dt = torch.bfloat16 if bf else torch.float16
+    inout = _t16(z["inout"], bf)
+    kc = torch.full((NB, bs, nKV, d), 7.0).to(dt)
+    vc = torch.full((NB, bs, nKV, d), -7.0).to(dt)
+    O.rope_and_cache_ref(inout, kc, vc, torch.from_numpy(z["position"].copy()), _t16(z["cosin"], bf),
+                         torch.from_numpy(z["slot_mapping"].copy()), nH, nKV, d, rot, bs)
+    for got, key in ((inout, "inout_after"), (kc, "k_cache_after"), (vc, "v_cache_after")):
+        assert np.array_equal(got.view(torch.int16).numpy().view(np.uint16).reshape(-1), z[key].reshape(-1))
+
+
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", GQA)
+def test_hip_attention_matches_golden(rt, name):
+    from gvirt_amd import _C
+    c = _gqa_case(name, "cuda:0")
+    out = torch.zeros(c["qkv"].shape[0], c["nH"] * c["d"], dtype=c["qkv"].dtype, device="cuda:0")
+    _C.attention(rt, c["qkv"], c["k_cache"], c["v_cache"], out, c["query_start_loc"], c["lens"], c["cached_lens"],
+                 c["block_tables"], c["nH"], c["nKV"], c["d"], c["bs"], c["batch"], c["maxblk"])
+    err = (out.float().cpu() - c["expected"]).abs()
+    assert float(err.max()) <= 2e-2 and float(err.mean()) <= 2e-3   # bf16 / fp16 storage of P and of the output
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", MLA)
+def test_hip_mla_matches_golden(rt, name):
+    from gvirt_amd import _C
+    c = _mla_case(name, "cuda:0")
+    T = c["q_absorb"].shape[0]
+    out = torch.zeros(T, c["nH"] * c["C"], dtype=torch.bfloat16, device="cuda:0")
+    _C.mla_attention(rt, c["q_absorb"].view(T, -1), c["qr"].view(T, -1), c["k_cache"], c["pe_cache"], out, c["query_start_loc"],
+                     c["lens"], c["cached_lens"], c["block_tables"], c["nH"], c["R"], c["C"], c["bs"], c["batch"], c["maxblk"], c["scale"],
+                     c["topk"], c["top_k"])
+    err = (out.float().cpu().view(c["expected"].shape) - c["expected"]).abs()
+    assert float(err.max()) <= 2e-2 and float(err.mean()) <= 2e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ROPE)
+def test_hip_rope_and_cache_matches_golden_bit_exact(rt, name):
+    from gvirt_amd import _C
+    z = _load(name)
+    T, nH, nKV, d, rot, bs, NB, bf = [int(x) for x in z["dims"]]
+    dt = torch.bfloat16 if bf else torch.float16
+    dev = "cuda:0"
+    inout = _t16(z["inout"], bf).to(dev)
+    kc = torch.full((NB, bs, nKV, d), 7.0).to(dt).to(dev)
+    vc = torch.full((NB, bs, nKV, d), -7.0).to(dt).to(dev)
+    _C.rope_and_cache(rt, inout, kc, vc, torch.from_numpy(z["position"].copy()).to(dev), _t16(z["cosin"], bf).to(dev),
+                      torch.from_numpy(z["slot_mapping"].copy()).to(dev), nH, nKV, d, rot, bs, True)
+    for got, key in ((inout, "inout_after"), (kc, "k_cache_after"), (vc, "v_cache_after")):
+        assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16).reshape(-1), z[key].reshape(-1))

@@ -144,3 +144,39 @@ def test_gather_then_mla_v3(rt, cached, topk):
            512, batch, topk, 192 ** -0.5)
     ref = O.mla_v3_ref(c["qa"], c["qr"], kd.cpu(), pd.cpu(), c["qsl"], c["lens"], c["clens"], 16, 64, 512, batch, topk, 192 ** -0.5)
     check(out.float().cpu(), ref)
+
+
+def _topk_indices(c, top_k, seed):
+    """Index lists as the reference test draws them (xlite/tests/kernels/mla.py:280-303): a random subset of the
+    causal range per query row, padded with its last element when the range is shorter than top_k, ascending."""
+    g = torch.Generator().manual_seed(seed)
+    rows = []
+    for l, cl in zip(c["lens"].tolist(), c["clens"].tolist()):
+        for r in range(l):
+            valid = cl + r + 1
+            perm = torch.randperm(valid, generator=g)
+            perm = torch.cat([perm, perm[-1:].expand(top_k - valid)]) if valid < top_k else perm[:top_k]
+            rows.append(torch.sort(perm).values)
+    return torch.stack(rows).int()
+
+
+@pytest.mark.parametrize("nH", [16, 128])
+@pytest.mark.parametrize("work,top_k", [(([300, 40, 2100], [1, 1, 1]), 64), (([100], [30]), 32), (([0, 500], [70, 3]), 128),
+                                        (([2500, 2047, 2048], [1, 1, 1]), 2048)])
+def test_mla_topk_index_mask(rt, nH, work, top_k):
+    """Rows longer than top_k attend to their listed positions only, shorter rows to their whole range."""
+    from gvirt_amd._C import mla_attention
+    clens, lens = work
+    if nH == 128 and top_k == 2048:
+        pytest.skip("bounded: covered with 16 heads")
+    c = mla_case(41, lens, clens, nH, bs=64)
+    scale = 192 ** -0.5
+    topk = _topk_indices(c, top_k, 42)
+    out = torch.zeros(c["T"], c["nH"], c["C"], dtype=torch.bfloat16, device=DEV)
+    mla_attention(rt, c["qa"].to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), out, c["qsl"].to(DEV),
+                  c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), c["nH"], c["R"], c["C"], c["bs"], c["batch"],
+                  c["maxblk"], scale, topk.to(DEV), top_k)
+    rt.synchronize()
+    ref = O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"],
+                              c["R"], c["C"], c["bs"], c["batch"], c["maxblk"], scale, topk, top_k)
+    check(out.float().cpu(), ref)
