@@ -89,18 +89,22 @@ struct DecodeMfmaParams {
 // 8 cache elements (uint4 = 16-bit, uint2 = int8) -> 8 x 16-bit in a uint4
 template <typename T>
 __device__ __forceinline__ uint4 widen(const uint4 &raw) { return raw; }
+// int8 -> fp16, exactly, in five vector instructions per four values: byte b ^ 0x80 = b + 128 as an
+// unsigned byte u; the half-precision bit pattern 0x6400 | u is 1024 + u; minus 1152 leaves b. (The
+// int8 path therefore runs its matrix products in fp16 whatever the activation type: every int8 value
+// and every probability is exact or as precise in fp16 as in bf16.)
 template <typename T>
 __device__ __forceinline__ uint4 widen(const uint2 &raw)
 {
-    const uint32_t src[2] = {raw.x, raw.y};
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    const h2_t bias = {static_cast<_Float16>(-1152.0f), static_cast<_Float16>(-1152.0f)};
+    const uint32_t src[2] = {raw.x ^ 0x80808080u, raw.y ^ 0x80808080u};
     uint32_t w[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const uint32_t word = src[j / 2];
-        const int sh = (j % 2) * 16;
-        const float a = static_cast<float>(static_cast<int8_t>((word >> sh) & 0xff));
-        const float b = static_cast<float>(static_cast<int8_t>((word >> (sh + 8)) & 0xff));
-        w[j] = T::pack(a, b);
+        const uint32_t spread = __builtin_amdgcn_perm(0x64646464u, src[j / 2], (j % 2) ? 0x04030402u : 0x04010400u);
+        const h2_t v = __builtin_bit_cast(h2_t, spread) + bias;
+        w[j] = __builtin_bit_cast(uint32_t, v);
     }
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
@@ -130,6 +134,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     constexpr int NV = kWaves * kStep * CH / NT;  // 16-byte vectors per thread, step and tensor
     constexpr int STAGE_BYTES = kWaves * 2 * TILE_BYTES;
     typedef typename std::conditional<KV8, uint2, uint4>::type gvec_t;
+    typedef typename std::conditional<KV8, FP16, T>::type TM;   // element type of the matrix products
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -239,6 +244,13 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 for (int ks = 0; ks < KS; ks++) {
                     qreg[ks] = (kv_ok && col < g_valid) ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8)
                                                         : make_uint4(0, 0, 0, 0);
+                    if constexpr (KV8 && !std::is_same<T, TM>::value) {   // bf16 activations: q as fp16
+                        uint32_t *w = reinterpret_cast<uint32_t *>(&qreg[ks]);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            w[j] = TM::pack(T::to_f32(static_cast<uint16_t>(w[j] & 0xffff)), T::to_f32(static_cast<uint16_t>(w[j] >> 16)));
+                        }
+                    }
                 }
                 // Consume the query registers here, before any cache load is issued: their first real
                 // use is inside the streaming loop, where waiting for them would mean waiting for
@@ -366,7 +378,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
                     const uint4 a = *reinterpret_cast<const uint4 *>(stage + kr_off[ks]);
-                    S = Mfma16<T>::run(a, qreg[ks], S);
+                    S = Mfma16<TM>::run(a, qreg[ks], S);
                 }
                 // V^T operands do not depend on the softmax: fetch them now
                 s16x4_t vt[MT];
@@ -412,7 +424,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                     }
                 }
                 l_run = l_run * alpha + psum;
-                const uint2 pb = make_uint2(T::pack(pe[0], pe[1]), T::pack(pe[2], pe[3]));
+                const uint2 pb = make_uint2(TM::pack(pe[0], pe[1]), TM::pack(pe[2], pe[3]));
                 // the running maximum rarely moves after the first steps: skip the rescale then
                 if (__any(alpha != 1.0f)) {
 #pragma unroll
@@ -426,7 +438,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 // ---- O^T += V^T . P^T (k = the 16 positions) ------------------------------------------------------
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
-                    O[mt] = Mfma16<T>::run16(vt[mt], pb, O[mt]);
+                    O[mt] = Mfma16<TM>::run16(vt[mt], pb, O[mt]);
                 }
             };
 
