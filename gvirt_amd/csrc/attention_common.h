@@ -55,6 +55,9 @@ size_t partial_bytes(uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_
 PartialBuffers carve_partials(void *workspace, uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots);
 int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
                  uint32_t n_heads, uint32_t dv, uint32_t max_slots);
+// acc holds O / l in the 16-bit activation type ([rows * n_heads][max_slots][dv], in the same allocation)
+int launch_merge_norm16(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
+                        uint32_t n_heads, uint32_t dv, uint32_t max_slots);
 
 // decode_attention.hip
 bool decode_supported(uint32_t head_dim);

@@ -51,6 +51,53 @@ merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
     }
 }
 
+// The same merge for partials whose O is stored normalised (O_s / l_s) in 16 bits, half the traffic:
+// out = sum_s (w_s l_s) Ohat_s / sum_s (w_s l_s). A thread owns eight output columns of a (row, head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_acc,
+                    const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t n_heads,
+                    uint32_t dv, uint32_t max_slots)
+{
+    const uint32_t row = blockIdx.x;
+    const uint32_t c8 = dv / 8;
+    for (uint32_t it = blockIdx.y * blockDim.x + threadIdx.x; it < n_heads * c8; it += gridDim.y * blockDim.x) {
+        const uint32_t head = it / c8, c = it % c8;
+        const uint64_t rh = static_cast<uint64_t>(row) * n_heads + head;
+        const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
+        if (n == 0) {
+            continue;  // the producer wrote the final value itself
+        }
+        const uint64_t base = rh * max_slots;
+        float mm = -INFINITY;
+        for (uint32_t s = 0; s < n; s++) {
+            mm = fmaxf(mm, part_ml[(base + s) * 2]);
+        }
+        const float ms = mm == -INFINITY ? 0.f : mm;
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float wsum = 0.f;
+        for (uint32_t s = 0; s < n; s++) {
+            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + (base + s) * 2);
+            const float w = fast_exp2(ml.x - ms) * ml.y;
+            wsum += w;
+            const uint4 x = *reinterpret_cast<const uint4 *>(part_acc + (base + s) * dv + c * 8);
+            const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc[2 * j] += T::lo(xs[j]) * w;
+                acc[2 * j + 1] += T::hi(xs[j]) * w;
+            }
+        }
+        const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+        uint4 o;
+        o.x = T::pack(acc[0] * inv, acc[1] * inv);
+        o.y = T::pack(acc[2] * inv, acc[3] * inv);
+        o.z = T::pack(acc[4] * inv, acc[5] * inv);
+        o.w = T::pack(acc[6] * inv, acc[7] * inv);
+        *reinterpret_cast<uint4 *>(out + rh * dv + c * 8) = o;
+    }
+}
+
 }  // namespace
 
 size_t partial_bytes(uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots)
@@ -85,6 +132,23 @@ int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers 
         merge_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
     } else {
         merge_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+int launch_merge_norm16(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
+                        uint32_t n_heads, uint32_t dv, uint32_t max_slots)
+{
+    if (rows == 0) {
+        return XLITE_HIP_OK;
+    }
+    const dim3 grid(rows, min(ceil_div(n_heads * (dv / 8), 256u), 65535u), 1);
+    const uint16_t *acc = reinterpret_cast<const uint16_t *>(b.acc);
+    if (dtype == XLITE_HIP_BF16) {
+        merge_norm16_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, n_heads, dv, max_slots);
+    } else {
+        merge_norm16_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, n_heads, dv, max_slots);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

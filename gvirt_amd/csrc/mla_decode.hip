@@ -13,7 +13,8 @@
 // operands with ds_read_b128; the latent is read again, transposed, with ds_read_b64_tr_b16, so the
 // same LDS bytes serve both products. The 16-byte chunks of a row are XOR-swizzled (by choosing
 // which global chunk a lane copies) so that both read shapes are bank-conflict free.
-// Every workgroup leaves fp32 partials (max, sum, O) that a second kernel merges (merge.hip).
+// Every workgroup leaves a partial (max and sum in fp32, O / sum in bf16: half the bytes of fp32, one more
+// rounding of the same size as the final one) that a second kernel merges (merge.hip).
 //
 // Replaces mla_v2.h / flash_mla_v2.h (paged cache, xlite/csrc/kernels/flash_mla_v2.h:537-847) and
 // mla_v3.h (dense per-sequence cache) of the reference for batches with one query row per sequence.
@@ -489,7 +490,7 @@ mla_decode_kernel(const MlaDecodeParams p)
                     const int dt = ch * 8 + d8;
 #pragma unroll
                     for (int kg = 0; kg < 4; kg++) {
-                        const float sc = single ? inv : 1.0f;
+                        const float sc = inv;   // partials are stored normalised too
                         *reinterpret_cast<float4 *>(my_stage + col * TR_ROWB + (d8 * 32 + kg * 8 + half * 4) * 4) =
                             make_float4(O[dt][kg * 4] * sc, O[dt][kg * 4 + 1] * sc, O[dt][kg * 4 + 2] * sc, O[dt][kg * 4 + 3] * sc);
                     }
@@ -497,14 +498,12 @@ mla_decode_kernel(const MlaDecodeParams p)
                 // wave-private region: the LDS counter wait the compiler inserts is all the ordering needed
                 for (uint32_t hr = 0; hr < heads_here; hr++) {
                     const float4 x = *reinterpret_cast<const float4 *>(my_stage + hr * TR_ROWB + lane * 16);
-                    if (single) {
-                        uint2 o;
-                        o.x = BF16::pack(x.x, x.y);
-                        o.y = BF16::pack(x.z, x.w);
-                        *reinterpret_cast<uint2 *>(p.out + (rh0 + hr) * C + ch * 256 + lane * 4) = o;
-                    } else {
-                        *reinterpret_cast<float4 *>(p.part_acc + ((rh0 + hr) * p.max_slots + tile) * C + ch * 256 + lane * 4) = x;
-                    }
+                    uint2 o;
+                    o.x = BF16::pack(x.x, x.y);
+                    o.y = BF16::pack(x.z, x.w);
+                    uint16_t *dst = single ? p.out + (rh0 + hr) * C
+                                           : reinterpret_cast<uint16_t *>(p.part_acc) + ((rh0 + hr) * p.max_slots + tile) * C;
+                    *reinterpret_cast<uint2 *>(dst + ch * 256 + lane * 4) = o;
                 }
             }
             if (h_ok && half == 0) {
@@ -595,7 +594,7 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
     if (max_slots == 1) {
         return XLITE_HIP_OK;
     }
-    return launch_merge(stream, a.dtype, a.o_absorb, pb, a.total_tokens, a.n_heads, C, max_slots);
+    return launch_merge_norm16(stream, a.dtype, a.o_absorb, pb, a.total_tokens, a.n_heads, C, max_slots);
 }
 
 }  // namespace xlite
