@@ -78,6 +78,28 @@ size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
 
 // mla_decode.hip
+struct MlaDecodeParams {
+    const uint16_t *q_absorb;
+    const uint16_t *qr;
+    const uint16_t *k_cache;
+    const uint16_t *pe_cache;
+    uint16_t *out;
+    const int32_t *query_start_loc;
+    const int32_t *lens;
+    const int32_t *cached_lens;
+    const int32_t *block_tables;   // nullptr: dense cache, dense_len rows per sequence, no causality
+    int32_t *part_cnt;
+    float *part_acc;
+    float *part_ml;
+    uint32_t n_heads;
+    uint32_t batch;
+    uint32_t block_size;
+    uint32_t max_num_blocks;
+    uint32_t dense_len;
+    uint32_t chunk_min_steps;
+    uint32_t max_slots;
+    float scale_log2e;
+};
 bool mla_decode_supported(const MlaArgs &a);
 size_t mla_decode_workspace_bytes(const MlaArgs &a);
 int launch_mla_decode(hipStream_t stream, const MlaArgs &a);
