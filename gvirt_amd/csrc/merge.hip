@@ -52,40 +52,63 @@ merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
 }
 
 // The same merge for partials whose O is stored normalised (O_s / l_s) in 16 bits, half the traffic:
-// out = sum_s (w_s l_s) Ohat_s / sum_s (w_s l_s). A thread owns eight output columns of a (row, head).
+// out = sum_s (w_s l_s) Ohat_s / sum_s (w_s l_s). A wave owns one (row, head): lane s computes the weight of
+// slot s, then the slots' rows (eight columns per lane) are read four at a time so that several loads are in
+// flight per lane.
 template <typename T>
 __global__ void __launch_bounds__(256)
 merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_acc,
-                    const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t n_heads,
+                    const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t total_rh,
                     uint32_t dv, uint32_t max_slots)
 {
-    const uint32_t row = blockIdx.x;
-    const uint32_t c8 = dv / 8;
-    for (uint32_t it = blockIdx.y * blockDim.x + threadIdx.x; it < n_heads * c8; it += gridDim.y * blockDim.x) {
-        const uint32_t head = it / c8, c = it % c8;
-        const uint64_t rh = static_cast<uint64_t>(row) * n_heads + head;
-        const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
-        if (n == 0) {
-            continue;  // the producer wrote the final value itself
-        }
-        const uint64_t base = rh * max_slots;
-        float mm = -INFINITY;
-        for (uint32_t s = 0; s < n; s++) {
-            mm = fmaxf(mm, part_ml[(base + s) * 2]);
-        }
-        const float ms = mm == -INFINITY ? 0.f : mm;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (rh >= total_rh) {
+        return;
+    }
+    const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
+    if (n == 0) {
+        return;  // the producer wrote the final value itself
+    }
+    const uint64_t base = rh * max_slots;
+    float mm = -INFINITY;
+    for (uint32_t s = lane; s < n; s += 64) {
+        mm = fmaxf(mm, part_ml[(base + s) * 2]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        mm = fmaxf(mm, __shfl_xor(mm, d));
+    }
+    const float ms = mm == -INFINITY ? 0.f : mm;
+    for (uint32_t c = lane; c < dv / 8; c += 64) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         float wsum = 0.f;
-        for (uint32_t s = 0; s < n; s++) {
-            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + (base + s) * 2);
-            const float w = fast_exp2(ml.x - ms) * ml.y;
-            wsum += w;
-            const uint4 x = *reinterpret_cast<const uint4 *>(part_acc + (base + s) * dv + c * 8);
-            const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
+        for (uint32_t s0 = 0; s0 < n; s0 += 64) {
+            const uint32_t cnt = min(64u, n - s0);
+            float w_lane = 0.f;
+            if (lane < cnt) {
+                const float2 ml = *reinterpret_cast<const float2 *>(part_ml + (base + s0 + lane) * 2);
+                w_lane = fast_exp2(ml.x - ms) * ml.y;
+            }
+            for (uint32_t j = 0; j < cnt; j += 4) {
+                uint4 x[4];
+                float w[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                acc[2 * j] += T::lo(xs[j]) * w;
-                acc[2 * j + 1] += T::hi(xs[j]) * w;
+                for (uint32_t u = 0; u < 4; u++) {
+                    const uint32_t idx = min(j + u, cnt - 1);
+                    x[u] = *reinterpret_cast<const uint4 *>(part_acc + (base + s0 + idx) * dv + c * 8);
+                    w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    const uint32_t xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+                    wsum += w[u];
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        acc[2 * k] += T::lo(xs[k]) * w[u];
+                        acc[2 * k + 1] += T::hi(xs[k]) * w[u];
+                    }
+                }
             }
         }
         const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
@@ -143,12 +166,13 @@ int launch_merge_norm16(hipStream_t stream, int dtype, void *out, const PartialB
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
-    const dim3 grid(rows, min(ceil_div(n_heads * (dv / 8), 256u), 65535u), 1);
+    const uint32_t total_rh = rows * n_heads;
+    const dim3 grid(ceil_div(total_rh, 4u), 1, 1);
     const uint16_t *acc = reinterpret_cast<const uint16_t *>(b.acc);
     if (dtype == XLITE_HIP_BF16) {
-        merge_norm16_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, n_heads, dv, max_slots);
+        merge_norm16_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, total_rh, dv, max_slots);
     } else {
-        merge_norm16_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, n_heads, dv, max_slots);
+        merge_norm16_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, total_rh, dv, max_slots);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

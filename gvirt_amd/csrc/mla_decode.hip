@@ -1,12 +1,22 @@
-// DeepSeek-style absorbed MLA decode, eight wavefronts of 16 heads each.
+// DeepSeek-style absorbed MLA decode on the matrix cores, split along the KV axis.
 //
-// Same algorithm, partial format and LDS ring as mla_decode.hip, but the 128 heads of a pass are split over
-// eight waves (two per SIMD, 256 registers each) that work on 16x16 tiles:
+// One latent "kv head" is shared by all query heads, so the heads are the MFMA columns: a workgroup of eight
+// wavefronts (two per SIMD, 256 registers each, all of them ordinary vector registers) covers up to 128
+// heads, 16 per wave. A row's positions are walked in steps of 32:
 //   S^T[pos][head]  = [kc | pe][pos][:] . [q_absorb | qr][head][:]   2 x 18 v_mfma_f32_16x16x32_bf16
 //   O^T[c][head]   += kc^T[c][pos] . P^T[pos][head]                   32 x v_mfma_f32_16x16x32_bf16
-// per step of 32 positions. A lane holds Q of one head for a quarter of every 32-element k-step (72
-// registers) and 128 O^T accumulators. Two waves share a SIMD, so the LDS reads, the softmax arithmetic and
-// the copy instructions of one overlap the matrix instructions of the other.
+// A lane holds Q of one head for a quarter of every 32-element k-step (72 registers) and 128 O^T
+// accumulators. The cache never passes through registers: every wave copies its share of a step straight
+// from global memory into LDS (global_load_lds_dwordx4, 1 KiB of consecutive cache bytes per instruction)
+// into a ring of four 36 KiB stages, three steps in flight while the fourth is consumed, one barrier per
+// step. K rows are read from LDS as MFMA A operands with ds_read_b128; the latent is read again,
+// transposed, with ds_read_b64_tr_b16, so the same LDS bytes serve both products. The 16-byte chunks of a
+// row are XOR-swizzled (by choosing which global chunk a lane copies) so that both read shapes are
+// bank-conflict free.
+// Work is balanced over the compute units on the device: the rows' steps, laid end to end, are cut into
+// equal chunks, one per workgroup. Every segment (a row's part inside a chunk) leaves a partial (max and
+// sum in fp32, O / sum in bf16: half the bytes of fp32, one more rounding of the same size as the final
+// one) that a second kernel merges (merge.hip); rows that fit one segment are stored directly.
 //
 // Replaces mla_v2.h / flash_mla_v2.h (paged cache, xlite/csrc/kernels/flash_mla_v2.h:537-847) and
 // mla_v3.h (dense per-sequence cache) of the reference for batches with one query row per sequence.
@@ -524,6 +534,9 @@ mla_decode_kernel(const MlaDecodeParams p)
             first += n;
             row++;
             a = 0;
+        }
+        if (c + gridDim.x >= ceil_div(total, chunk)) {
+            return;   // the usual case: one chunk per workgroup, no second scan
         }
     }
 }
