@@ -10,44 +10,80 @@ namespace xlite {
 
 namespace {
 
+// A wave owns one (row, head): lane s computes the weight and the weighted sum of slot s, then the slots'
+// rows (four columns per lane) are read four at a time so that several loads are in flight per lane.
 template <typename T>
 __global__ void __launch_bounds__(256)
 merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
-             const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t n_heads,
+             const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t total_rh,
              uint32_t dv, uint32_t max_slots)
 {
-    const uint32_t row = blockIdx.x;
-    const uint32_t c4 = dv / 4;
-    for (uint32_t it = blockIdx.y * blockDim.x + threadIdx.x; it < n_heads * c4; it += gridDim.y * blockDim.x) {
-        const uint32_t head = it / c4, c = it % c4;
-        const uint64_t rh = static_cast<uint64_t>(row) * n_heads + head;
-        const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
-        if (n == 0) {
-            continue;  // the producer wrote the final value itself
-        }
-        const uint64_t base = rh * max_slots;
-        float mm = -INFINITY;
-        for (uint32_t s = 0; s < n; s++) {
-            mm = fmaxf(mm, part_ml[(base + s) * 2]);
-        }
-        const float ms = mm == -INFINITY ? 0.f : mm;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (rh >= total_rh) {
+        return;
+    }
+    const uint64_t base = rh * max_slots;
+    // the count, the first maxima and the first rows are fetched together (one round trip to memory instead
+    // of three); what lies beyond the count is discarded unseen
+    const float2 ml_first = *reinterpret_cast<const float2 *>(part_ml + (base + min(lane, max_slots - 1)) * 2);
+    const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
+    if (n == 0) {
+        return;  // the producer wrote the final value itself
+    }
+    float mm = lane < n ? ml_first.x : -INFINITY;
+    for (uint32_t s = lane + 64; s < n; s += 64) {
+        mm = fmaxf(mm, part_ml[(base + s) * 2]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        mm = fmaxf(mm, __shfl_xor(mm, d));
+    }
+    const float ms = mm == -INFINITY ? 0.f : mm;
+    for (uint32_t c0 = 0; c0 < dv / 4; c0 += 64) {
+        const uint32_t c = c0 + lane;
+        const bool c_ok = c < dv / 4;   // idle lanes still take part in the exchanges
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
         float lsum = 0.f;
-        for (uint32_t s = 0; s < n; s++) {
-            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + (base + s) * 2);
-            const float w = fast_exp2(ml.x - ms);
-            lsum += ml.y * w;
-            const float4 x = *reinterpret_cast<const float4 *>(part_acc + (base + s) * dv + c * 4);
-            acc.x += x.x * w;
-            acc.y += x.y * w;
-            acc.z += x.z * w;
-            acc.w += x.w * w;
+        for (uint32_t s0 = 0; s0 < n; s0 += 64) {
+            const uint32_t cnt = min(64u, n - s0);
+            float w_lane = 0.f, l_lane = 0.f;
+            if (lane < cnt) {
+                const float2 ml = s0 == 0 ? ml_first : *reinterpret_cast<const float2 *>(part_ml + (base + s0 + lane) * 2);
+                w_lane = fast_exp2(ml.x - ms);
+                l_lane = ml.y * w_lane;
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                l_lane += __shfl_xor(l_lane, d);
+            }
+            lsum += l_lane;
+            for (uint32_t j = 0; j < cnt; j += 4) {
+                float4 x[4];
+                float w[4];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    const uint32_t idx = min(j + u, cnt - 1);
+                    x[u] = c_ok ? *reinterpret_cast<const float4 *>(part_acc + (base + s0 + idx) * dv + c * 4)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+                    w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    acc.x += x[u].x * w[u];
+                    acc.y += x[u].y * w[u];
+                    acc.z += x[u].z * w[u];
+                    acc.w += x[u].w * w[u];
+                }
+            }
         }
-        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-        uint2 o;
-        o.x = T::pack(acc.x * inv, acc.y * inv);
-        o.y = T::pack(acc.z * inv, acc.w * inv);
-        *reinterpret_cast<uint2 *>(out + rh * dv + c * 4) = o;
+        if (c_ok) {
+            const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+            uint2 o;
+            o.x = T::pack(acc.x * inv, acc.y * inv);
+            o.y = T::pack(acc.z * inv, acc.w * inv);
+            *reinterpret_cast<uint2 *>(out + rh * dv + c * 4) = o;
+        }
     }
 }
 
@@ -80,7 +116,9 @@ merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ par
         mm = fmaxf(mm, __shfl_xor(mm, d));
     }
     const float ms = mm == -INFINITY ? 0.f : mm;
-    for (uint32_t c = lane; c < dv / 8; c += 64) {
+    for (uint32_t c0 = 0; c0 < dv / 8; c0 += 64) {
+        const uint32_t c = c0 + lane;
+        const bool c_ok = c < dv / 8;   // idle lanes still take part in the exchanges
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         float wsum = 0.f;
         for (uint32_t s0 = 0; s0 < n; s0 += 64) {
@@ -96,7 +134,8 @@ merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ par
 #pragma unroll
                 for (uint32_t u = 0; u < 4; u++) {
                     const uint32_t idx = min(j + u, cnt - 1);
-                    x[u] = *reinterpret_cast<const uint4 *>(part_acc + (base + s0 + idx) * dv + c * 8);
+                    x[u] = c_ok ? *reinterpret_cast<const uint4 *>(part_acc + (base + s0 + idx) * dv + c * 8)
+                                : make_uint4(0, 0, 0, 0);
                     w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
                 }
 #pragma unroll
@@ -117,7 +156,9 @@ merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ par
         o.y = T::pack(acc[2] * inv, acc[3] * inv);
         o.z = T::pack(acc[4] * inv, acc[5] * inv);
         o.w = T::pack(acc[6] * inv, acc[7] * inv);
-        *reinterpret_cast<uint4 *>(out + rh * dv + c * 8) = o;
+        if (c_ok) {
+            *reinterpret_cast<uint4 *>(out + rh * dv + c * 8) = o;
+        }
     }
 }
 
@@ -149,12 +190,13 @@ int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers 
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
-    // one thread per (row, head, four output columns)
-    const dim3 grid(rows, min(ceil_div(n_heads * (dv / 4), 256u), 65535u), 1);
+    // one wave per (row, head), four per workgroup
+    const uint32_t total_rh = rows * n_heads;
+    const dim3 grid(ceil_div(total_rh, 4u), 1, 1);
     if (dtype == XLITE_HIP_BF16) {
-        merge_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+        merge_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, total_rh, dv, max_slots);
     } else {
-        merge_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, n_heads, dv, max_slots);
+        merge_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), b.acc, b.ml, b.cnt, total_rh, dv, max_slots);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
