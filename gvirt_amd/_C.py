@@ -321,6 +321,65 @@ def mla_v3(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_dense_cache:
     rt.finish()
 
 
+def _indexer_check(name: str, q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables, n_heads: int,
+                   head_dim: int, batch: int, max_num_block: int) -> int:
+    for n, t in (("q", q), ("k_cache", k_cache), ("weight", weight)):
+        _dev(n, t)
+    for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens),
+                 ("block_tables", block_tables)):
+        _dev(n, t, torch.int32)
+    dt = _act_dtype(name, q, k_cache, weight)
+    T = q.shape[0]
+    _req(q.numel() == T * n_heads * head_dim, "%s: q shape mismatch" % name)
+    _req(weight.numel() == T * (head_dim + n_heads), "%s: weight shape mismatch" % name)
+    _req(block_tables.numel() >= batch * max_num_block, "%s: block_tables too short" % name)
+    return dt
+
+
+def indexer_scores(rt: Runtime, q: torch.Tensor, k_cache: torch.Tensor, weight: torch.Tensor, scores: torch.Tensor,
+                   query_start_loc: torch.Tensor, lens: torch.Tensor, cached_lens: torch.Tensor,
+                   block_tables: torch.Tensor, n_heads: int, head_dim: int, block_size: int, batch: int,
+                   max_num_block: int) -> None:
+    """DSA indexer scores over the cached keys (xlite/_C.pyi:1946-1983): row t of `scores`
+    [total_query_len, max_num_block * block_size] gets sum_h weight[t, head_dim + h] * (q[t, h] . k[j]) for
+    every position j of its sequence."""
+    dt = _indexer_check("indexer_scores", q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables,
+                        n_heads, head_dim, batch, max_num_block)
+    _dev("scores", scores)
+    _req(scores.dtype == q.dtype, "indexer_scores: scores dtype %s unsupported!" % scores.dtype)
+    T = q.shape[0]
+    _req(scores.numel() == T * max_num_block * block_size, "indexer_scores: scores shape mismatch")
+    _lib.check(rt._lib.xlite_hip_indexer_scores(
+        rt.stream(), _ptr(q), _ptr(k_cache), _ptr(weight), _ptr(scores), _ptr(query_start_loc), _ptr(lens),
+        _ptr(cached_lens), _ptr(block_tables), T, n_heads, head_dim, block_size, batch, max_num_block, dt))
+    rt.finish()
+
+
+def indexer_topk(rt: Runtime, q: torch.Tensor, k_cache: torch.Tensor, weight: torch.Tensor, indices: torch.Tensor,
+                 topk_indices: torch.Tensor, query_start_loc: torch.Tensor, lens: torch.Tensor,
+                 cached_lens: torch.Tensor, block_tables: torch.Tensor, n_heads: int, head_dim: int, block_size: int,
+                 batch: int, max_num_block: int, top_k: int) -> None:
+    """Fused indexer scores + top-k selection (xlite/_C.pyi:1985-2040): the first
+    min(top_k, cached + query length) entries of every row of `topk_indices` [total_query_len, top_k] are
+    written; the score rows live in the runtime's scratch pool."""
+    dt = _indexer_check("indexer_topk", q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables,
+                        n_heads, head_dim, batch, max_num_block)
+    _dev("indices", indices, torch.int32)
+    _dev("topk_indices", topk_indices, torch.int32)
+    if top_k > 2048:
+        raise RuntimeError("indexer_topk: topK should be less than or equal to 2048")
+    T = q.shape[0]
+    _req(indices.numel() >= max_num_block * block_size, "indexer_topk: indices too short")
+    _req(topk_indices.numel() == T * top_k, "indexer_topk: topk_indices shape mismatch")
+    need = rt._lib.xlite_hip_indexer_topk_workspace_bytes(T, block_size, max_num_block)
+    ws = rt.workspace(need)
+    _lib.check(rt._lib.xlite_hip_indexer_topk(
+        rt.stream(), _ptr(q), _ptr(k_cache), _ptr(weight), _ptr(indices), _ptr(topk_indices), _ptr(query_start_loc),
+        _ptr(lens), _ptr(cached_lens), _ptr(block_tables), T, n_heads, head_dim, block_size, batch, max_num_block,
+        top_k, dt, _ptr(ws), ws.numel() * ws.element_size()))
+    rt.finish()
+
+
 def _freqs_f32(freqs: torch.Tensor, rope_dim: int) -> torch.Tensor:
     """complex64 [max_pos, rope_dim/2] is read as interleaved fp32 (cos, sin), as the reference does."""
     _req(freqs.is_cuda and freqs.is_contiguous(), "freqs: contiguous GPU tensor expected")

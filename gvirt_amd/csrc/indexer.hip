@@ -1,0 +1,401 @@
+// DSA indexer: scores of every cached position for every query row, and the top-k positions per row.
+//
+//   scores[t][j] = sum_h weight[t][head_dim + h] * round16(q[t][h][:] . k[j][:])      j < cached + query length
+// The per-head dot products are rounded to the 16-bit activation type before they are weighted, as in the
+// reference (xlite/csrc/kernels/indexer_scores.h:176-243: scores -> L1 as Dtype, then a second product with
+// the weights); there is no causal limit inside a sequence and no activation function. Golden:
+// xlite/tests/kernels/indexer_scores.py:96-118.
+//
+// One wavefront owns one query row and a range of 256 positions. Q sits in registers as the A operand of
+// v_mfma_f32_16x16x32 (16 heads x 32 dims per tile), K rows are loaded straight from the paged cache as
+// the B operand (a lane holds 8 dims of one position), so a result tile holds 16 heads x 16 positions
+// with one position per lane column: rounded and packed, it is already the B operand of the second
+// product, whose A operand carries the 16 weights in row 0.
+//
+// The top-k selection (xlite/csrc/kernels/indexer_topk.h, golden xlite/tests/kernels/indexer_topk.py:139-152)
+// runs on the 16-bit scores: a two-pass radix select finds the k-th largest key, then one ordered pass
+// writes the positions above it, and the lowest positions among its ties, in ascending order (the order the
+// top-k mask of the MLA attention wants). Rows with at most k candidates list them all.
+#include "attention_common.h"
+
+namespace xlite {
+
+namespace {
+
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+constexpr int kWavesPerWg = 4;
+constexpr int kRange = 256;          // positions per wave
+constexpr int kSelThreads = 256;
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<BF16> {
+    static __device__ __forceinline__ f32x4_t k32(const uint4 &a, const uint4 &b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t k16(const uint2 &a, const uint2 &b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
+                                                         __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<FP16> {
+    typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 f16x4_t;
+    static __device__ __forceinline__ f32x4_t k32(const uint4 &a, const uint4 &b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t k16(const uint2 &a, const uint2 &b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+                                                     __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+    }
+};
+
+// The sequence that owns query row t, and its number of candidate positions.
+__device__ __forceinline__ bool find_row(uint32_t t, const int32_t *query_start_loc, const int32_t *lens,
+                                         const int32_t *cached_lens, uint32_t batch, uint32_t *seq, uint32_t *total)
+{
+    for (uint32_t i = 0; i < batch; i++) {
+        const int32_t s = query_start_loc[i], l = lens[i];
+        if (static_cast<int32_t>(t) >= s && static_cast<int32_t>(t) < s + l) {
+            *seq = i;
+            *total = static_cast<uint32_t>(cached_lens[i] + l);
+            return true;
+        }
+    }
+    return false;
+}
+
+// NT = n_heads / 16, head_dim = 128.
+template <typename T, int NT>
+__global__ void __launch_bounds__(kWavesPerWg * 64)
+indexer_scores_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
+                      const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
+                      const int32_t *__restrict__ query_start_loc, const int32_t *__restrict__ lens,
+                      const int32_t *__restrict__ cached_lens, const int32_t *__restrict__ block_tables,
+                      uint32_t total_tokens, uint32_t batch, uint32_t block_size, uint32_t max_num_block,
+                      uint32_t ld_scores)
+{
+    constexpr int D = 128;
+    constexpr int KS = D / 32;
+    constexpr int H = NT * 16;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t t = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    if (t >= total_tokens) {
+        return;
+    }
+    uint32_t seq = 0, total = 0;
+    if (!find_row(t, query_start_loc, lens, cached_lens, batch, &seq, &total)) {
+        return;
+    }
+    const uint32_t p0 = blockIdx.y * kRange;
+    if (p0 >= total) {
+        return;
+    }
+    const uint32_t p1 = min(total, p0 + kRange);
+    const uint32_t col = lane & 15, kg = lane >> 4;
+
+    // A operands: Q of head 16 nt + col, dims 32 ks + 8 kg .. +8; weights of heads 16 nt + 4 kg .. +4 in the
+    // lanes of row 0 only
+    uint4 qa[NT][KS];
+    uint2 wa[NT];
+    const uint16_t *qrow = q + static_cast<uint64_t>(t) * H * D;
+    const uint16_t *wrow = weight + static_cast<uint64_t>(t) * (D + H) + D;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            qa[nt][ks] = *reinterpret_cast<const uint4 *>(qrow + (16 * nt + col) * D + 32 * ks + 8 * kg);
+        }
+        uint2 w = make_uint2(0u, 0u);
+        if (col == 0) {
+            const uint16_t *wp = wrow + 16 * nt + 4 * kg;   // 2-byte aligned only: the row pitch may be odd pairs
+            w.x = static_cast<uint32_t>(wp[0]) | (static_cast<uint32_t>(wp[1]) << 16);
+            w.y = static_cast<uint32_t>(wp[2]) | (static_cast<uint32_t>(wp[3]) << 16);
+        }
+        wa[nt] = w;
+    }
+
+    // the block-table entries of the range sit in the lanes of one register (lane i: block p0 / bs + i), so that
+    // a K load does not wait for a table load first; ranges of more than 64 blocks look the table up directly
+    const int32_t *table = block_tables + static_cast<uint64_t>(seq) * max_num_block;
+    const uint32_t blk0 = p0 / block_size;
+    const uint32_t nblk = (p1 - 1) / block_size - blk0 + 1;
+    const bool tbl_in_reg = nblk <= 64;
+    const int32_t tbl_reg = tbl_in_reg && lane < nblk ? table[blk0 + lane] : 0;
+    auto load_k = [&](uint32_t pos0, uint4 (&kb)[KS]) {
+        const uint32_t pos = min(pos0 + col, total - 1);   // positions past the end repeat the last one
+        const uint32_t blk = pos / block_size;
+        const uint32_t phys = static_cast<uint32_t>(tbl_in_reg ? __shfl(tbl_reg, static_cast<int>(min(blk - blk0, 63u)))
+                                                               : table[blk]);
+        const uint16_t *row = k_cache + (static_cast<uint64_t>(phys) * block_size + pos % block_size) * D + 8 * kg;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            kb[ks] = *reinterpret_cast<const uint4 *>(row + 32 * ks);
+        }
+    };
+    constexpr int kPre = 3;   // K tiles in registers: two are in flight while one is consumed
+    uint4 kb[kPre][KS];
+    load_k(p0, kb[0]);
+    if (p0 + 16 < p1) {
+        load_k(p0 + 16, kb[1]);
+    }
+    uint16_t *out = scores + static_cast<uint64_t>(t) * ld_scores;
+    auto tile = [&](uint32_t pos0, const uint4 (&kt)[KS], uint4 (&knext)[KS]) {
+        if (pos0 + 32 < p1) {
+            load_k(pos0 + 32, knext);
+        }
+        f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+            f32x4_t s = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                s = Mma<T>::k32(qa[nt][ks], kt[ks], s);
+            }
+            // lane: position `col`, heads 16 nt + 4 kg + r: the B operand of the weighting product
+            const uint2 sb = make_uint2(T::pack(s[0], s[1]), T::pack(s[2], s[3]));
+            acc = Mma<T>::k16(wa[nt], sb, acc);
+        }
+        // row 0 of the result: lanes 0 .. 15, register 0
+        if (kg == 0 && pos0 + col < p1) {
+            out[pos0 + col] = T::from_f32(acc[0]);
+        }
+    };
+    // the ring of three register tiles, unrolled so that every index is a constant
+    for (uint32_t pos0 = p0; pos0 < p1; pos0 += 48) {
+        tile(pos0, kb[0], kb[2]);
+        if (pos0 + 16 < p1) {
+            tile(pos0 + 16, kb[1], kb[0]);
+        }
+        if (pos0 + 32 < p1) {
+            tile(pos0 + 32, kb[2], kb[1]);
+        }
+    }
+}
+
+// 16-bit float bits -> unsigned key with the same order
+__device__ __forceinline__ uint32_t order_key(uint16_t bits)
+{
+    return (bits & 0x8000u) ? (~static_cast<uint32_t>(bits) & 0xffffu) : (static_cast<uint32_t>(bits) | 0x8000u);
+}
+
+// One workgroup per query row.
+__global__ void __launch_bounds__(kSelThreads)
+indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__restrict__ indices,
+                      int32_t *__restrict__ topk_indices, const int32_t *__restrict__ query_start_loc,
+                      const int32_t *__restrict__ lens, const int32_t *__restrict__ cached_lens,
+                      uint32_t batch, uint32_t top_k, uint32_t ld_scores)
+{
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t wave_cnt[2][kSelThreads / 64];
+    __shared__ uint32_t sel[4];
+    const uint32_t t = blockIdx.x;
+    uint32_t seq = 0, n = 0;
+    if (!find_row(t, query_start_loc, lens, cached_lens, batch, &seq, &n)) {
+        return;
+    }
+    const uint16_t *row = scores + static_cast<uint64_t>(t) * ld_scores;
+    int32_t *out = topk_indices + static_cast<uint64_t>(t) * top_k;
+    if (n <= top_k) {
+        for (uint32_t j = threadIdx.x; j < n; j += kSelThreads) {
+            out[j] = indices[j];
+        }
+        return;
+    }
+    // ---- the k-th largest key: high byte, then low byte
+    uint32_t prefix = 0, above = 0;   // keys whose high byte equals `prefix` are the candidates of pass 2
+    for (int pass = 0; pass < 2; pass++) {
+        hist[threadIdx.x] = 0;
+        __syncthreads();
+        for (uint32_t j = threadIdx.x; j < n; j += kSelThreads) {
+            const uint32_t key = order_key(row[j]);
+            if (pass == 0) {
+                atomicAdd(&hist[key >> 8], 1u);
+            } else if ((key >> 8) == prefix) {
+                atomicAdd(&hist[key & 0xffu], 1u);
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t cum = above;
+            int b = 255;
+            for (; b > 0; b--) {
+                if (cum + hist[b] >= top_k) {
+                    break;
+                }
+                cum += hist[b];
+            }
+            sel[0] = static_cast<uint32_t>(b);
+            sel[1] = cum;
+        }
+        __syncthreads();
+        if (pass == 0) {
+            prefix = sel[0];
+        } else {
+            prefix = (prefix << 8) | sel[0];
+        }
+        above = sel[1];
+        __syncthreads();
+    }
+    const uint32_t thr = prefix;            // the k-th largest key
+    const uint32_t need = top_k - above;    // ties of it to take, lowest positions first
+    // ---- ordered output
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t done = 0, ties = 0;   // running totals, the same in every thread
+    for (uint32_t base = 0; base < n; base += kSelThreads) {
+        const uint32_t j = base + threadIdx.x;
+        const uint32_t key = j < n ? order_key(row[j]) : 0u;
+        const bool gt = j < n && key > thr;
+        const bool eq = j < n && key == thr;
+        const uint64_t m_eq = __ballot(eq);
+        const uint32_t eq_before = __builtin_popcountll(m_eq & ((1ull << lane) - 1));
+        if (lane == 0) {
+            wave_cnt[0][wave] = __builtin_popcountll(m_eq);
+        }
+        __syncthreads();
+        uint32_t eq_rank = ties + eq_before, eq_total = 0;
+#pragma unroll
+        for (uint32_t w = 0; w < kSelThreads / 64; w++) {
+            const uint32_t c = wave_cnt[0][w];
+            eq_rank += w < wave ? c : 0;
+            eq_total += c;
+        }
+        const bool take = gt || (eq && eq_rank < need);
+        const uint64_t m_tk = __ballot(take);
+        const uint32_t tk_before = __builtin_popcountll(m_tk & ((1ull << lane) - 1));
+        if (lane == 0) {
+            wave_cnt[1][wave] = __builtin_popcountll(m_tk);
+        }
+        __syncthreads();
+        uint32_t o = done + tk_before, tk_total = 0;
+#pragma unroll
+        for (uint32_t w = 0; w < kSelThreads / 64; w++) {
+            const uint32_t c = wave_cnt[1][w];
+            o += w < wave ? c : 0;
+            tk_total += c;
+        }
+        if (take && o < top_k) {
+            out[o] = indices[j];
+        }
+        done += tk_total;
+        ties += eq_total;
+    }
+}
+
+template <typename T>
+int launch_scores(hipStream_t stream, const void *q, const void *k_cache, const void *weight, void *scores,
+                  const int32_t *query_start_loc, const int32_t *lens, const int32_t *cached_lens,
+                  const int32_t *block_tables, uint32_t total_tokens, uint32_t n_heads, uint32_t block_size,
+                  uint32_t batch, uint32_t max_num_block, uint32_t ld_scores)
+{
+    const dim3 grid(ceil_div(total_tokens, kWavesPerWg), ceil_div(max_num_block * block_size, kRange), 1);
+#define XL_IDX(NT)                                                                                                    \
+    indexer_scores_kernel<T, NT><<<grid, kWavesPerWg * 64, 0, stream>>>(                                              \
+        static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k_cache), static_cast<const uint16_t *>(weight), \
+        static_cast<uint16_t *>(scores), query_start_loc, lens, cached_lens, block_tables, total_tokens, batch,      \
+        block_size, max_num_block, ld_scores)
+    switch (n_heads / 16) {
+    case 1: XL_IDX(1); break;
+    case 2: XL_IDX(2); break;
+    case 4: XL_IDX(4); break;
+    case 8: XL_IDX(8); break;
+    default: return fail(XLITE_HIP_EINVAL, __func__, "n_heads must be 16, 32, 64 or 128");
+    }
+#undef XL_IDX
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+int check_common(const void *q, const void *k_cache, const void *weight, const int32_t *query_start_loc,
+                 const int32_t *lens, const int32_t *cached_lens, const int32_t *block_tables, uint32_t n_heads,
+                 uint32_t head_dim, uint32_t block_size, int dtype)
+{
+    XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype unsupported!");
+    XL_REQUIRE(q && k_cache && weight && query_start_loc && lens && cached_lens && block_tables, "null tensor");
+    XL_REQUIRE(head_dim == 128, "head_dim must be 128");
+    XL_REQUIRE(n_heads == 16 || n_heads == 32 || n_heads == 64 || n_heads == 128, "n_heads must be 16, 32, 64 or 128");
+    XL_REQUIRE(block_size > 0, "block_size must be positive");
+    return XLITE_HIP_OK;
+}
+
+}  // namespace
+
+}  // namespace xlite
+
+using namespace xlite;
+
+extern "C" int xlite_hip_indexer_scores(void *stream, const void *q, const void *k_cache, const void *weight,
+                                        void *scores, const int32_t *query_start_loc, const int32_t *lens,
+                                        const int32_t *cached_lens, const int32_t *block_tables,
+                                        uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim,
+                                        uint32_t block_size, uint32_t batch, uint32_t max_num_block, int dtype)
+{
+    if (total_tokens == 0 || batch == 0 || max_num_block == 0) {
+        return XLITE_HIP_OK;
+    }
+    const int rc = check_common(q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables, n_heads,
+                                head_dim, block_size, dtype);
+    if (rc != XLITE_HIP_OK) {
+        return rc;
+    }
+    XL_REQUIRE(scores != nullptr, "null tensor");
+    const uint32_t ld = max_num_block * block_size;
+    return dtype == XLITE_HIP_BF16
+               ? launch_scores<BF16>(as_stream(stream), q, k_cache, weight, scores, query_start_loc, lens, cached_lens,
+                                     block_tables, total_tokens, n_heads, block_size, batch, max_num_block, ld)
+               : launch_scores<FP16>(as_stream(stream), q, k_cache, weight, scores, query_start_loc, lens, cached_lens,
+                                     block_tables, total_tokens, n_heads, block_size, batch, max_num_block, ld);
+}
+
+extern "C" size_t xlite_hip_indexer_topk_workspace_bytes(uint32_t total_tokens, uint32_t block_size,
+                                                         uint32_t max_num_block)
+{
+    return static_cast<size_t>(total_tokens) * max_num_block * block_size * sizeof(uint16_t);
+}
+
+extern "C" int xlite_hip_indexer_topk(void *stream, const void *q, const void *k_cache, const void *weight,
+                                      const int32_t *indices, int32_t *topk_indices,
+                                      const int32_t *query_start_loc, const int32_t *lens,
+                                      const int32_t *cached_lens, const int32_t *block_tables,
+                                      uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim,
+                                      uint32_t block_size, uint32_t batch, uint32_t max_num_block, uint32_t top_k,
+                                      int dtype, void *workspace, size_t workspace_bytes)
+{
+    if (total_tokens == 0 || batch == 0 || max_num_block == 0 || top_k == 0) {
+        return XLITE_HIP_OK;
+    }
+    const int rc = check_common(q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables, n_heads,
+                                head_dim, block_size, dtype);
+    if (rc != XLITE_HIP_OK) {
+        return rc;
+    }
+    XL_REQUIRE(indices != nullptr && topk_indices != nullptr, "null tensor");
+    XL_REQUIRE(top_k <= 2048, "topK should be less than or equal to 2048");
+    const size_t need = xlite_hip_indexer_topk_workspace_bytes(total_tokens, block_size, max_num_block);
+    if (workspace == nullptr || workspace_bytes < need) {
+        return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) + " bytes, have " +
+                                                    std::to_string(workspace_bytes));
+    }
+    const uint32_t ld = max_num_block * block_size;
+    const int rc2 =
+        dtype == XLITE_HIP_BF16
+            ? launch_scores<BF16>(as_stream(stream), q, k_cache, weight, workspace, query_start_loc, lens, cached_lens,
+                                  block_tables, total_tokens, n_heads, block_size, batch, max_num_block, ld)
+            : launch_scores<FP16>(as_stream(stream), q, k_cache, weight, workspace, query_start_loc, lens, cached_lens,
+                                  block_tables, total_tokens, n_heads, block_size, batch, max_num_block, ld);
+    if (rc2 != XLITE_HIP_OK) {
+        return rc2;
+    }
+    indexer_select_kernel<<<total_tokens, kSelThreads, 0, as_stream(stream)>>>(
+        static_cast<const uint16_t *>(workspace), indices, topk_indices, query_start_loc, lens, cached_lens, batch,
+        top_k, ld);
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}

@@ -221,6 +221,46 @@ int xlite_hip_prepare_attn(const uint32_t *lens, const uint32_t *cached_lens, ui
                            uint32_t *max_num_blocks, uint32_t *batched_tokens, int *is_decode);
 
 /* ------------------------------------------------------------------------
+ * indexer_scores — replaces XliteOpIndexerScores and kernel
+ * xlite/csrc/kernels/indexer_scores.h:14-290 (API xlite/_C.pyi:1946-1983).
+ * q       [total_tokens, n_heads, head_dim]
+ * k_cache [num_blocks, block_size, head_dim] (one key head)
+ * weight  [total_tokens, head_dim + n_heads]; the last n_heads columns weigh the heads
+ * scores  [total_tokens, max_num_block * block_size]; row t gets
+ *         scores[t][j] = sum_h weight[t][head_dim + h] * round16(q[t][h] . k[j])
+ *         for j < cached_lens[i] + lens[i] of the sequence i that owns row t (no causal limit
+ *         inside the sequence); the rest of the row is left untouched.
+ * head_dim must be 128, n_heads 16, 32, 64 or 128.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_indexer_scores(void *stream, const void *q, const void *k_cache, const void *weight,
+                             void *scores, const int32_t *query_start_loc, const int32_t *lens,
+                             const int32_t *cached_lens, const int32_t *block_tables,
+                             uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim,
+                             uint32_t block_size, uint32_t batch, uint32_t max_num_block, int dtype);
+
+/* ------------------------------------------------------------------------
+ * indexer_topk — replaces XliteOpIndexerTopk and kernel
+ * xlite/csrc/kernels/indexer_topk.h:14-660 (API xlite/_C.pyi:1985-2040): the scores
+ * above, then for every row the top_k positions by score.
+ * indices      [max_num_block * block_size] int32, the value reported for each position
+ *              (the caller fills it with 0, 1, 2, ...)
+ * topk_indices [total_tokens, top_k] int32: the first min(top_k, cached + query length)
+ *              entries of a row are written, in ascending position order (the reference
+ *              leaves the order unspecified; its test compares sets); ties at the k-th
+ *              score go to the lower positions. top_k <= 2048.
+ * workspace: xlite_hip_indexer_topk_workspace_bytes (the 16-bit score rows).
+ * ---------------------------------------------------------------------- */
+size_t xlite_hip_indexer_topk_workspace_bytes(uint32_t total_tokens, uint32_t block_size,
+                                              uint32_t max_num_block);
+int xlite_hip_indexer_topk(void *stream, const void *q, const void *k_cache, const void *weight,
+                           const int32_t *indices, int32_t *topk_indices,
+                           const int32_t *query_start_loc, const int32_t *lens,
+                           const int32_t *cached_lens, const int32_t *block_tables,
+                           uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim,
+                           uint32_t block_size, uint32_t batch, uint32_t max_num_block,
+                           uint32_t top_k, int dtype, void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
  * int8 KV-cache helper (no counterpart in the reference, whose caches are always
  * the activation dtype): quantise rows of `src` [rows, head_dim] into `dst` int8
  * with one fp32 scale per row, scale = absmax/127, q = clamp(rint(x/scale), -127, 127).

@@ -19,6 +19,9 @@ piece of the reference (paths under /root/reference/):
   mla_v2_ref           xlite/csrc/_C.cpp:1234-1301 (einsum + attention + einsum)
   mla_v3_ref           xlite/tests/kernels/mla_v3.py:163-192; xlite/csrc/kernels/mla_v3.h:534-536
   gather_sparse_kv_cache_ref  xlite/tests/kernels/gather_sparse_kv_cache.py:102-116
+  indexer_scores_ref   xlite/tests/kernels/indexer_scores.py:96-118 (golden) with the 16-bit rounding of
+                       the per-head products of xlite/csrc/kernels/indexer_scores.h:214-217
+  indexer_topk_ref     xlite/tests/kernels/indexer_topk.py:139-152
   rope_complex_ref     xlite/tests/kernels/rope_complex.py:31-41 with the fp32 operation order of
                        xlite/csrc/kernels/rope_complex_and_cache.h:165-205
   mla_prepare_ref      xlite/tests/kernels/mla_prepare.py:27-45,90-109
@@ -41,6 +44,9 @@ tests/test_oracle_pins.py):
       preservation, complex-multiply identity in fp64.
   mla_prepare_ref: composition of the two pinned pieces + RMSNorm closed forms.
   gather_*: brute-force Python loops.
+  indexer_scores_ref: pure-Python triple loop in float (tiny case); one head with weight 1 reduces to
+      q . k; with no intermediate rounding the weighted sum equals (sum_h w_h q_h) . k (linearity).
+  indexer_topk_ref: numpy argsort on the same scores; every selected score >= every unselected one.
   get_tile_size_of_cached_kv_ref, prepare_attn_ref: hand-computed cases.
   int8 KV: parity unpinned by the reference (feature absent there); pinned only by
       the round-trip bound |x - dequant(quant(x))| <= scale/2.
@@ -293,6 +299,52 @@ def gather_sparse_kv_cache_ref(k_cache, pe_cache, block_tables, topk_indices, qu
             phys = int(tables[b, tok // block_size])
             kd[b, i] = kc[phys, tok % block_size]
             pd[b, i] = pc[phys, tok % block_size]
+
+
+# --------------------------------------------------------------------------
+# DSA indexer
+# --------------------------------------------------------------------------
+def indexer_scores_ref(q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables, n_heads, head_dim,
+                       block_size, batch, max_num_block, round_heads: bool = True) -> List[torch.Tensor]:
+    """Per sequence i: fp32 tensor [lens[i], cached_lens[i] + lens[i]] of
+    sum_h weight[t, head_dim + h] * (q[t, h] . k[j]); every query row sees every position of its sequence.
+    `round_heads` rounds the per-head products to the activation dtype first, as the reference kernel does
+    when it parks them in L1 (the golden, computed in the activation dtype, rounds there too)."""
+    kc = k_cache.view(-1, block_size, head_dim)
+    tables = block_tables.view(batch, max_num_block)
+    out = []
+    for i in range(batch):
+        s, ql, cl = int(query_start_loc[i]), int(lens[i]), int(cached_lens[i])
+        total = cl + ql
+        k = gather_paged(kc, tables[i].tolist(), total).float()                      # [total, d]
+        qi = q[s:s + ql].reshape(ql, n_heads, head_dim).float()
+        w = weight[s:s + ql].reshape(ql, head_dim + n_heads)[:, head_dim:].float()    # [ql, H]
+        res = torch.empty(ql, total)
+        for r0 in range(0, ql, 64):      # row chunks bound the [rows, heads, positions] intermediate
+            dots = torch.einsum("shd,td->sht", qi[r0:r0 + 64], k)
+            if round_heads:
+                dots = dots.to(q.dtype).float()
+            res[r0:r0 + 64] = torch.einsum("sht,sh->st", dots, w[r0:r0 + 64])
+        out.append(res)
+    return out
+
+
+def indexer_topk_ref(scores: Sequence[torch.Tensor], top_k: int) -> List[List[List[int]]]:
+    """Per sequence, per query row: the positions of the min(top_k, n) largest scores, ascending; ties at
+    the k-th score go to the lower positions."""
+    res = []
+    for sc in scores:
+        rows = []
+        n = sc.shape[1]
+        for r in range(sc.shape[0]):
+            if n <= top_k:
+                rows.append(list(range(n)))
+                continue
+            v = sc[r].double().numpy()
+            order = np.lexsort((np.arange(n), -v))      # by score descending, then position ascending
+            rows.append(sorted(int(x) for x in order[:top_k]))
+        res.append(rows)
+    return res
 
 
 # --------------------------------------------------------------------------

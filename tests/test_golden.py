@@ -116,3 +116,65 @@ def test_hip_rope_and_cache_matches_golden_bit_exact(rt, name):
                       torch.from_numpy(z["slot_mapping"].copy()).to(dev), nH, nKV, d, rot, bs, True)
     for got, key in ((inout, "inout_after"), (kc, "k_cache_after"), (vc, "v_cache_after")):
         assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16).reshape(-1), z[key].reshape(-1))
+
+
+def _indexer_case(device="cpu"):
+    z = _load("indexer_bf16.npz")
+    nH, D, bs, batch, maxblk, top_k = [int(x) for x in z["dims"]]
+    t = lambda a: torch.from_numpy(a.copy()).to(device)
+    return dict(q=_t16(z["q"], True).to(device), w=_t16(z["weight"], True).to(device), kc=_t16(z["k_cache"], True).to(device),
+                tables=t(z["block_tables"]), qsl=t(z["query_start_loc"]), lens=t(z["lens"]), clens=t(z["cached_lens"]),
+                nH=nH, D=D, bs=bs, batch=batch, maxblk=maxblk, top_k=top_k,
+                scores=torch.from_numpy(z["expected_scores"].copy()), topk=z["expected_topk"])
+
+
+def _check_indexer_scores(c, rows):
+    """rows: per sequence [qlen, n] fp32. The golden holds the exact sum; a 16-bit result is within 2^-8."""
+    for i in range(c["batch"]):
+        s, ql = int(c["qsl"][i]), int(c["lens"][i])
+        n = ql + int(c["clens"][i])
+        ref = c["scores"][s:s + ql, :n]
+        assert bool(((rows[i] - ref).abs() <= ref.abs() * 2.0 ** -7 + 0.3).all())
+
+
+def test_oracle_indexer_matches_golden():
+    c = _indexer_case()
+    sc = O.indexer_scores_ref(c["q"], c["kc"], c["w"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"], c["D"],
+                              c["bs"], c["batch"], c["maxblk"])
+    _check_indexer_scores(c, sc)
+    # the selection rule on the golden's own scores reproduces the golden's lists exactly
+    gold_rows = [c["scores"][int(c["qsl"][i]):int(c["qsl"][i]) + int(c["lens"][i]), :int(c["lens"][i]) + int(c["clens"][i])]
+                 .bfloat16().float() for i in range(c["batch"])]
+    sel = O.indexer_topk_ref(gold_rows, c["top_k"])
+    for i in range(c["batch"]):
+        for r in range(int(c["lens"][i])):
+            exp = [int(x) for x in c["topk"][int(c["qsl"][i]) + r] if x >= 0]
+            assert sel[i][r] == exp
+
+
+@pytest.mark.gpu
+def test_hip_indexer_matches_golden(rt):
+    from gvirt_amd import _C
+    c = _indexer_case("cuda:0")
+    T, ld = c["q"].shape[0], c["maxblk"] * c["bs"]
+    scores = torch.zeros(T, ld, dtype=torch.bfloat16, device="cuda:0")
+    args = (c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"], c["D"], c["bs"], c["batch"], c["maxblk"])
+    _C.indexer_scores(rt, c["q"], c["kc"], c["w"], scores, *args)
+    got = scores.float().cpu()
+    rows = [got[int(c["qsl"][i]):int(c["qsl"][i]) + int(c["lens"][i]), :int(c["lens"][i]) + int(c["clens"][i])]
+            for i in range(c["batch"])]
+    _check_indexer_scores(c, rows)
+    out = torch.full((T, c["top_k"]), -1, dtype=torch.int32, device="cuda:0")
+    _C.indexer_topk(rt, c["q"], c["kc"], c["w"], torch.arange(ld, dtype=torch.int32, device="cuda:0"), out, *args, c["top_k"])
+    out = out.cpu().numpy()
+    # near-ties may fall the other way after the 16-bit rounding of slightly different sums: the selected
+    # scores must be the golden's, position by position in sorted order, to within that rounding
+    for i in range(c["batch"]):
+        s, ql = int(c["qsl"][i]), int(c["lens"][i])
+        n = ql + int(c["clens"][i])
+        for r in range(ql):
+            k = min(c["top_k"], n)
+            mine = sorted(float(c["scores"][s + r, j]) for j in out[s + r, :k])
+            gold = sorted(float(c["scores"][s + r, j]) for j in c["topk"][s + r, :k])
+            assert all(abs(a - b) <= abs(b) * 2.0 ** -6 + 0.5 for a, b in zip(mine, gold))
+            assert list(out[s + r, :k]) == sorted(set(out[s + r, :k].tolist()))

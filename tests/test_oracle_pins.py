@@ -299,3 +299,68 @@ def test_fp16_conversions_in_c_match_torch():
         f = L.brute_f16_to_f32(h)
         t = torch.tensor(h if h < 32768 else h - 65536, dtype=torch.int16).view(torch.float16).float().item()
         assert (math.isnan(f) and math.isnan(t)) or f == t
+
+
+def test_indexer_scores_pins():
+    """Triple loop on a tiny case; one head of weight 1 is q . k; without the intermediate rounding the
+    weighted sum is linear in q."""
+    torch.manual_seed(5)
+    H, D, bs = 16, 128, 16
+    lens, clens = [3, 1], [5, 20]
+    batch = 2
+    MB = max((l + c + bs - 1) // bs for l, c in zip(lens, clens))
+    T = sum(lens)
+    q = torch.randn(T, H, D).bfloat16()
+    w = torch.randn(T, D + H).bfloat16()
+    kc = torch.randn(batch * MB + 1, bs, D).bfloat16()
+    perm = torch.randperm(batch * MB + 1)[:batch * MB].to(torch.int32)
+    qsl = torch.tensor([0, 3], dtype=torch.int32)
+    args = (qsl, torch.tensor(lens, dtype=torch.int32), torch.tensor(clens, dtype=torch.int32), perm, H, D, bs, batch, MB)
+    got = O.indexer_scores_ref(q, kc, w, *args, round_heads=False)
+    # brute force
+    for i in range(batch):
+        for r in range(lens[i]):
+            t = int(qsl[i]) + r
+            for j in range(clens[i] + lens[i]):
+                row = kc[int(perm[i * MB + j // bs]), j % bs].float()
+                acc = 0.0
+                for h in range(H):
+                    acc += float(w[t, D + h]) * float((q[t, h].float() * row).sum())
+                assert abs(acc - float(got[i][r, j])) <= 1e-3 * max(1.0, abs(acc))
+    # linearity: (sum_h w_h q_h) . k
+    for i in range(batch):
+        s = int(qsl[i])
+        qw = torch.einsum("shd,sh->sd", q[s:s + lens[i]].double(), w[s:s + lens[i], D:].double())
+        k = O.gather_paged(kc, perm.view(batch, MB)[i].tolist(), clens[i] + lens[i]).double()
+        torch.testing.assert_close(got[i].double(), qw @ k.T, rtol=1e-4, atol=1e-3)
+    # one head with weight 1, the others 0: the rounded product itself
+    w1 = torch.zeros_like(w)
+    w1[:, D + 3] = 1.0
+    one = O.indexer_scores_ref(q, kc, w1, *args)
+    k0 = O.gather_paged(kc, perm.view(batch, MB)[0].tolist(), clens[0] + lens[0]).float()
+    torch.testing.assert_close(one[0], (q[:3, 3].float() @ k0.T).bfloat16().float(), rtol=0, atol=0)
+    # the rounding of the per-head products moves the result by no more than a 16-bit rounding of each term
+    rounded = O.indexer_scores_ref(q, kc, w, *args)
+    for i in range(batch):
+        bound = (w[int(qsl[i]):int(qsl[i]) + lens[i], D:].float().abs().sum(-1, keepdim=True)) * 2.0 ** -8 * 40
+        assert ((rounded[i] - got[i]).abs() <= bound).all()
+
+
+def test_indexer_topk_pins():
+    torch.manual_seed(6)
+    sc = [torch.randn(4, 50).bfloat16().float(), torch.randn(2, 7)]
+    res = O.indexer_topk_ref(sc, 10)
+    for s, rows in zip(sc, res):
+        for r, sel in enumerate(rows):
+            n = s.shape[1]
+            assert sel == sorted(set(sel)) and len(sel) == min(10, n)
+            if n > 10:
+                rest = [j for j in range(n) if j not in sel]
+                assert min(float(s[r, j]) for j in sel) >= max(float(s[r, j]) for j in rest)
+                # ties at the threshold go to the lower positions
+                thr = min(float(s[r, j]) for j in sel)
+                ties_in = [j for j in sel if float(s[r, j]) == thr]
+                ties_out = [j for j in rest if float(s[r, j]) == thr]
+                assert not ties_out or max(ties_in) < min(ties_out)
+                top = torch.topk(s[r], 10).values
+                assert sorted(float(s[r, j]) for j in sel) == sorted(top.tolist())
