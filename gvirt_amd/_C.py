@@ -126,14 +126,22 @@ class Runtime:
 def rope_and_cache(rt: Runtime, inout: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    position: torch.Tensor, cosin: torch.Tensor, slot_mapping: torch.Tensor, n_heads: int,
                    n_kv_heads: int, head_dim: int, rot_dim: int, block_size: int, is_neox: bool,
-                   mrope_mask_h: int = 0, mrope_mask_w: int = 0) -> None:
+                   mrope_mask_h: int = 0, mrope_mask_w: int = 0, *, k_scale: Optional[torch.Tensor] = None,
+                   v_scale: Optional[torch.Tensor] = None) -> None:
+    """RoPE in place on the fused q|k|v rows and the write of K and V into the paged caches
+    (xlite/_C.pyi:1251-1290). Extension (keyword-only): with `k_scale` and `v_scale`
+    [num_blocks, block_size, n_kv_heads] fp32 the caches are int8 and the rows are quantised as they are
+    written (scale = absmax / 127 per token and kv head)."""
     if not is_neox:
         raise RuntimeError("rope_and_cache: unsupported rope type gptj")
-    for n, t in (("inout", inout), ("k_cache", k_cache), ("v_cache", v_cache), ("cosin", cosin)):
+    int8 = k_scale is not None or v_scale is not None
+    for n, t in (("inout", inout), ("cosin", cosin)):
         _dev(n, t)
+    for n, t in (("k_cache", k_cache), ("v_cache", v_cache)):
+        _dev(n, t, torch.int8 if int8 else None)
     _dev("position", position, torch.int64)
     _dev("slot_mapping", slot_mapping, torch.int32)
-    dt = _act_dtype("rope_and_cache", inout, k_cache, v_cache, cosin)
+    dt = _act_dtype("rope_and_cache", inout, cosin) if int8 else _act_dtype("rope_and_cache", inout, k_cache, v_cache, cosin)
     T = inout.shape[0]
     _req(inout.numel() == T * (n_heads + 2 * n_kv_heads) * head_dim, "rope_and_cache: inout shape mismatch")
     _req(k_cache.shape == v_cache.shape, "rope_and_cache: cache shapes differ")
@@ -142,9 +150,19 @@ def rope_and_cache(rt: Runtime, inout: torch.Tensor, k_cache: torch.Tensor, v_ca
     _req(position.numel() == (3 * T if mrope else T), "rope_and_cache: position shape mismatch")
     _req(slot_mapping.numel() >= T, "rope_and_cache: slot_mapping too short")
     _req(cosin.shape[-1] == rot_dim, "rope_and_cache: cosin row must hold rot_dim values")
-    _lib.check(rt._lib.xlite_hip_rope_and_cache(
-        rt.stream(), _ptr(inout), _ptr(k_cache), _ptr(v_cache), _ptr(position), _ptr(cosin), _ptr(slot_mapping),
-        T, n_heads, n_kv_heads, head_dim, rot_dim, block_size, 1, mrope_mask_h, mrope_mask_w, dt))
+    if int8:
+        _req(k_scale is not None and v_scale is not None, "rope_and_cache: int8 caches need k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _dev(n, t, torch.float32)
+            _req(t.numel() * head_dim == k_cache.numel(), "rope_and_cache: %s shape mismatch" % n)
+        _lib.check(rt._lib.xlite_hip_rope_and_cache_int8(
+            rt.stream(), _ptr(inout), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(position),
+            _ptr(cosin), _ptr(slot_mapping), T, n_heads, n_kv_heads, head_dim, rot_dim, block_size, 1, mrope_mask_h,
+            mrope_mask_w, dt))
+    else:
+        _lib.check(rt._lib.xlite_hip_rope_and_cache(
+            rt.stream(), _ptr(inout), _ptr(k_cache), _ptr(v_cache), _ptr(position), _ptr(cosin), _ptr(slot_mapping),
+            T, n_heads, n_kv_heads, head_dim, rot_dim, block_size, 1, mrope_mask_h, mrope_mask_w, dt))
     rt.finish()
 
 

@@ -49,7 +49,7 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
         const bool is_q = hs < n_heads;
         const bool is_k = !is_q && hs < n_heads + n_kv_heads;
         uint16_t *cache_row = nullptr;
-        if (!is_q) {
+        if (!is_q && k_cache != nullptr) {   // no 16-bit caches: the caller quantises the rows afterwards
             const uint32_t slot = static_cast<uint32_t>(slot_mapping[t]);
             const uint32_t kvh = is_k ? hs - n_heads : hs - n_heads - n_kv_heads;
             const uint64_t off =
@@ -121,7 +121,7 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
                     a.h[j] = T::from_f32(T::to_f32(a.h[j]) * q_scale);
                 }
                 *reinterpret_cast<uint4 *>(row + e0) = a.v;
-            } else {
+            } else if (cache_row) {
                 *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
             }
         }
@@ -295,6 +295,31 @@ mla_prepare_kernel(uint16_t *__restrict__ qkvc, const uint16_t *__restrict__ q_w
 // int8 KV quantisation: one 16-lane group per row of head_dim elements (head_dim % 8 == 0,
 // head_dim <= 128*... handled by a strided loop). scale = absmax / 127.
 // ---------------------------------------------------------------------------------------
+// one row by the 16 lanes of a group
+template <typename T>
+__device__ __forceinline__ void quantize_row(const uint16_t *x, int8_t *dst, float *scale_out, uint32_t head_dim,
+                                             uint32_t lane)
+{
+    float amax = 0.f;
+    for (uint32_t i = lane; i < head_dim; i += 16) {
+        amax = fmaxf(amax, fabsf(T::to_f32(x[i])));
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, o));
+    }
+    const float scale = amax / 127.0f;
+    const float safe = scale > 0.f ? scale : 1.0f;
+    for (uint32_t i = lane; i < head_dim; i += 16) {
+        float q = rintf(T::to_f32(x[i]) / safe);
+        q = fminf(fmaxf(q, -127.f), 127.f);
+        dst[i] = static_cast<int8_t>(q);
+    }
+    if (lane == 0) {
+        *scale_out = scale;
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 quantize_kv_kernel(const uint16_t *__restrict__ src, int8_t *__restrict__ dst,
@@ -304,25 +329,32 @@ quantize_kv_kernel(const uint16_t *__restrict__ src, int8_t *__restrict__ dst,
     const uint32_t groups = blockDim.x / 16;
     for (uint64_t r = blockIdx.x * static_cast<uint64_t>(groups) + group; r < rows;
          r += static_cast<uint64_t>(gridDim.x) * groups) {
-        const uint16_t *x = src + r * head_dim;
-        float amax = 0.f;
-        for (uint32_t i = lane; i < head_dim; i += 16) {
-            amax = fmaxf(amax, fabsf(T::to_f32(x[i])));
-        }
-#pragma unroll
-        for (int o = 8; o > 0; o >>= 1) {
-            amax = fmaxf(amax, __shfl_xor(amax, o));
-        }
-        const float scale = amax / 127.0f;
-        const float safe = scale > 0.f ? scale : 1.0f;
-        for (uint32_t i = lane; i < head_dim; i += 16) {
-            float q = rintf(T::to_f32(x[i]) / safe);
-            q = fminf(fmaxf(q, -127.f), 127.f);
-            dst[r * head_dim + i] = static_cast<int8_t>(q);
-        }
-        if (lane == 0) {
-            scales[r] = scale;
-        }
+        quantize_row<T>(src + r * head_dim, dst + r * head_dim, scales + r, head_dim, lane);
+    }
+}
+
+// The K (already rotated) and V rows of the fused activation rows, quantised into the int8 caches at the
+// tokens' slots: row r = (token, K | V, kv head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+quantize_to_cache_kernel(const uint16_t *__restrict__ inout, int8_t *__restrict__ k_cache,
+                         int8_t *__restrict__ v_cache, float *__restrict__ k_scale, float *__restrict__ v_scale,
+                         const int32_t *__restrict__ slot_mapping, uint32_t num_tokens, uint32_t n_heads,
+                         uint32_t n_kv_heads, uint32_t head_dim)
+{
+    const uint32_t group = threadIdx.x / 16, lane = threadIdx.x % 16;
+    const uint32_t groups = blockDim.x / 16;
+    const uint64_t rows = static_cast<uint64_t>(num_tokens) * 2 * n_kv_heads;
+    const uint32_t slots = n_heads + 2 * n_kv_heads;
+    for (uint64_t r = blockIdx.x * static_cast<uint64_t>(groups) + group; r < rows;
+         r += static_cast<uint64_t>(gridDim.x) * groups) {
+        const uint32_t t = static_cast<uint32_t>(r / (2 * n_kv_heads));
+        const uint32_t rem = static_cast<uint32_t>(r % (2 * n_kv_heads));
+        const bool is_v = rem >= n_kv_heads;
+        const uint32_t kvh = is_v ? rem - n_kv_heads : rem;
+        const uint16_t *x = inout + (static_cast<uint64_t>(t) * slots + n_heads + rem) * head_dim;
+        const uint64_t row = static_cast<uint64_t>(static_cast<uint32_t>(slot_mapping[t])) * n_kv_heads + kvh;
+        quantize_row<T>(x, (is_v ? v_cache : k_cache) + row * head_dim, (is_v ? v_scale : k_scale) + row, head_dim, lane);
     }
 }
 
@@ -337,19 +369,18 @@ static uint32_t grid_for(uint64_t work_threads, uint32_t block)
 
 using namespace xlite;
 
-extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_cache,
-                                        const int64_t *position, const void *cosin,
-                                        const int32_t *slot_mapping, uint32_t num_tokens,
-                                        uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
-                                        uint32_t rot_dim, uint32_t block_size, int is_neox,
-                                        uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype)
+// Argument checks and launch of the rope kernel; with `with_cache` false the 16-bit caches are not written.
+static int rope_launch(void *stream, void *inout, void *k_cache, void *v_cache, const int64_t *position,
+                       const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads,
+                       uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, int is_neox,
+                       uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, bool with_cache)
 {
     XL_REQUIRE(is_neox, "unsupported rope type gptj");
     XL_REQUIRE(dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16, "dtype unsupported!");
     if (num_tokens == 0) {
         return XLITE_HIP_OK;
     }
-    XL_REQUIRE(inout && k_cache && v_cache && position && cosin && slot_mapping, "null tensor");
+    XL_REQUIRE(inout && position && cosin && slot_mapping && (!with_cache || (k_cache && v_cache)), "null tensor");
     XL_REQUIRE(n_heads > 0 && n_kv_heads > 0 && block_size > 0, "zero head count or block size");
     XL_REQUIRE(head_dim % 8 == 0 && head_dim > 0, "head_dim must be a multiple of 8");
     XL_REQUIRE(rot_dim % 16 == 0 && rot_dim > 0 && rot_dim <= head_dim,
@@ -357,9 +388,6 @@ extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache
     XL_REQUIRE(((mrope_mask_h | mrope_mask_w) == 0) || rot_dim <= 128,
                "mrope masks address at most 64 rotary lanes");
     XL_REQUIRE((mrope_mask_h & mrope_mask_w) == 0, "mrope masks must be disjoint");
-    if (num_tokens == 0) {
-        return XLITE_HIP_OK;
-    }
     float scale = 1.0f / sqrtf(static_cast<float>(head_dim));
     if (dtype == XLITE_HIP_FP16) {
         // the fp16 kernel of the reference multiplies by the scale rounded to fp16
@@ -371,8 +399,8 @@ extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache
     auto launch = [&](auto tag) {
         using T = decltype(tag);
         rope_and_cache_kernel<T><<<grid, 256, 0, as_stream(stream)>>>(
-            static_cast<uint16_t *>(inout), static_cast<uint16_t *>(k_cache),
-            static_cast<uint16_t *>(v_cache), position, static_cast<const uint16_t *>(cosin),
+            static_cast<uint16_t *>(inout), with_cache ? static_cast<uint16_t *>(k_cache) : nullptr,
+            with_cache ? static_cast<uint16_t *>(v_cache) : nullptr, position, static_cast<const uint16_t *>(cosin),
             slot_mapping, num_tokens, n_heads, n_kv_heads, head_dim, rot_dim, block_size, scale,
             mrope_mask_h, mrope_mask_w);
     };
@@ -380,6 +408,45 @@ extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache
         launch(BF16{});
     } else {
         launch(FP16{});
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_cache,
+                                        const int64_t *position, const void *cosin,
+                                        const int32_t *slot_mapping, uint32_t num_tokens,
+                                        uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                        uint32_t rot_dim, uint32_t block_size, int is_neox,
+                                        uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype)
+{
+    return rope_launch(stream, inout, k_cache, v_cache, position, cosin, slot_mapping, num_tokens, n_heads, n_kv_heads,
+                       head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype, true);
+}
+
+extern "C" int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *k_cache, int8_t *v_cache,
+                                             float *k_scale, float *v_scale, const int64_t *position,
+                                             const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens,
+                                             uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                             uint32_t rot_dim, uint32_t block_size, int is_neox,
+                                             uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype)
+{
+    const int rc = rope_launch(stream, inout, nullptr, nullptr, position, cosin, slot_mapping, num_tokens, n_heads,
+                               n_kv_heads, head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype,
+                               false);
+    if (rc != XLITE_HIP_OK || num_tokens == 0) {
+        return rc;
+    }
+    XL_REQUIRE(k_cache && v_cache && k_scale && v_scale, "null tensor");
+    const uint32_t grid = grid_for(static_cast<uint64_t>(num_tokens) * 2 * n_kv_heads * 16, 256);
+    if (dtype == XLITE_HIP_BF16) {
+        quantize_to_cache_kernel<BF16><<<grid, 256, 0, as_stream(stream)>>>(
+            static_cast<const uint16_t *>(inout), k_cache, v_cache, k_scale, v_scale, slot_mapping, num_tokens, n_heads,
+            n_kv_heads, head_dim);
+    } else {
+        quantize_to_cache_kernel<FP16><<<grid, 256, 0, as_stream(stream)>>>(
+            static_cast<const uint16_t *>(inout), k_cache, v_cache, k_scale, v_scale, slot_mapping, num_tokens, n_heads,
+            n_kv_heads, head_dim);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

@@ -268,6 +268,20 @@ int xlite_hip_indexer_topk(void *stream, const void *q, const void *k_cache, con
 int xlite_hip_quantize_kv_int8(void *stream, const void *src, int8_t *dst, float *scales,
                                uint64_t rows, uint32_t head_dim, int dtype);
 
+/* ------------------------------------------------------------------------
+ * rope_and_cache with quantise-on-write for the int8 KV cache (no counterpart in the
+ * reference): the same rotation and q scaling as xlite_hip_rope_and_cache, in place; the
+ * rotated K rows and the V rows are then quantised as above into
+ * k_cache / v_cache [num_blocks, block_size, n_kv_heads, head_dim] int8 with
+ * k_scale / v_scale [num_blocks, block_size, n_kv_heads] fp32 at the tokens' slots.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *k_cache, int8_t *v_cache,
+                                  float *k_scale, float *v_scale, const int64_t *position,
+                                  const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens,
+                                  uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                  uint32_t rot_dim, uint32_t block_size, int is_neox,
+                                  uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype);
+
 #ifdef __cplusplus
 }
 #endif

@@ -144,3 +144,39 @@ def test_quantize_kv_int8_matches_definition(rt):
     q, s = quantize_kv_int8(rt, x.to(DEV))
     qr, sr = O.quantize_kv_int8(x)
     assert torch.equal(q.cpu(), qr) and torch.equal(s.cpu(), sr)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nH,nKV,d,rot", [(32, 8, 128, 128), (14, 2, 64, 64), (8, 4, 128, 64)])
+def test_rope_and_cache_int8_quantise_on_write(rt, dtype, nH, nKV, d, rot):
+    """The rows land in the int8 cache as the oracle's quantisation of the oracle's rotated rows: bit-exact
+    (values and scales); slots of other tokens keep their contents."""
+    from gvirt_amd._C import rope_and_cache
+    g = torch.Generator().manual_seed(300 + nH + d + rot)
+    T, bs, NB = 37, 16, 5
+    inout = torch.randn(T, (nH + 2 * nKV) * d, generator=g).to(dtype)
+    inout[3, nH * d:(nH + 1) * d] = 0          # an all-zero K row: scale 0, values 0
+    cosin = _cosin(rot, 512, dtype)
+    pos = torch.randint(0, 512, (T,), generator=g)
+    slots = torch.randperm(NB * bs, generator=g)[:T].int()
+    kq = torch.full((NB, bs, nKV, d), 9, dtype=torch.int8, device=DEV)
+    vq = torch.full((NB, bs, nKV, d), -9, dtype=torch.int8, device=DEV)
+    ks = torch.full((NB, bs, nKV), 5.0, device=DEV)
+    vs = torch.full((NB, bs, nKV), -5.0, device=DEV)
+    dev_inout = inout.to(DEV)
+    rope_and_cache(rt, dev_inout, kq, vq, pos.to(DEV), cosin.to(DEV), slots.to(DEV), nH, nKV, d, rot, bs, True,
+                   k_scale=ks, v_scale=vs)
+    # oracle: 16-bit rope and cache write, then the quantiser on the written rows
+    kc = torch.zeros(NB, bs, nKV, d).to(dtype)
+    vc = torch.zeros(NB, bs, nKV, d).to(dtype)
+    O.rope_and_cache_ref(inout, kc, vc, pos, cosin, slots, nH, nKV, d, rot, bs)
+    assert torch.equal(_bits(dev_inout), _bits(inout))
+    kq_ref, ks_ref = O.quantize_kv_int8(kc)
+    vq_ref, vs_ref = O.quantize_kv_int8(vc)
+    written = torch.zeros(NB * bs, dtype=torch.bool)
+    written[slots.long()] = True
+    w = written.view(NB, bs)
+    assert torch.equal(kq.cpu()[w], kq_ref[w]) and torch.equal(vq.cpu()[w], vq_ref[w])
+    assert torch.equal(ks.cpu()[w], ks_ref[w]) and torch.equal(vs.cpu()[w], vs_ref[w])
+    assert bool((kq.cpu()[~w] == 9).all()) and bool((vq.cpu()[~w] == -9).all())
+    assert bool((ks.cpu()[~w] == 5.0).all()) and bool((vs.cpu()[~w] == -5.0).all())
