@@ -339,6 +339,31 @@ def mla_v3(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_dense_cache:
     rt.finish()
 
 
+def qk_rms_norm(rt: Runtime, qkv: torch.Tensor, q_norm: torch.Tensor, q_norm_bias: Optional[torch.Tensor],
+                k_norm: torch.Tensor, k_norm_bias: Optional[torch.Tensor], out: torch.Tensor, norm_eps: float,
+                q_norm_dim: int, q_cnt_per_token: int, k_norm_dim: int, k_cnt_per_token: int,
+                k_start_offset: int) -> None:
+    """RMSNorm of the Q and K segments of the fused qkv rows, argument order of the reference's C++ operator
+    (xlite/csrc/op.cpp:1177-1182; it has no Python binding there). `out` may be `qkv`."""
+    for n, t in (("qkv", qkv), ("q_norm", q_norm), ("k_norm", k_norm), ("out", out)):
+        _dev(n, t)
+    tensors = [qkv, q_norm, k_norm, out]
+    for n, t in (("q_norm_bias", q_norm_bias), ("k_norm_bias", k_norm_bias)):
+        if t is not None:
+            _dev(n, t)
+            tensors.append(t)
+    dt = _act_dtype("qk_rms_norm", *tensors)
+    _req(qkv.dim() == 2 and out.shape == qkv.shape, "qk_rms_norm: qkv and out must be [tokens, row] of one shape")
+    _req(q_norm.numel() == q_norm_dim and k_norm.numel() == k_norm_dim, "qk_rms_norm: weight shape mismatch")
+    _req(q_norm_bias is None or q_norm_bias.numel() == q_norm_dim, "qk_rms_norm: q bias shape mismatch")
+    _req(k_norm_bias is None or k_norm_bias.numel() == k_norm_dim, "qk_rms_norm: k bias shape mismatch")
+    _lib.check(rt._lib.xlite_hip_qk_rms_norm(
+        rt.stream(), _ptr(qkv), _ptr(out), _ptr(q_norm), _ptr(q_norm_bias), _ptr(k_norm), _ptr(k_norm_bias),
+        qkv.shape[0], qkv.shape[1], q_norm_dim, q_cnt_per_token, k_norm_dim, k_cnt_per_token, k_start_offset,
+        float(norm_eps), dt))
+    rt.finish()
+
+
 def _indexer_check(name: str, q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables, n_heads: int,
                    head_dim: int, batch: int, max_num_block: int) -> int:
     for n, t in (("q", q), ("k_cache", k_cache), ("weight", weight)):

@@ -28,6 +28,7 @@ SIGNATURES = {
     "xlite_hip_prepare_attn": (_i32, [_vp, _vp, _u32, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp]),
     "xlite_hip_quantize_kv_int8": (_i32, [_vp] * 4 + [_u64, _u32, _i32]),
     "xlite_hip_rope_and_cache_int8": (_i32, [_vp] * 9 + [_u32] * 6 + [_i32, _u64, _u64, _i32]),
+    "xlite_hip_qk_rms_norm": (_i32, [_vp] * 7 + [_u32] * 7 + [_f32, _i32]),
     "xlite_hip_indexer_scores": (_i32, [_vp] * 9 + [_u32] * 6 + [_i32]),
     "xlite_hip_indexer_topk_workspace_bytes": (_sz, [_u32] * 3),
     "xlite_hip_indexer_topk": (_i32, [_vp] * 10 + [_u32] * 7 + [_i32, _vp, _sz]),

@@ -295,6 +295,53 @@ mla_prepare_kernel(uint16_t *__restrict__ qkvc, const uint16_t *__restrict__ q_w
 // int8 KV quantisation: one 16-lane group per row of head_dim elements (head_dim % 8 == 0,
 // head_dim <= 128*... handled by a strided loop). scale = absmax / 127.
 // ---------------------------------------------------------------------------------------
+// ---------------------------------------------------------------------------------------
+// qk_rms_norm (xlite/csrc/kernels/qk_rms_norm.h:32-54, arithmetic of xlite/csrc/kernels/norm.h:272-320):
+// RMSNorm of the Q segment (q_cnt vectors of q_dim elements from column 0) and of the K segment (k_cnt
+// vectors of k_dim elements from column k_start) of every row; other columns are not touched. One 16-lane
+// group per vector: y = x * rsqrt(mean(x^2) + eps) * w + b in fp32, rounded once.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_rms_norm_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, const uint16_t *__restrict__ q_w,
+                   const uint16_t *__restrict__ q_b, const uint16_t *__restrict__ k_w,
+                   const uint16_t *__restrict__ k_b, uint32_t num_tokens, uint32_t row_elems, uint32_t q_dim,
+                   uint32_t q_cnt, uint32_t k_dim, uint32_t k_cnt, uint32_t k_start, float eps)
+{
+    const uint32_t group = threadIdx.x / 16, lane = threadIdx.x % 16;
+    const uint32_t groups = blockDim.x / 16;
+    const uint32_t per_token = q_cnt + k_cnt;
+    const uint64_t vectors = static_cast<uint64_t>(num_tokens) * per_token;
+    for (uint64_t v = blockIdx.x * static_cast<uint64_t>(groups) + group; v < vectors;
+         v += static_cast<uint64_t>(gridDim.x) * groups) {
+        const uint32_t t = static_cast<uint32_t>(v / per_token);
+        const uint32_t j = static_cast<uint32_t>(v % per_token);
+        const bool is_k = j >= q_cnt;
+        const uint32_t dim = is_k ? k_dim : q_dim;
+        const uint64_t off = static_cast<uint64_t>(t) * row_elems + (is_k ? k_start + (j - q_cnt) * k_dim : j * q_dim);
+        const uint16_t *w = is_k ? k_w : q_w, *b = is_k ? k_b : q_b;
+        const uint16_t *x = in + off;
+        float acc = 0.f;
+        for (uint32_t i = lane; i < dim; i += 16) {
+            const float xv = T::to_f32(x[i]);
+            acc += xv * xv;
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) {
+            acc += __shfl_xor(acc, o);
+        }
+        const float inv = rsqrtf(acc / static_cast<float>(dim) + eps);
+        for (uint32_t i = lane; i < dim; i += 16) {
+            float y = __fmul_rn(T::to_f32(x[i]), inv);
+            y = __fmul_rn(T::to_f32(w[i]), y);
+            if (b != nullptr) {
+                y = __fadd_rn(y, T::to_f32(b[i]));
+            }
+            out[off + i] = T::from_f32(y);
+        }
+    }
+}
+
 // one row by the 16 lanes of a group
 template <typename T>
 __device__ __forceinline__ void quantize_row(const uint16_t *x, int8_t *dst, float *scale_out, uint32_t head_dim,
@@ -447,6 +494,42 @@ extern "C" int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *
         quantize_to_cache_kernel<FP16><<<grid, 256, 0, as_stream(stream)>>>(
             static_cast<const uint16_t *>(inout), k_cache, v_cache, k_scale, v_scale, slot_mapping, num_tokens, n_heads,
             n_kv_heads, head_dim);
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+extern "C" int xlite_hip_qk_rms_norm(void *stream, const void *in, void *out, const void *q_norm,
+                                     const void *q_norm_bias, const void *k_norm, const void *k_norm_bias,
+                                     uint32_t num_tokens, uint32_t row_elems, uint32_t q_norm_dim,
+                                     uint32_t q_cnt_per_token, uint32_t k_norm_dim, uint32_t k_cnt_per_token,
+                                     uint32_t k_start_offset, float norm_eps, int dtype)
+{
+    XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype unsupported!");
+    if (num_tokens == 0 || q_cnt_per_token + k_cnt_per_token == 0) {
+        return XLITE_HIP_OK;
+    }
+    XL_REQUIRE(in && out, "null tensor");
+    XL_REQUIRE(q_cnt_per_token == 0 || (q_norm && q_norm_dim > 0), "Q segment needs a weight and a positive size");
+    XL_REQUIRE(k_cnt_per_token == 0 || (k_norm && k_norm_dim > 0), "K segment needs a weight and a positive size");
+    XL_REQUIRE(static_cast<uint64_t>(q_norm_dim) * q_cnt_per_token <= k_start_offset || k_cnt_per_token == 0,
+               "segments overlap");
+    XL_REQUIRE(static_cast<uint64_t>(k_start_offset) + static_cast<uint64_t>(k_norm_dim) * k_cnt_per_token <= row_elems &&
+                   static_cast<uint64_t>(q_norm_dim) * q_cnt_per_token <= row_elems,
+               "segments exceed the row");
+    const uint32_t grid = grid_for(static_cast<uint64_t>(num_tokens) * (q_cnt_per_token + k_cnt_per_token) * 16, 256);
+    auto launch = [&](auto tag) {
+        using T = decltype(tag);
+        qk_rms_norm_kernel<T><<<grid, 256, 0, as_stream(stream)>>>(
+            static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), static_cast<const uint16_t *>(q_norm),
+            static_cast<const uint16_t *>(q_norm_bias), static_cast<const uint16_t *>(k_norm),
+            static_cast<const uint16_t *>(k_norm_bias), num_tokens, row_elems, q_norm_dim, q_cnt_per_token, k_norm_dim,
+            k_cnt_per_token, k_start_offset, norm_eps);
+    };
+    if (dtype == XLITE_HIP_BF16) {
+        launch(BF16{});
+    } else {
+        launch(FP16{});
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

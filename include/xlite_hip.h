@@ -141,6 +141,22 @@ int xlite_hip_mla_v3(void *stream, const void *q_absorb, const void *qr, const v
                      size_t workspace_bytes);
 
 /* ------------------------------------------------------------------------
+ * qk_rms_norm — replaces XliteOpQkRmsNorm (xlite/csrc/op.cpp:1177-1203) + kernel
+ * qk_rms_norm.h:32-54 in its normalising mode without pre-reduced variances (the
+ * call of xlite/csrc/model.cpp:516-519): for every row of `in` [num_tokens, row_elems],
+ * RMSNorm of q_cnt_per_token vectors of q_norm_dim elements from column 0 with weight
+ * q_norm [q_norm_dim] (+ q_norm_bias or NULL), and of k_cnt_per_token vectors of
+ * k_norm_dim elements from column k_start_offset with k_norm (+ k_norm_bias or NULL):
+ * y = x * rsqrt(mean(x^2) + eps) * w + b in fp32. Results go to the same columns of
+ * `out` (same row pitch; may be `in`); other columns are not written.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_qk_rms_norm(void *stream, const void *in, void *out, const void *q_norm,
+                          const void *q_norm_bias, const void *k_norm, const void *k_norm_bias,
+                          uint32_t num_tokens, uint32_t row_elems, uint32_t q_norm_dim,
+                          uint32_t q_cnt_per_token, uint32_t k_norm_dim, uint32_t k_cnt_per_token,
+                          uint32_t k_start_offset, float norm_eps, int dtype);
+
+/* ------------------------------------------------------------------------
  * gather_sparse_kv_cache — replaces XliteOpGatherSparseKVCache
  * (xlite/csrc/op.cpp:1060-1084) + kernel gather_sparse_kv_cache.h:15-134.
  * dense[b, i] = paged[block_tables[b*max_num_blocks + tok / block_size], tok % block_size]

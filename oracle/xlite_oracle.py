@@ -25,6 +25,8 @@ piece of the reference (paths under /root/reference/):
   rope_complex_ref     xlite/tests/kernels/rope_complex.py:31-41 with the fp32 operation order of
                        xlite/csrc/kernels/rope_complex_and_cache.h:165-205
   mla_prepare_ref      xlite/tests/kernels/mla_prepare.py:27-45,90-109
+  qk_rms_norm_ref      xlite/csrc/kernels/qk_rms_norm.h:32-54 over rmsnorm_ref
+                       (xlite/tests/kernels/rmsnorm.py:24-30)
   einsum_ref           xlite/tests/kernels/einsum_mht_mhd.py:44
   prepare_attn_ref     xlite/csrc/runtime.cpp:438-534
   get_tile_size_of_cached_kv_ref  xlite/csrc/auto_tuner.cpp:10-210
@@ -42,7 +44,8 @@ tests/test_oracle_pins.py):
   rope_and_cache_ref, rope_complex_ref: C restatement with explicit bf16/fp16
       rounding (oracle/brute.c), rotation by position 0 is the identity, norm
       preservation, complex-multiply identity in fp64.
-  mla_prepare_ref: composition of the two pinned pieces + RMSNorm closed forms.
+  mla_prepare_ref, qk_rms_norm_ref: composition of pinned pieces + RMSNorm closed forms (a vector of
+      equal entries c normalises to sign(c) * w + b; scale invariance; per-vector Python loop).
   gather_*: brute-force Python loops.
   indexer_scores_ref: pure-Python triple loop in float (tiny case); one head with weight 1 reduces to
       q . k; with no intermediate rounding the weighted sum equals (sum_h w_h q_h) . k (linearity).
@@ -381,6 +384,22 @@ def rmsnorm_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: 
     var = xf.pow(2).mean(-1, keepdim=True)
     y = xf * torch.rsqrt(var + eps)
     return (weight.float() * y + bias.float()).to(x.dtype)
+
+
+def qk_rms_norm_ref(qkv, q_norm, q_norm_bias, k_norm, k_norm_bias, norm_eps, q_norm_dim, q_cnt_per_token,
+                    k_norm_dim, k_cnt_per_token, k_start_offset) -> torch.Tensor:
+    """xlite/csrc/kernels/qk_rms_norm.h:32-54 (two independent RMSNorm passes over disjoint column ranges of
+    the same rows), each pass the golden of xlite/tests/kernels/rmsnorm.py:24-30,49-51. Returns the new rows."""
+    out = qkv.clone()
+    T = qkv.shape[0]
+    zq = torch.zeros(q_norm_dim, dtype=qkv.dtype) if q_norm_bias is None else q_norm_bias
+    zk = torch.zeros(k_norm_dim, dtype=qkv.dtype) if k_norm_bias is None else k_norm_bias
+    qs = qkv[:, :q_norm_dim * q_cnt_per_token].reshape(T, q_cnt_per_token, q_norm_dim)
+    out[:, :q_norm_dim * q_cnt_per_token] = rmsnorm_ref(qs, q_norm, zq, norm_eps).reshape(T, -1)
+    k_end = k_start_offset + k_norm_dim * k_cnt_per_token
+    ks = qkv[:, k_start_offset:k_end].reshape(T, k_cnt_per_token, k_norm_dim)
+    out[:, k_start_offset:k_end] = rmsnorm_ref(ks, k_norm, zk, norm_eps).reshape(T, -1)
+    return out
 
 
 def mla_prepare_ref(attn_qkvc, q_norm, q_norm_bias, attn_norm_qc, kv_norm, kv_norm_bias,

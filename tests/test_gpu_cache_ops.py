@@ -180,3 +180,32 @@ def test_rope_and_cache_int8_quantise_on_write(rt, dtype, nH, nKV, d, rot):
     assert torch.equal(ks.cpu()[w], ks_ref[w]) and torch.equal(vs.cpu()[w], vs_ref[w])
     assert bool((kq.cpu()[~w] == 9).all()) and bool((vq.cpu()[~w] == -9).all())
     assert bool((ks.cpu()[~w] == 5.0).all()) and bool((vs.cpu()[~w] == -5.0).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nH,nKV,d,bias,full", [(32, 8, 128, True, False), (14, 2, 64, False, False), (16, 4, 128, False, True)])
+def test_qk_rms_norm(rt, dtype, nH, nKV, d, bias, full):
+    """Per-head (xlite/csrc/model.cpp:516-519) and whole-segment granularity; V columns bit-identical; the
+    normalised values within one 16-bit unit of the oracle (the fp32 sum of squares is reduced in another
+    order), as for mla_prepare."""
+    from gvirt_amd._C import qk_rms_norm
+    g = torch.Generator().manual_seed(400 + nH + d)
+    T = 41
+    x = torch.randn(T, (nH + 2 * nKV) * d, generator=g).to(dtype)
+    qd, qc, kd, kc_ = (nH * d, 1, nKV * d, 1) if full else (d, nH, d, nKV)
+    wq, wk = torch.randn(qd, generator=g).to(dtype), torch.randn(kd, generator=g).to(dtype)
+    bq = torch.randn(qd, generator=g).to(dtype) if bias else None
+    bk = torch.randn(kd, generator=g).to(dtype) if bias else None
+    ref = O.qk_rms_norm_ref(x, wq, bq, wk, bk, 1e-6, qd, qc, kd, kc_, nH * d)
+    dev = x.to(DEV)
+    mv = lambda t: None if t is None else t.to(DEV)
+    qk_rms_norm(rt, dev, mv(wq), mv(bq), mv(wk), mv(bk), dev, 1e-6, qd, qc, kd, kc_, nH * d)   # in place
+    got = dev.cpu()
+    assert torch.equal(_bits(got[:, (nH + nKV) * d:]), _bits(x[:, (nH + nKV) * d:]))
+    torch.testing.assert_close(got[:, :(nH + nKV) * d].float(), ref[:, :(nH + nKV) * d].float(), atol=2e-5,
+                               rtol=1e-3 if dtype == torch.float16 else 8e-3)
+    # into a separate output: only the two segments are written
+    out = torch.full_like(dev, 7.0)
+    qk_rms_norm(rt, x.to(DEV), mv(wq), mv(bq), mv(wk), mv(bk), out, 1e-6, qd, qc, kd, kc_, nH * d)
+    assert torch.equal(_bits(out.cpu()[:, :(nH + nKV) * d]), _bits(got[:, :(nH + nKV) * d]))
+    assert bool((out.cpu()[:, (nH + nKV) * d:] == 7.0).all())

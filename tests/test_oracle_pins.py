@@ -364,3 +364,29 @@ def test_indexer_topk_pins():
                 assert not ties_out or max(ties_in) < min(ties_out)
                 top = torch.topk(s[r], 10).values
                 assert sorted(float(s[r, j]) for j in sel) == sorted(top.tolist())
+
+
+def test_qk_rms_norm_pins():
+    torch.manual_seed(8)
+    nH, nKV, d = 3, 2, 16
+    x = torch.randn(5, (nH + 2 * nKV) * d).bfloat16()
+    wq, wk = torch.randn(d).bfloat16(), torch.randn(d).bfloat16()
+    bq = torch.randn(d).bfloat16()
+    got = O.qk_rms_norm_ref(x, wq, bq, wk, None, 1e-6, d, nH, d, nKV, nH * d)
+    # V columns untouched; every Q / K vector by a plain Python loop in double precision
+    assert torch.equal(got[:, (nH + nKV) * d:], x[:, (nH + nKV) * d:])
+    for t in range(5):
+        for h in range(nH + nKV):
+            v = x[t, h * d:(h + 1) * d].double()
+            w = (wq if h < nH else wk).double()
+            b = bq.double() if h < nH else torch.zeros(d, dtype=torch.double)
+            ref = v / math.sqrt(float((v * v).sum()) / d + 1e-6) * w + b
+            torch.testing.assert_close(got[t, h * d:(h + 1) * d].double(), ref, rtol=2 ** -7, atol=1e-6)
+    # closed form: equal entries c -> sign(c) * w + b (eps negligible)
+    c = torch.full((1, (nH + 2 * nKV) * d), -3.0).bfloat16()
+    one = O.qk_rms_norm_ref(c, wq, bq, wk, None, 1e-12, d, nH, d, nKV, nH * d)
+    torch.testing.assert_close(one[0, :d].float(), (-wq.float() + bq.float()).bfloat16().float(), rtol=2 ** -7, atol=1e-6)
+    # the whole-segment form (one vector per segment) differs from the per-head form
+    full = O.qk_rms_norm_ref(x, torch.ones(nH * d).bfloat16(), None, torch.ones(nKV * d).bfloat16(), None, 1e-6,
+                             nH * d, 1, nKV * d, 1, nH * d)
+    torch.testing.assert_close(full[:, :nH * d].float().pow(2).mean(-1), torch.ones(5), rtol=2e-2, atol=0)
