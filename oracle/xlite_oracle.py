@@ -19,6 +19,8 @@ piece of the reference (paths under /root/reference/):
   mla_v2_ref           xlite/csrc/_C.cpp:1234-1301 (einsum + attention + einsum)
   mla_v3_ref           xlite/tests/kernels/mla_v3.py:163-192; xlite/csrc/kernels/mla_v3.h:534-536
   gather_sparse_kv_cache_ref  xlite/tests/kernels/gather_sparse_kv_cache.py:102-116
+  mha_forward_ref      xlite/csrc/model.cpp:480-600 (composition of the pieces; the projections are fp32
+                       matrix products rounded once)
   indexer_scores_ref   xlite/tests/kernels/indexer_scores.py:96-118 (golden) with the 16-bit rounding of
                        the per-head products of xlite/csrc/kernels/indexer_scores.h:214-217
   indexer_topk_ref     xlite/tests/kernels/indexer_topk.py:139-152
@@ -302,6 +304,31 @@ def gather_sparse_kv_cache_ref(k_cache, pe_cache, block_tables, topk_indices, qu
             phys = int(tables[b, tok // block_size])
             kd[b, i] = kc[phys, tok % block_size]
             pd[b, i] = pc[phys, tok % block_size]
+
+
+# --------------------------------------------------------------------------
+# model-level caller
+# --------------------------------------------------------------------------
+def mha_forward_ref(hidden, wqkv, wo, k_cache, v_cache, lens, cached_lens, block_tables, cosin, n_heads, n_kv_heads,
+                    head_dim, rot_dim, block_size, q_norm=None, k_norm=None, norm_eps=1e-6):
+    """xlite/csrc/model.cpp:480-600 as a composition of the pieces above: metadata (prepare_attn_ref), QKV
+    projection (fp32 accumulate, one rounding), optional per-head qk RMSNorm, rope_and_cache (in place on the
+    caches), attention, output projection. `block_tables[i]` lists the blocks of sequence i."""
+    dt = hidden.dtype
+    meta = prepare_attn_ref(lens, cached_lens, block_tables, block_size)
+    qkv = (hidden.float() @ wqkv.float()).to(dt)
+    if q_norm is not None:
+        qkv = qk_rms_norm_ref(qkv, q_norm, None, k_norm, None, norm_eps, head_dim, n_heads, head_dim, n_kv_heads,
+                              n_heads * head_dim)
+    pos = torch.tensor(meta["position"], dtype=torch.int64)
+    slots = torch.tensor(meta["slot_mapping"], dtype=torch.int32)
+    rope_and_cache_ref(qkv, k_cache, v_cache, pos, cosin, slots, n_heads, n_kv_heads, head_dim, rot_dim, block_size)
+    batch = len(lens)
+    attn = attention_ref(qkv, k_cache, v_cache, torch.tensor(meta["query_start_loc"], dtype=torch.int32),
+                         torch.tensor(list(lens), dtype=torch.int32), torch.tensor(list(cached_lens), dtype=torch.int32),
+                         torch.from_numpy(meta["block_tables"]).flatten(), n_heads, n_kv_heads, head_dim, block_size, batch,
+                         meta["max_num_blocks"])
+    return (attn.to(dt).float().reshape(hidden.shape[0], -1) @ wo.float()).to(dt)
 
 
 # --------------------------------------------------------------------------
