@@ -209,80 +209,133 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
         }
         return;
     }
-    // ---- the k-th largest key: high byte, then low byte
+    // ---- the k-th largest key: high byte, then low byte. Threads read eight keys (16 bytes) at a time.
+    const uint32_t n8 = ld_scores % 8 == 0 ? n & ~7u : 0u;   // vector loads need 16-byte aligned rows
     uint32_t prefix = 0, above = 0;   // keys whose high byte equals `prefix` are the candidates of pass 2
     for (int pass = 0; pass < 2; pass++) {
         hist[threadIdx.x] = 0;
         __syncthreads();
-        for (uint32_t j = threadIdx.x; j < n; j += kSelThreads) {
-            const uint32_t key = order_key(row[j]);
+        auto count = [&](uint32_t key) {
             if (pass == 0) {
                 atomicAdd(&hist[key >> 8], 1u);
             } else if ((key >> 8) == prefix) {
                 atomicAdd(&hist[key & 0xffu], 1u);
             }
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            uint32_t cum = above;
-            int b = 255;
-            for (; b > 0; b--) {
-                if (cum + hist[b] >= top_k) {
-                    break;
-                }
-                cum += hist[b];
+        };
+        for (uint32_t j = threadIdx.x * 8; j < n8; j += kSelThreads * 8) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(row + j);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                count(order_key(static_cast<uint16_t>(w[e] & 0xffffu)));
+                count(order_key(static_cast<uint16_t>(w[e] >> 16)));
             }
-            sel[0] = static_cast<uint32_t>(b);
-            sel[1] = cum;
+        }
+        for (uint32_t j = n8 + threadIdx.x; j < n; j += kSelThreads) {
+            count(order_key(row[j]));
         }
         __syncthreads();
-        if (pass == 0) {
-            prefix = sel[0];
-        } else {
-            prefix = (prefix << 8) | sel[0];
+        // the bin that holds the k-th key, counted from the top: a suffix sum over the 256 bins by one wave
+        if (threadIdx.x < 64) {
+            const uint32_t b0 = 255 - 4 * threadIdx.x;   // this lane's four bins, highest first
+            const uint32_t c0 = hist[b0], c1 = hist[b0 - 1], c2 = hist[b0 - 2], c3 = hist[b0 - 3];
+            uint32_t incl = c0 + c1 + c2 + c3;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(incl, d);
+                incl += threadIdx.x >= static_cast<uint32_t>(d) ? up : 0;
+            }
+            uint32_t cum = above + incl - (c0 + c1 + c2 + c3);   // keys in the bins above this lane's
+            const uint32_t cs[4] = {c0, c1, c2, c3};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (cum < top_k && cum + cs[e] >= top_k) {
+                    sel[0] = b0 - e;
+                    sel[1] = cum;
+                }
+                cum += cs[e];
+            }
         }
+        __syncthreads();
+        prefix = pass == 0 ? sel[0] : ((prefix << 8) | sel[0]);
         above = sel[1];
         __syncthreads();
     }
     const uint32_t thr = prefix;            // the k-th largest key
     const uint32_t need = top_k - above;    // ties of it to take, lowest positions first
-    // ---- ordered output
+    // ---- ordered output: 1024 positions per round, four consecutive ones per thread
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t done = 0, ties = 0;   // running totals, the same in every thread
-    for (uint32_t base = 0; base < n; base += kSelThreads) {
-        const uint32_t j = base + threadIdx.x;
-        const uint32_t key = j < n ? order_key(row[j]) : 0u;
-        const bool gt = j < n && key > thr;
-        const bool eq = j < n && key == thr;
-        const uint64_t m_eq = __ballot(eq);
-        const uint32_t eq_before = __builtin_popcountll(m_eq & ((1ull << lane) - 1));
-        if (lane == 0) {
-            wave_cnt[0][wave] = __builtin_popcountll(m_eq);
+    for (uint32_t base = 0; base < n; base += kSelThreads * 4) {
+        const uint32_t j0 = base + threadIdx.x * 4;
+        uint32_t key[4];
+        if (j0 + 4 <= n8) {
+            const uint2 v = *reinterpret_cast<const uint2 *>(row + j0);
+            key[0] = order_key(static_cast<uint16_t>(v.x & 0xffffu));
+            key[1] = order_key(static_cast<uint16_t>(v.x >> 16));
+            key[2] = order_key(static_cast<uint16_t>(v.y & 0xffffu));
+            key[3] = order_key(static_cast<uint16_t>(v.y >> 16));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                key[e] = j0 + e < n ? order_key(row[j0 + e]) : 0u;   // key 0 is below every threshold reached here
+            }
+        }
+        uint32_t n_eq = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            n_eq += (j0 + e < n && key[e] == thr) ? 1u : 0u;
+        }
+        // ties before this thread: wave prefix, then the waves before
+        uint32_t eq_incl = n_eq;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(eq_incl, d);
+            eq_incl += lane >= static_cast<uint32_t>(d) ? up : 0;
+        }
+        if (lane == 63) {
+            wave_cnt[0][wave] = eq_incl;
         }
         __syncthreads();
-        uint32_t eq_rank = ties + eq_before, eq_total = 0;
+        uint32_t eq_rank = ties + eq_incl - n_eq, eq_total = 0;
 #pragma unroll
         for (uint32_t w = 0; w < kSelThreads / 64; w++) {
             const uint32_t c = wave_cnt[0][w];
             eq_rank += w < wave ? c : 0;
             eq_total += c;
         }
-        const bool take = gt || (eq && eq_rank < need);
-        const uint64_t m_tk = __ballot(take);
-        const uint32_t tk_before = __builtin_popcountll(m_tk & ((1ull << lane) - 1));
-        if (lane == 0) {
-            wave_cnt[1][wave] = __builtin_popcountll(m_tk);
+        bool take[4];
+        uint32_t n_tk = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const bool in = j0 + e < n;
+            const bool eq = in && key[e] == thr;
+            take[e] = in && (key[e] > thr || (eq && eq_rank < need));
+            eq_rank += eq ? 1u : 0u;
+            n_tk += take[e] ? 1u : 0u;
+        }
+        uint32_t tk_incl = n_tk;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(tk_incl, d);
+            tk_incl += lane >= static_cast<uint32_t>(d) ? up : 0;
+        }
+        if (lane == 63) {
+            wave_cnt[1][wave] = tk_incl;
         }
         __syncthreads();
-        uint32_t o = done + tk_before, tk_total = 0;
+        uint32_t o = done + tk_incl - n_tk, tk_total = 0;
 #pragma unroll
         for (uint32_t w = 0; w < kSelThreads / 64; w++) {
             const uint32_t c = wave_cnt[1][w];
             o += w < wave ? c : 0;
             tk_total += c;
         }
-        if (take && o < top_k) {
-            out[o] = indices[j];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (take[e] && o < top_k) {
+                out[o++] = indices[j0 + e];
+            }
         }
         done += tk_total;
         ties += eq_total;
