@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c3|c4|c5|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c3|c4|c5|idx|all]
 
 Default (what the driver runs): configuration 2 of BASELINE.json — Llama-3-8B-shape GQA
 flash-decode, batch 64, every sequence at context 4096, bf16 paged KV cache with block size 128,
@@ -238,6 +238,49 @@ def bench_mla(args, torch, rt):
             "cpu_baseline": None}
 
 
+def bench_indexer(args, torch, rt):
+    """DSA indexer on the decode batch of configuration 4 (64 indexer heads of 128, one key head): the
+    `indexer_topk` operator (scores + selection of 2048 positions per row). Not a BASELINE configuration:
+    printed only with --config idx."""
+    import numpy as np
+    from gvirt_amd import workloads as W
+    from gvirt_amd import _C
+    dev = "cuda:0"
+    ctx = W.c4_context_lengths()
+    nH, D, bs, top_k = 64, 128, 64, 2048
+    batch = len(ctx)
+    maxblk = max((c + bs - 1) // bs for c in ctx)
+    NB = batch * maxblk + 1
+    g = torch.Generator(device=dev).manual_seed(W.SEED_BASE + 6)
+    q = torch.randn(batch, nH, D, generator=g, device=dev).bfloat16()
+    wgt = torch.randn(batch, D + nH, generator=g, device=dev).bfloat16()
+    kc = torch.randn(NB, bs, D, generator=g, device=dev).bfloat16()
+    tables = torch.randperm(NB, generator=g, device=dev)[: batch * maxblk].int()
+    qsl = torch.arange(batch, dtype=torch.int32, device=dev)
+    lens = torch.ones(batch, dtype=torch.int32, device=dev)
+    clens = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=dev)
+    idx = torch.arange(maxblk * bs, dtype=torch.int32, device=dev)
+    out = torch.zeros(batch, top_k, dtype=torch.int32, device=dev)
+    rt.blocking = False
+
+    def step():
+        _C.indexer_topk(rt, q, kc, wgt, idx, out, qsl, lens, clens, tables, nH, D, bs, batch, maxblk, top_k)
+
+    for _ in range(args.warmup):
+        step()
+    ms = _time_region(torch, step, args.steps)
+    kbytes = sum(ctx) * D * 2
+    gbs = kbytes / (ms * 1e-3) / 1e9
+    return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
+            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "idx DSA indexer_topk on the c4 decode batch", "batch": batch, "n_heads": nH, "head_dim": D,
+                       "top_k": top_k, "ctx_total": int(sum(ctx)), "key_bytes_per_step": int(kbytes)},
+            "roofline": {"bound": "hbm", "kernel": "indexer_scores_kernel (+ indexer_select_kernel)", "achieved": round(gbs, 2),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+            "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -283,6 +326,8 @@ def main():
             out = bench_prefill(args, torch, rt)
         elif c == "c4":
             out = bench_mla(args, torch, rt)
+        elif c == "idx":
+            out = bench_indexer(args, torch, rt)
         else:
             raise SystemExit("unknown config " + c)
         print(json.dumps(out), flush=True)
