@@ -180,3 +180,23 @@ def test_mla_topk_index_mask(rt, nH, work, top_k):
     ref = O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"],
                               c["R"], c["C"], c["bs"], c["batch"], c["maxblk"], scale, topk, top_k)
     check(out.float().cpu(), ref)
+
+
+def test_mla_decode_large_batch_of_short_sequences(rt):
+    """More rows than threads in the work-splitting scan (two rows per thread), chunks that span many rows,
+    and rows far shorter than a step."""
+    g = np.random.default_rng(5)
+    B = 700
+    clens = [int(x) for x in g.integers(0, 90, size=B)]
+    clens[3] = 0
+    c = mla_case(33, [1] * B, clens, 16, bs=32)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
+def test_mla_decode_one_long_row_among_short_ones(rt):
+    """A chunk boundary inside a long row and many short rows inside one chunk."""
+    clens = [5, 9000, 17, 300, 2, 64, 1000]
+    c = mla_case(34, [1] * len(clens), clens, 16, bs=64)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
