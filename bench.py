@@ -195,6 +195,38 @@ def bench_prefill(args, torch, rt):
     flops = sum(w["flops"] for w in chunks)
     tokens = sum(w["tokens"] for w in chunks)
     tf = flops / (ms * 1e-3) / 1e12
+    cpu = None
+    if not args.no_cpu:
+        # the oracle on the shortest sequence's part of the first chunk: parity, then its rate
+        sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+        from oracle import xlite_oracle as O
+        ncpu = _cpu_threads(torch)
+        torch.cuda.synchronize()
+        w0 = chunks[0]
+        c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in w0.items() if k != "caches"}
+        i = min(range(len(lens)), key=lambda j: lens[j])
+        got = w0["output"].float().cpu()
+
+        def run_oracle():
+            return O.attention_ref(c["qkv"], c["k_cache"], c["v_cache"], c["query_start_loc"], c["lens"], c["cached_lens"],
+                                   c["block_tables"], shape.n_heads, shape.n_kv_heads, shape.head_dim, shape.block_size,
+                                   w0["batch"], w0["max_num_block"], seqs=[i])
+        ref = run_oracle()
+        r0, rl = int(c["query_start_loc"][i]), int(c["lens"][i])
+        err = (got[r0:r0 + rl] - ref[r0:r0 + rl]).abs()
+        if float(err.max()) > 2e-2:
+            raise SystemExit("parity check failed in bench: max abs err %g" % float(err.max()))
+        reps, t_cpu = 0, 0.0
+        while reps < 3 and t_cpu < 20.0:
+            t1 = time.perf_counter()
+            run_oracle()
+            t_cpu += time.perf_counter() - t1
+            reps += 1
+        sample_flops = 4 * shape.n_heads * shape.head_dim * (rl * (rl + 1) // 2)
+        cpu = {"value": round(sample_flops / (t_cpu / reps) / 1e12, 4), "unit": "TFLOP/s", "cores": ncpu, "kind": "port",
+               "sample": "sequence %d of the first chunk (%d rows, causal), %d timed runs of the PyTorch oracle, %s" %
+                         (i, rl, reps, _cpu_info()),
+               "max_abs_err_vs_gpu": float(err.max())}
     return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(tf, 2),
             "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": max(1, args.warmup // 4), "ms_per_step": round(ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -204,7 +236,7 @@ def bench_prefill(args, torch, rt):
             "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                          "traffic": None, "algorithmic_flops_per_step": int(flops)},
-            "cpu_baseline": None}
+            "cpu_baseline": cpu}
 
 
 def bench_mla(args, torch, rt):
@@ -225,6 +257,40 @@ def bench_mla(args, torch, rt):
     ms = _time_region(torch, step, args.steps)
     gbs = w["kv_bytes"] / (ms * 1e-3) / 1e9
     tf = w["flops"] / (ms * 1e-3) / 1e12
+    cpu = None
+    if not args.no_cpu:
+        # the oracle (the checker, not the thing measured) on two of the sequences: parity, then its rate
+        sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+        from oracle import xlite_oracle as O
+        ncpu = _cpu_threads(torch)
+        torch.cuda.synchronize()
+        sample = [0, len(ctx) // 2]
+        c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in w.items()}
+        mb = w["max_num_blocks"]
+        sub_tables = torch.cat([c["block_tables"].view(len(ctx), mb)[i] for i in sample])
+        sub = lambda t: torch.stack([t[i] for i in sample])
+
+        def run_oracle():
+            return O.mla_attention_ref(sub(c["q_absorb"]), sub(c["qr"]), c["k_cache"], c["pe_cache"],
+                                       torch.arange(len(sample), dtype=torch.int32), torch.ones(len(sample), dtype=torch.int32),
+                                       sub(c["cached_lens"]), sub_tables, s.n_heads, s.rope_head_dim, s.kv_lora_rank,
+                                       s.block_size, len(sample), mb, s.scale)
+        ref = run_oracle()
+        got = sub(w["o_absorb"].float().cpu()).reshape(ref.shape)
+        err = (got - ref).abs()
+        if float(err.max()) > 2e-2:
+            raise SystemExit("parity check failed in bench: max abs err %g" % float(err.max()))
+        reps, t_cpu = 0, 0.0
+        while reps < 3 and t_cpu < 20.0:
+            t1 = time.perf_counter()
+            run_oracle()
+            t_cpu += time.perf_counter() - t1
+            reps += 1
+        sample_bytes = sum(ctx[i] for i in sample) * (s.kv_lora_rank + s.rope_head_dim) * 2
+        cpu = {"value": round(sample_bytes / (t_cpu / reps) / 1e9, 3), "unit": "GB/s", "cores": ncpu, "kind": "port",
+               "sample": "%d of %d sequences (indices %s), %d timed runs of the PyTorch oracle, %s" %
+                         (len(sample), len(ctx), sample, reps, _cpu_info()),
+               "max_abs_err_vs_gpu": float(err.max())}
     floor_ms = max(w["kv_bytes"] / (HBM_PEAK_GBS * 1e9), w["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12)) * 1e3
     return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
             "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
@@ -235,7 +301,7 @@ def bench_mla(args, torch, rt):
             "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_norm16_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c4"),
                          "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
-            "cpu_baseline": None}
+            "cpu_baseline": cpu}
 
 
 def bench_indexer(args, torch, rt):
