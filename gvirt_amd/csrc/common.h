@@ -14,6 +14,8 @@ namespace xlite {
 // ---- error plumbing ---------------------------------------------------------
 void set_error(const std::string &msg);
 int fail(int code, const char *func, const std::string &msg);
+// allows `bytes` of dynamic LDS for `kernel` on the current device (once per kernel, device and size)
+int ensure_dynamic_lds(const void *kernel, size_t bytes);
 
 #define XL_REQUIRE(cond, msg)                                                      \
     do {                                                                           \

@@ -748,11 +748,8 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) + (p.tile_tokens / kStep + 2) * sizeof(uint32_t);
     auto kernel = decode_dma_kernel<T>;
-    static size_t configured = 0;
-    if (configured < lds) {
-        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        configured = lds;
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
+        return rc;
     }
     dim3 grid(p.max_slots, batch, 1);
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
@@ -767,11 +764,8 @@ int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
                        (p.tile_tokens / kStep + 2) * sizeof(uint32_t);
     auto kernel = decode_mfma_kernel<T, D, KV8, MULTI_SUB>;
     if (lds > 64 * 1024) {
-        static size_t configured = 0;
-        if (configured < lds) {
-            XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            configured = lds;
+        if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
+            return rc;
         }
     }
     dim3 grid(ceil_div(p.max_slots, p.n_sub), batch, 1);

@@ -5,6 +5,10 @@
 #include <cstring>
 #include <vector>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "common.h"
 
 namespace xlite {
@@ -12,6 +16,23 @@ namespace xlite {
 static thread_local std::string g_last_error;
 
 void set_error(const std::string &msg) { g_last_error = msg; }
+
+// Dynamic LDS above 64 KiB has to be allowed per kernel function and per device; remember the largest
+// request granted for each pair.
+int ensure_dynamic_lds(const void *kernel, size_t bytes)
+{
+    static std::mutex mu;
+    static std::map<std::pair<const void *, int>, size_t> granted;
+    int dev = 0;
+    XL_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mu);
+    size_t &have = granted[std::make_pair(kernel, dev)];
+    if (have < bytes) {
+        XL_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+        have = bytes;
+    }
+    return XLITE_HIP_OK;
+}
 
 int fail(int code, const char *func, const std::string &msg)
 {

@@ -360,11 +360,8 @@ int launch_kernel(hipStream_t stream, const MfmaParams &p, dim3 grid)
     constexpr size_t lds = lds_bytes<DQ0 + DQ1, DV, BN>();
     auto kernel = mfma_attention_kernel<T, DQ0, DQ1, DV, BN, SEPARATE_V>;
     if (lds > 64 * 1024) {
-        static bool configured = false;  // per instantiation
-        if (!configured) {
-            XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            configured = true;
+        if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
+            return rc;
         }
     }
     kernel<<<grid, kThreads, lds, stream>>>(p);

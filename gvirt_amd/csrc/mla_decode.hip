@@ -607,15 +607,16 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
 
     // one workgroup per compute unit (the LDS ring allows no more)
     const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + kTblCap * sizeof(uint32_t);
-    static int n_cu = 0;
-    if (n_cu == 0) {
-        int dev = 0, cus = 0;
-        XL_HIP(hipGetDevice(&dev));
-        XL_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        // the kernel also has a few words of static LDS: ask for exactly the dynamic part
-        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mla_decode_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        n_cu = cus;
+    int dev = 0;
+    XL_HIP(hipGetDevice(&dev));
+    thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
+    if (cu_dev != dev) {
+        XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+        cu_dev = dev;
+    }
+    // the kernel also has a few words of static LDS: ask for exactly the dynamic part
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(mla_decode_kernel), lds)) {
+        return rc;
     }
     mla_decode_kernel<<<dim3(static_cast<uint32_t>(n_cu), 1, 1), kNT, lds, stream>>>(p);
     XL_LAUNCH_CHECK();

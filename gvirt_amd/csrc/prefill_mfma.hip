@@ -444,13 +444,9 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     const size_t lds = static_cast<size_t>(kStages) * STAGE + (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     const bool bf = a.dtype == XLITE_HIP_BF16;
     XL_REQUIRE(lds <= 160 * 1024, "block table too long for the prefill kernel");
-    static size_t configured = 0;
-    if (configured < lds) {
-        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_kernel<BF16>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        XL_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_kernel<FP16>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        configured = lds;
+    if (const int rc = ensure_dynamic_lds(bf ? reinterpret_cast<const void *>(prefill_kernel<BF16>)
+                                             : reinterpret_cast<const void *>(prefill_kernel<FP16>), lds)) {
+        return rc;
     }
     uint32_t n_wg;
     if (a.n_kv_heads % kXcds == 0) {
