@@ -57,19 +57,31 @@ struct Mma<FP16> {
     }
 };
 
-// The sequence that owns query row t, and its number of candidate positions.
+// The sequence that owns query row t, and its number of candidate positions. query_start_loc is a prefix sum
+// (non-decreasing): the owner is the last sequence that starts at or before t, if t lies inside it.
 __device__ __forceinline__ bool find_row(uint32_t t, const int32_t *query_start_loc, const int32_t *lens,
                                          const int32_t *cached_lens, uint32_t batch, uint32_t *seq, uint32_t *total)
 {
-    for (uint32_t i = 0; i < batch; i++) {
-        const int32_t s = query_start_loc[i], l = lens[i];
-        if (static_cast<int32_t>(t) >= s && static_cast<int32_t>(t) < s + l) {
-            *seq = i;
-            *total = static_cast<uint32_t>(cached_lens[i] + l);
-            return true;
+    uint32_t lo = 0, hi = batch;   // first index in [lo, hi) whose start is beyond t
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) / 2;
+        if (query_start_loc[mid] <= static_cast<int32_t>(t)) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
         }
     }
-    return false;
+    if (lo == 0) {
+        return false;
+    }
+    const uint32_t i = lo - 1;
+    const int32_t s = query_start_loc[i], l = lens[i];
+    if (static_cast<int32_t>(t) >= s + l) {
+        return false;
+    }
+    *seq = i;
+    *total = static_cast<uint32_t>(cached_lens[i] + l);
+    return true;
 }
 
 // NT = n_heads / 16, head_dim = 128.

@@ -33,13 +33,24 @@ topk_gather_kernel(const uint4 *__restrict__ k_cache, const uint4 *__restrict__ 
     uint32_t seq = 0;
     int32_t r = 0;
     bool found = false;
-    for (uint32_t i = 0; i < batch; i++) {
-        const int32_t s = query_start_loc[i], l = lens[i];
-        if (static_cast<int32_t>(t) >= s && static_cast<int32_t>(t) < s + l) {
-            seq = i;
-            r = static_cast<int32_t>(t) - s;
-            found = true;
-            break;
+    {
+        // query_start_loc is a prefix sum: the owner is the last sequence that starts at or before t
+        uint32_t lo = 0, hi = batch;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) / 2;
+            if (query_start_loc[mid] <= static_cast<int32_t>(t)) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        if (lo > 0) {
+            const int32_t s = query_start_loc[lo - 1], l = lens[lo - 1];
+            if (static_cast<int32_t>(t) < s + l) {
+                seq = lo - 1;
+                r = static_cast<int32_t>(t) - s;
+                found = true;
+            }
         }
     }
     const uint32_t limit = found ? static_cast<uint32_t>(cached_lens[seq] + r + 1) : 0u;
