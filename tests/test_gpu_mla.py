@@ -200,3 +200,38 @@ def test_mla_decode_one_long_row_among_short_ones(rt):
     c = mla_case(34, [1] * len(clens), clens, 16, bs=64)
     scale = 192 ** -0.5
     check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
+def test_dsa_decode_pipeline_indexer_to_masked_mla(rt):
+    """DeepSeek sparse attention, decode step: indexer_topk picks the positions, mla_attention attends to
+    them (xlite/csrc/model.cpp:384-427). The lists go from one operator to the other untouched; the result is
+    checked against the oracle attention on the same lists, and the lists against the oracle's own."""
+    from gvirt_amd._C import indexer_topk, mla_attention
+    clens, lens, top_k, bs = [3000, 2100, 500, 1023], [1, 1, 1, 1], 1024, 64
+    c = mla_case(51, lens, clens, 16, bs=bs)
+    g = torch.Generator().manual_seed(52)
+    NB = c["kc"].shape[0]
+    iq = torch.randn(c["T"], 64, 128, generator=g).bfloat16()
+    iw = torch.randn(c["T"], 128 + 64, generator=g).bfloat16()
+    ik = torch.randn(NB, bs, 128, generator=g).bfloat16()
+    ld = c["maxblk"] * bs
+    lists = torch.full((c["T"], top_k), -1, dtype=torch.int32, device=DEV)
+    dev = lambda t: t.to(DEV)
+    meta = (dev(c["qsl"]), dev(c["lens"]), dev(c["clens"]), dev(c["tables"]))
+    indexer_topk(rt, dev(iq), dev(ik), dev(iw), torch.arange(ld, dtype=torch.int32, device=DEV), lists, *meta, 64, 128, bs,
+                 c["batch"], c["maxblk"], top_k)
+    scale = 192 ** -0.5
+    out = torch.zeros(c["T"], c["nH"], c["C"], dtype=torch.bfloat16, device=DEV)
+    mla_attention(rt, dev(c["qa"]), dev(c["qr"]), dev(c["kc"]), dev(c["pc"]), out, *meta, c["nH"], c["R"], c["C"], bs,
+                  c["batch"], c["maxblk"], scale, lists, top_k)
+    rt.synchronize()
+    got_lists = lists.cpu()
+    ref = O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"],
+                              c["R"], c["C"], bs, c["batch"], c["maxblk"], scale, got_lists.clamp(min=0), top_k)
+    check(out.float().cpu(), ref)
+    want = O.indexer_topk_ref(O.indexer_scores_ref(iq, ik, iw, c["qsl"], c["lens"], c["clens"], c["tables"], 64, 128, bs,
+                                                   c["batch"], c["maxblk"]), top_k)
+    for i in range(c["batch"]):
+        n = clens[i] + 1
+        row = got_lists[i, :min(top_k, n)].tolist()
+        assert len(set(want[i][0]) - set(row)) * 100.0 <= 3.0 * len(row)
