@@ -112,6 +112,8 @@ int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, cons
  * listed positions (ascending, inside the range); shorter rows see their whole range
  * (xlite/csrc/kernels/mla_v2.h:697-699). The listed rows are gathered into the workspace
  * first, so the workspace size depends on top_k. bf16 only (xlite/csrc/op.cpp:1014).
+ * workspace: at least xlite_hip_mla_workspace_bytes() for the same shape (required:
+ * XLITE_HIP_ENOSPC otherwise; split-KV partials, no initialisation needed).
  * ---------------------------------------------------------------------- */
 size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t kv_lora_rank,
                                      uint32_t rope_head_dim, uint32_t block_size, uint32_t batch,
