@@ -117,8 +117,8 @@ extern "C" size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t 
     const uint32_t max_ctx = max_num_blocks * block_size;
     const uint32_t splits = mfma_pick_splits(total_tokens, n_heads, batch, 1, max_ctx, 32);
     size_t need = mfma_workspace_bytes(total_tokens, n_heads, kv_lora_rank, splits + 1);
-    if (total_tokens == batch && block_size > 0) {
-        // the decode kernel plans its own tiles; block_size == 1 describes a dense cache of
+    if (block_size > 0) {
+        // the decode kernel plans its own work split; block_size == 1 describes a dense cache of
         // max_num_blocks rows per sequence
         MlaArgs a{};
         a.total_tokens = total_tokens;

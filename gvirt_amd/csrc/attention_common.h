@@ -55,9 +55,10 @@ size_t partial_bytes(uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_
 PartialBuffers carve_partials(void *workspace, uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots);
 int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
                  uint32_t n_heads, uint32_t dv, uint32_t max_slots);
-// acc holds O / l in the 16-bit activation type ([rows * n_heads][max_slots][dv], in the same allocation)
-int launch_merge_norm16(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
-                        uint32_t n_heads, uint32_t dv, uint32_t max_slots);
+// Partials of the MLA decode kernel: a row's s-th segment sits in slot 2 c0 + (1 - first flag) for s = 0 and
+// 2 (c0 + s) after that (meta = segments, c0, first flag per row); acc holds O / l in the 16-bit activation type.
+int launch_merge_mla(hipStream_t stream, int dtype, void *out, const uint16_t *acc, const float *ml, const int32_t *meta,
+                     uint32_t rows, uint32_t n_heads, uint32_t dv);
 
 // decode_attention.hip
 bool decode_supported(uint32_t head_dim);
@@ -88,16 +89,16 @@ struct MlaDecodeParams {
     const int32_t *lens;
     const int32_t *cached_lens;
     const int32_t *block_tables;   // nullptr: dense cache, dense_len rows per sequence, no causality
-    int32_t *part_cnt;
-    float *part_acc;
-    float *part_ml;
+    int32_t *part_meta;   // [total_rows][4]: segments of the row (0: stored directly), first chunk, first-in-chunk flag
+    float *part_acc;      // [2 * chunks][n_heads][512] 16-bit, O / l of a partial slot
+    float *part_ml;       // [2 * chunks][n_heads][2]: running maximum (log2 domain), sum
     uint32_t n_heads;
     uint32_t batch;
+    uint32_t total_rows;
     uint32_t block_size;
     uint32_t max_num_blocks;
     uint32_t dense_len;
     uint32_t chunk_min_steps;
-    uint32_t max_slots;
     float scale_log2e;
 };
 bool mla_decode_supported(const MlaArgs &a);

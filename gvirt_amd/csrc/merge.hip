@@ -87,37 +87,43 @@ merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
     }
 }
 
-// The same merge for partials whose O is stored normalised (O_s / l_s) in 16 bits, half the traffic:
-// out = sum_s (w_s l_s) Ohat_s / sum_s (w_s l_s). A wave owns one (row, head): lane s computes the weight of
-// slot s, then the slots' rows (eight columns per lane) are read four at a time so that several loads are in
-// flight per lane.
+// The merge of the MLA decode kernel's partials: O is stored normalised (O_s / l_s) in 16 bits,
+// out = sum_s (w_s l_s) Ohat_s / sum_s (w_s l_s). A row's segments sit in per-chunk slots: meta[row] =
+// (segments n, first chunk c0, first-in-chunk flag f); segment 0 is slot 2 c0 + (1 - f), segment s slot
+// 2 (c0 + s). A wave owns one (row, head): lane s computes the weight of segment s, then the segments' rows
+// (eight columns per lane) are read four at a time so that several loads are in flight per lane.
 template <typename T>
 __global__ void __launch_bounds__(256)
-merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_acc,
-                    const float *__restrict__ part_ml, const int32_t *__restrict__ part_cnt, uint32_t total_rh,
-                    uint32_t dv, uint32_t max_slots)
+merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_acc, const float *__restrict__ part_ml,
+                 const int4 *__restrict__ meta, uint32_t rows, uint32_t n_heads, uint32_t dv)
 {
     const uint32_t lane = threadIdx.x & 63;
     const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (rh >= total_rh) {
+    if (rh >= static_cast<uint64_t>(rows) * n_heads) {
         return;
     }
-    const uint32_t n = static_cast<uint32_t>(part_cnt[rh]);
+    const uint32_t row = static_cast<uint32_t>(rh / n_heads), head = static_cast<uint32_t>(rh % n_heads);
+    const int4 mt = meta[row];
+    const uint32_t n = static_cast<uint32_t>(mt.x);
     if (n == 0) {
         return;  // the producer wrote the final value itself
     }
-    const uint64_t base = rh * max_slots;
+    const uint32_t c0 = static_cast<uint32_t>(mt.y), first_flag = static_cast<uint32_t>(mt.z);
+    auto slot_of = [&](uint32_t s) -> uint64_t {
+        const uint32_t ps = s == 0 ? 2 * c0 + (1 - first_flag) : 2 * (c0 + s);
+        return static_cast<uint64_t>(ps) * n_heads + head;
+    };
     float mm = -INFINITY;
     for (uint32_t s = lane; s < n; s += 64) {
-        mm = fmaxf(mm, part_ml[(base + s) * 2]);
+        mm = fmaxf(mm, part_ml[slot_of(s) * 2]);
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
         mm = fmaxf(mm, __shfl_xor(mm, d));
     }
     const float ms = mm == -INFINITY ? 0.f : mm;
-    for (uint32_t c0 = 0; c0 < dv / 8; c0 += 64) {
-        const uint32_t c = c0 + lane;
+    for (uint32_t cc = 0; cc < dv / 8; cc += 64) {
+        const uint32_t c = cc + lane;
         const bool c_ok = c < dv / 8;   // idle lanes still take part in the exchanges
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         float wsum = 0.f;
@@ -125,7 +131,7 @@ merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ par
             const uint32_t cnt = min(64u, n - s0);
             float w_lane = 0.f;
             if (lane < cnt) {
-                const float2 ml = *reinterpret_cast<const float2 *>(part_ml + (base + s0 + lane) * 2);
+                const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
                 w_lane = fast_exp2(ml.x - ms) * ml.y;
             }
             for (uint32_t j = 0; j < cnt; j += 4) {
@@ -134,7 +140,7 @@ merge_norm16_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ par
 #pragma unroll
                 for (uint32_t u = 0; u < 4; u++) {
                     const uint32_t idx = min(j + u, cnt - 1);
-                    x[u] = c_ok ? *reinterpret_cast<const uint4 *>(part_acc + (base + s0 + idx) * dv + c * 8)
+                    x[u] = c_ok ? *reinterpret_cast<const uint4 *>(part_acc + slot_of(s0 + idx) * dv + c * 8)
                                 : make_uint4(0, 0, 0, 0);
                     w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
                 }
@@ -202,19 +208,19 @@ int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers 
     return XLITE_HIP_OK;
 }
 
-int launch_merge_norm16(hipStream_t stream, int dtype, void *out, const PartialBuffers &b, uint32_t rows,
-                        uint32_t n_heads, uint32_t dv, uint32_t max_slots)
+int launch_merge_mla(hipStream_t stream, int dtype, void *out, const uint16_t *acc, const float *ml, const int32_t *meta,
+                     uint32_t rows, uint32_t n_heads, uint32_t dv)
 {
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
-    const uint32_t total_rh = rows * n_heads;
-    const dim3 grid(ceil_div(total_rh, 4u), 1, 1);
-    const uint16_t *acc = reinterpret_cast<const uint16_t *>(b.acc);
+    const uint64_t total_rh = static_cast<uint64_t>(rows) * n_heads;
+    const dim3 grid(static_cast<uint32_t>((total_rh + 3) / 4), 1, 1);
+    const int4 *m4 = reinterpret_cast<const int4 *>(meta);
     if (dtype == XLITE_HIP_BF16) {
-        merge_norm16_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, total_rh, dv, max_slots);
+        merge_mla_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
     } else {
-        merge_norm16_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, b.ml, b.cnt, total_rh, dv, max_slots);
+        merge_mla_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

@@ -121,8 +121,10 @@ mla_decode_kernel(const MlaDecodeParams p)
     set_roles(lane);
 
     // ---- one (sequence, query row, range of steps) at a time
-    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t limit, uint32_t step_a, uint32_t step_b, uint32_t slot,
-                           uint32_t n_slots) {
+    // `n_slots`: segments the row is cut into; `pslot`: where this segment's partial goes when there are several;
+    // `meta`: what the merge needs to find the row's partials (written with the row's first segment).
+    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t limit, uint32_t step_a, uint32_t step_b, uint32_t n_slots,
+                           uint32_t pslot, int4 meta) {
         const int32_t *table = dense ? nullptr : p.block_tables + static_cast<uint64_t>(seq) * p.max_num_blocks;
         const uint32_t t0 = step_a * kStep;
         const uint32_t t1 = min(limit, step_b * kStep);
@@ -414,17 +416,16 @@ mla_decode_kernel(const MlaDecodeParams p)
             for (uint32_t hr = 0; hr < heads_here; hr++) {
                 const uint4 x = *reinterpret_cast<const uint4 *>(my_tr + hr * TR_ROWB + lane * 16);
                 uint16_t *dst = single ? p.out + (rh0 + hr) * C
-                                       : reinterpret_cast<uint16_t *>(p.part_acc) + ((rh0 + hr) * p.max_slots + slot) * C;
+                                       : reinterpret_cast<uint16_t *>(p.part_acc) +
+                                             (static_cast<uint64_t>(pslot) * p.n_heads + hw + hr) * C;
                 *reinterpret_cast<uint4 *>(dst + lane * 8) = x;
             }
-            if (h_ok && gi == 0) {
-                const uint64_t rh = rh0 + col;
-                if (!single) {
-                    *reinterpret_cast<float2 *>(p.part_ml + (rh * p.max_slots + slot) * 2) = make_float2(m_run, l_tot);
-                }
-                if (slot == 0 && p.part_cnt != nullptr) {
-                    p.part_cnt[rh] = single ? 0 : static_cast<int32_t>(n_slots);
-                }
+            if (h_ok && gi == 0 && !single) {
+                *reinterpret_cast<float2 *>(p.part_ml + (static_cast<uint64_t>(pslot) * p.n_heads + head) * 2) =
+                    make_float2(m_run, l_tot);
+            }
+            if (step_a == 0 && h0 == 0 && threadIdx.x == 0) {
+                reinterpret_cast<int4 *>(p.part_meta)[tok] = meta;
             }
         }
         __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
@@ -433,26 +434,62 @@ mla_decode_kernel(const MlaDecodeParams p)
     // ---- the work list. Every query row owns ceil(limit / 32) steps; the rows' steps, laid end to end, are
     // cut into chunks of equal length, one chunk per workgroup (more when a chunk would not fit the block
     // table staging), so that ragged batches keep every compute unit equally busy. A chunk that crosses a
-    // row boundary is processed as several segments. Slot s of a row is its s-th segment.
+    // row boundary is processed as several segments. Only a chunk's first and last segment can be parts of
+    // rows that continue in other chunks: chunk c owns the partial slots 2c (its first segment) and 2c + 1
+    // (its last, when that is another one), and a row cut into n segments starting in chunk c0 finds them at
+    // 2 c0 (+ 1 unless it is that chunk's first segment), 2 (c0 + 1), 2 (c0 + 2), ...
     __shared__ uint32_t scan_ws[kWaves];
-    __shared__ uint32_t scan_bad;
-    __shared__ uint32_t found[2];
-    const uint32_t B = p.batch;
-    auto row_steps = [&](uint32_t i) {
-        const uint32_t lim = dense ? min(static_cast<uint32_t>(p.cached_lens[i] + p.lens[i]), p.dense_len)
-                                   : static_cast<uint32_t>(p.cached_lens[i] + 1);
-        return ceil_div(lim, kStep);
+    __shared__ uint32_t found[4];
+    const uint32_t B = p.batch, T = p.total_rows;
+    // the sequence that owns query row t (query_start_loc is a prefix sum), or B
+    auto seq_of = [&](uint32_t t) {
+        uint32_t lo = 0, hi = B;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) / 2;
+            if (p.query_start_loc[mid] <= static_cast<int32_t>(t)) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        if (lo == 0) {
+            return B;
+        }
+        return static_cast<int32_t>(t) < p.query_start_loc[lo - 1] + p.lens[lo - 1] ? lo - 1 : B;
+    };
+    // first sequence at or after `seq` that contains row t (rows are in sequence order), or B
+    auto advance = [&](uint32_t seq, uint32_t t) {
+        while (seq < B && static_cast<int32_t>(t) >= p.query_start_loc[seq] + p.lens[seq]) {
+            seq++;
+        }
+        return seq < B && static_cast<int32_t>(t) >= p.query_start_loc[seq] ? seq : B;
+    };
+    auto row_limit = [&](uint32_t t, uint32_t seq) -> uint32_t {
+        if (seq >= B) {
+            return 0;   // a row outside every sequence
+        }
+        const uint32_t clen = static_cast<uint32_t>(p.cached_lens[seq]);
+        return dense ? min(clen + static_cast<uint32_t>(p.lens[seq]), p.dense_len)
+                     : clen + (t - static_cast<uint32_t>(p.query_start_loc[seq])) + 1;
     };
     for (uint32_t c = blockIdx.x;; c += gridDim.x) {
         // block-wide prefix sums of the rows' step counts (redone for every chunk: nothing of it stays in
         // registers while a segment runs)
-        const uint32_t per = ceil_div(B, kNT);
-        const uint32_t i_lo = min(B, threadIdx.x * per), i_hi = min(B, i_lo + per);
+        const uint32_t per = ceil_div(T, kNT);
+        const uint32_t i_lo = min(T, threadIdx.x * per), i_hi = min(T, i_lo + per);
         uint32_t local = 0;
-        bool bad = false;   // a sequence with zero or several query rows: not a plain decode batch
-        for (uint32_t i = i_lo; i < i_hi; i++) {
-            local += row_steps(i);
-            bad |= p.lens[i] != 1;
+        {
+            uint32_t seq = i_lo < i_hi ? seq_of(i_lo) : B;
+            for (uint32_t t = i_lo; t < i_hi; t++) {
+                if (t > i_lo) {
+                    seq = advance(seq < B ? seq : 0, t);
+                }
+                const uint32_t n = ceil_div(row_limit(t, seq), kStep);
+                local += n;
+                if (n == 0 && blockIdx.x == 0 && c == 0) {
+                    reinterpret_cast<int4 *>(p.part_meta)[t] = make_int4(0, 0, 0, 0);   // a row without keys: nothing to merge
+                }
+            }
         }
         uint32_t incl = local;
 #pragma unroll
@@ -460,15 +497,9 @@ mla_decode_kernel(const MlaDecodeParams p)
             const uint32_t up = __shfl_up(incl, d);
             incl += lane >= static_cast<uint32_t>(d) ? up : 0;
         }
-        if (threadIdx.x == 0) {
-            scan_bad = 0;
-        }
-        __syncthreads();
+        __syncthreads();   // the previous chunk's readers of scan_ws and found are done
         if (lane == 63) {
             scan_ws[wave] = incl;
-        }
-        if (bad) {
-            scan_bad = 1;
         }
         __syncthreads();
         uint32_t excl = incl - local, total = 0;
@@ -478,20 +509,6 @@ mla_decode_kernel(const MlaDecodeParams p)
             excl += w < wave ? ws : 0;
             total += ws;
         }
-        if (scan_bad != 0) {
-            // general batches (total_tokens == batch, but not one row per sequence): whole rows, no split
-            for (uint32_t seq = blockIdx.x; seq < B; seq += gridDim.x) {
-                const int32_t qlen = p.lens[seq], clen = p.cached_lens[seq], qstart = p.query_start_loc[seq];
-                for (int32_t r = 0; r < qlen; r++) {
-                    const uint32_t limit = dense ? min(static_cast<uint32_t>(clen + qlen), p.dense_len)
-                                                 : static_cast<uint32_t>(clen + r + 1);
-                    if (limit > 0) {
-                        run_segment(seq, static_cast<uint32_t>(qstart + r), limit, 0, ceil_div(limit, kStep), 0, 1);
-                    }
-                }
-            }
-            return;
-        }
         total = __builtin_amdgcn_readfirstlane(total);
         uint32_t chunk = max(ceil_div(total, gridDim.x), p.chunk_min_steps);
         chunk = min(chunk, (kTblCap - 2) * p.block_size / kStep);
@@ -500,40 +517,49 @@ mla_decode_kernel(const MlaDecodeParams p)
         }
         const uint32_t start = c * chunk;
         uint32_t remaining = min(total, start + chunk) - start;
-        // the thread whose rows contain flat step `start` finds the row and the row's first flat step
+        // the thread whose rows contain flat step `start` finds the row, its sequence and its first flat step
         if (excl <= start && start < excl + local) {
-            uint32_t i = i_lo, first = excl;
+            uint32_t t = i_lo, first = excl, seq = seq_of(i_lo);
             for (;;) {
-                const uint32_t n = row_steps(i);
+                const uint32_t n = ceil_div(row_limit(t, seq), kStep);
                 if (start < first + n) {
                     break;
                 }
                 first += n;
-                i++;
+                t++;
+                seq = advance(seq < B ? seq : 0, t);
             }
-            found[0] = i;
+            found[0] = t;
             found[1] = first;
+            found[2] = seq;
         }
         __syncthreads();
         uint32_t row = __builtin_amdgcn_readfirstlane(found[0]);
         uint32_t first = __builtin_amdgcn_readfirstlane(found[1]);
+        uint32_t seq = __builtin_amdgcn_readfirstlane(found[2]);
         uint32_t a = start - first;
-        while (remaining > 0) {
-            const uint32_t clen = static_cast<uint32_t>(p.cached_lens[row]);
-            const uint32_t limit = dense ? min(clen + 1, p.dense_len) : clen + 1;
+        bool first_seg = true;
+        for (;;) {
+            const uint32_t limit = row_limit(row, seq);
             const uint32_t n = ceil_div(limit, kStep);
-            if (n == 0) {
-                row++;
-                continue;
+            if (n > 0) {
+                const uint32_t b = min(n, a + remaining);
+                const uint32_t c0 = first / chunk;
+                const uint32_t n_slots = (first + n - 1) / chunk - c0 + 1;
+                // written with the row's first segment (a == 0): then c0 == c
+                const int4 meta = make_int4(n_slots > 1 ? static_cast<int>(n_slots) : 0, static_cast<int>(c),
+                                            first_seg ? 1 : 0, 0);
+                run_segment(seq, row, limit, a, b, n_slots, 2 * c + (first_seg ? 0 : 1), meta);
+                remaining -= b - a;
+                first_seg = false;
             }
-            const uint32_t b = min(n, a + remaining);
-            const uint32_t slot0 = first / chunk;
-            run_segment(row, static_cast<uint32_t>(p.query_start_loc[row]), limit, a, b, (first + a) / chunk - slot0,
-                        (first + n - 1) / chunk - slot0 + 1);
-            remaining -= b - a;
+            if (remaining == 0) {
+                break;
+            }
             first += n;
             row++;
             a = 0;
+            seq = advance(seq < B ? seq : 0, row);
         }
         if (c + gridDim.x >= ceil_div(total, chunk)) {
             return;   // the usual case: one chunk per workgroup, no second scan
@@ -546,43 +572,71 @@ mla_decode_kernel(const MlaDecodeParams p)
 bool mla_decode_supported(const MlaArgs &a)
 {
     const bool dense = a.block_tables == nullptr;
-    return a.total_tokens == a.batch && a.kv_lora_rank == C && a.rope_head_dim == R && a.top_k == 0 &&
-           (dense || a.block_size % kStep == 0);
+    return a.kv_lora_rank == C && a.rope_head_dim == R && a.top_k == 0 && (dense || a.block_size % kStep == 0);
 }
 
-// Smallest chunk (in steps) a workgroup takes, and the number of partial slots a row can then need. The
-// chunk the kernel really uses is the batch's total step count over the number of workgroups, which the
-// host cannot know (the lengths live in device memory); it is never smaller than this.
-static void mla_decode_plan(const MlaArgs &a, uint32_t *chunk_min_steps, uint32_t *max_slots)
+namespace {
+
+struct MlaPlan {
+    uint32_t chunk_min_steps;   // smallest chunk a workgroup takes
+    uint32_t n_workgroups;      // one per compute unit (the LDS ring allows no more)
+    uint32_t max_chunks;        // bound on the number of chunks, hence of partial slots (two per chunk)
+    size_t meta_bytes, ml_bytes, acc_bytes;
+};
+
+// The chunk the kernel really uses is the batch's total step count over the number of workgroups, which the
+// host cannot know (the lengths live in device memory); it is never smaller than chunk_min_steps nor larger
+// than what the block-table staging holds.
+int mla_decode_plan(const MlaArgs &a, MlaPlan *pl)
 {
     const bool dense = a.block_tables == nullptr;
     const uint64_t max_ctx = dense ? a.dense_len : static_cast<uint64_t>(a.max_num_blocks) * a.block_size;
-    // half of what one workgroup per compute unit would get if every sequence were as long as allowed,
-    // between 256 and 512 positions
-    uint64_t tok = max_ctx * a.batch / 256 / 2;
+    int dev = 0;
+    XL_HIP(hipGetDevice(&dev));
+    thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
+    if (cu_dev != dev) {
+        XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+        cu_dev = dev;
+    }
+    // half of what one workgroup per compute unit would get if every row were as long as allowed, between 256
+    // and 512 positions
+    uint64_t tok = max_ctx * a.total_tokens / static_cast<uint64_t>(n_cu) / 2;
     tok = tok > 512 ? 512 : (tok < 256 ? 256 : tok);
-    *chunk_min_steps = static_cast<uint32_t>(tok / kStep);
+    pl->chunk_min_steps = static_cast<uint32_t>(tok / kStep);
+    pl->n_workgroups = static_cast<uint32_t>(n_cu);
     const uint64_t max_steps = (max_ctx + kStep - 1) / kStep;
-    *max_slots = static_cast<uint32_t>((max_steps + *chunk_min_steps - 1) / *chunk_min_steps + 1);
+    const uint64_t chunk_cap = static_cast<uint64_t>(kTblCap - 2) * (dense ? kStep : a.block_size) / kStep;
+    const uint64_t by_cap = (static_cast<uint64_t>(a.total_tokens) * max_steps + chunk_cap - 1) / chunk_cap;
+    pl->max_chunks = static_cast<uint32_t>(by_cap > pl->n_workgroups ? by_cap : pl->n_workgroups);
+    pl->meta_bytes = ((static_cast<size_t>(a.total_tokens) * sizeof(int4) + 255) / 256) * 256;
+    pl->ml_bytes = static_cast<size_t>(2) * pl->max_chunks * a.n_heads * 2 * sizeof(float);
+    pl->acc_bytes = static_cast<size_t>(2) * pl->max_chunks * a.n_heads * C * sizeof(uint16_t);
+    return XLITE_HIP_OK;
 }
+
+}  // namespace
 
 size_t mla_decode_workspace_bytes(const MlaArgs &a)
 {
-    uint32_t chunk_min, max_slots;
-    mla_decode_plan(a, &chunk_min, &max_slots);
-    return partial_bytes(a.total_tokens, a.n_heads, C, max_slots);
+    MlaPlan pl{};
+    if (mla_decode_plan(a, &pl) != XLITE_HIP_OK) {
+        return 0;
+    }
+    return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
 }
 
 int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
 {
-    uint32_t chunk_min, max_slots;
-    mla_decode_plan(a, &chunk_min, &max_slots);
-    const size_t need = mla_decode_workspace_bytes(a);
+    MlaPlan pl{};
+    if (const int rc = mla_decode_plan(a, &pl)) {
+        return rc;
+    }
+    const size_t need = pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
     if (a.workspace == nullptr || a.workspace_bytes < need) {
         return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
                                                     " bytes, have " + std::to_string(a.workspace_bytes));
     }
-    const PartialBuffers pb = carve_partials(a.workspace, a.total_tokens, a.n_heads, C, max_slots);
+    char *ws = static_cast<char *>(a.workspace);
     MlaDecodeParams p{};
     p.q_absorb = static_cast<const uint16_t *>(a.q_absorb);
     p.qr = static_cast<const uint16_t *>(a.qr);
@@ -593,35 +647,28 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
     p.lens = a.lens;
     p.cached_lens = a.cached_lens;
     p.block_tables = a.block_tables;
-    p.part_cnt = pb.cnt;
-    p.part_acc = pb.acc;
-    p.part_ml = pb.ml;
+    p.part_meta = reinterpret_cast<int32_t *>(ws);
+    p.part_ml = reinterpret_cast<float *>(ws + pl.meta_bytes);
+    p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
     p.n_heads = a.n_heads;
     p.batch = a.batch;
+    p.total_rows = a.total_tokens;
     p.block_size = a.block_tables == nullptr ? kStep : a.block_size;
     p.max_num_blocks = a.max_num_blocks;
     p.dense_len = a.dense_len;
-    p.chunk_min_steps = chunk_min;
-    p.max_slots = max_slots;
+    p.chunk_min_steps = pl.chunk_min_steps;
     p.scale_log2e = a.scale * kLog2e;
 
-    // one workgroup per compute unit (the LDS ring allows no more)
     const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + kTblCap * sizeof(uint32_t);
-    int dev = 0;
-    XL_HIP(hipGetDevice(&dev));
-    thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
-    if (cu_dev != dev) {
-        XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-        cu_dev = dev;
-    }
     // the kernel also has a few words of static LDS: ask for exactly the dynamic part
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(mla_decode_kernel), lds)) {
         return rc;
     }
-    mla_decode_kernel<<<dim3(static_cast<uint32_t>(n_cu), 1, 1), kNT, lds, stream>>>(p);
+    mla_decode_kernel<<<dim3(pl.n_workgroups, 1, 1), kNT, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
-    // rows that ended up in a single segment were stored directly (their count is 0)
-    return launch_merge_norm16(stream, a.dtype, a.o_absorb, pb, a.total_tokens, a.n_heads, C, max_slots);
+    // rows that ended up in a single segment were stored directly
+    return launch_merge_mla(stream, a.dtype, a.o_absorb, reinterpret_cast<const uint16_t *>(p.part_acc), p.part_ml,
+                            p.part_meta, a.total_tokens, a.n_heads, C);
 }
 
 }  // namespace xlite
