@@ -25,7 +25,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
-MEASURED_TRAFFIC_BYTES = {"c2": 1080392150, "c4": 322660348}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080394039, "c4": 325249588}
 
 
 def _events(torch):
@@ -298,7 +298,7 @@ def bench_mla(args, torch, rt):
             "config": {"workload": "c4 deepseek-r1 MLA absorbed decode", "batch": 32, "n_heads": 128, "ctx_total": int(sum(ctx)),
                        "kv_bytes_per_step": int(w["kv_bytes"]), "flops_per_step": int(w["flops"])},
             "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1),
-            "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_norm16_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
+            "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_mla_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c4"),
                          "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
             "cpu_baseline": cpu}

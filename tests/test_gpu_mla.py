@@ -235,3 +235,11 @@ def test_dsa_decode_pipeline_indexer_to_masked_mla(rt):
         n = clens[i] + 1
         row = got_lists[i, :min(top_k, n)].tolist()
         assert len(set(want[i][0]) - set(row)) * 100.0 <= 3.0 * len(row)
+
+
+def test_mla_prefill_128_heads_rows_of_several_sequences(rt):
+    """Chunked prefill at the full head count: hundreds of query rows, each with its own causal limit, cut
+    into chunks that cross row and sequence boundaries; a sequence without query rows in between."""
+    c = mla_case(61, [300, 0, 77, 1], [700, 50, 0, 2000], 128, bs=64)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
