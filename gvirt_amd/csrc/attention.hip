@@ -35,7 +35,9 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
     }
     const uint32_t splits =
         mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx, 64);
-    return mfma_workspace_bytes(total_tokens, n_heads, head_dim, splits + 1);
+    // whichever prefill kernel serves the shape
+    return std::max(mfma_workspace_bytes(total_tokens, n_heads, head_dim, splits + 1),
+                    prefill_mfma_workspace_bytes(total_tokens, n_heads, n_kv_heads, head_dim, batch, max_ctx));
 }
 
 extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache,
@@ -93,13 +95,7 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
     XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME, "the int8 KV cache is supported for decode batches only");
     XL_REQUIRE(mfma_gqa_supported(head_dim), "head_dim must be 64 or 128");
     if (prefill_mfma_supported(a)) {
-        // the streaming kernel walks each M tile's whole KV range; only few M tiles over a long
-        // context (where splitting the KV range is what fills the chip) go to the split kernel
-        const uint32_t max_ctx = max_num_block * block_size;
-        const uint32_t splits = mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx, 64);
-        if (splits == 1 || max_ctx < 4096) {
-            return launch_prefill_mfma(s, a);
-        }
+        return launch_prefill_mfma(s, a);
     }
     return launch_mfma_gqa(s, a);
 }

@@ -108,6 +108,8 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a);
 // prefill_mfma.hip
 bool prefill_mfma_supported(const AttentionArgs &a);
 int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a);
+size_t prefill_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                    uint32_t batch, uint32_t max_ctx);
 
 // mla_topk.hip
 size_t mla_topk_scratch_bytes(uint32_t total_tokens, uint32_t kv_lora_rank, uint32_t rope_head_dim, uint32_t top_k);

@@ -12,7 +12,10 @@
 // 16-byte chunks of a row are XOR-swizzled by the position (the lane chooses which global chunk lands
 // in its LDS slot) so that both read shapes are bank-conflict free.
 // M tiles are numbered sequence by sequence and launched last-first: the tiles with the longest
-// visible range start first.
+// visible range start first. When there are fewer M tiles than compute units (a short chunk after a
+// long cached context, decode rows mixed into the batch), grid.y splits every tile's visible range into
+// equal runs of KV tiles; the runs leave fp32 partials (O, reference maximum, normaliser) that the merge
+// kernel combines.
 //
 // Replaces attention.h / flash_attention.h for batches with multi-token queries
 // (xlite/csrc/kernels/attention.h:308-492, causal rule softmax_attn_aiv.h:739-741).
@@ -38,6 +41,7 @@ constexpr int KS = D / 16;                // k-steps of the QK product
 constexpr int NT = BN / 32;               // 32-position sub tiles
 constexpr int DT = D / 32;                // 32-row tiles of O^T
 constexpr int PER_WAVE = 2 * BN / 4 / kWaves;   // copies per wave and tile (4)
+constexpr uint32_t kMinSplitTiles = 8;          // a KV split walks at least 512 positions
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 
@@ -78,6 +82,11 @@ struct PrefillParams {
     uint32_t block_shift;
     uint32_t max_num_block;
     uint32_t n_mtiles;         // grid.x
+    uint32_t max_splits;       // grid.y: KV splits per M tile (1: none, results are final)
+    uint32_t n_heads;
+    int32_t *part_cnt;         // [token][head] number of partials to merge (0: the value is final)
+    float *part_acc;           // [token][head][max_splits][D]
+    float *part_ml;            // [token][head][max_splits][2]: reference maximum (log2 domain), normaliser
 };
 
 // XOR pattern of the 16-byte chunk index of LDS row `row` (rows are 256 bytes = one bank window). The
@@ -154,11 +163,26 @@ prefill_kernel(const PrefillParams p)
     const uint32_t m_last = min(m_rows, m_first + kMTile) - 1;
     // keys visible to at least one row of the tile
     const uint32_t range_end = static_cast<uint32_t>(clen) + m_last / G + 1;
-    const uint32_t n_tiles = ceil_div(range_end, static_cast<uint32_t>(BN));
+    // ---- this workgroup's run of KV tiles [first_tile, n_tiles): the whole range, or one of n_splits equal
+    // runs of at least kMinSplitTiles tiles
+    uint32_t n_tiles = ceil_div(range_end, static_cast<uint32_t>(BN));
+    uint32_t first_tile = 0, n_splits = 1;
+    const uint32_t split = blockIdx.y;
+    if (p.max_splits > 1) {
+        const uint32_t want = min(p.max_splits, max(1u, n_tiles / kMinSplitTiles));
+        const uint32_t per = ceil_div(n_tiles, want);
+        n_splits = ceil_div(n_tiles, per);
+        if (split >= n_splits) {
+            return;
+        }
+        first_tile = split * per;
+        n_tiles = min(n_tiles, first_tile + per);
+    }
     const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const uint32_t row_bytes = p.n_kv_heads * ROWB;
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE);
-    for (uint32_t i = threadIdx.x; i <= (range_end - 1) >> p.block_shift; i += kThreads) {
+    for (uint32_t i = ((first_tile * BN) >> p.block_shift) + threadIdx.x;
+         i <= (min(n_tiles * BN, range_end) - 1) >> p.block_shift; i += kThreads) {
         tbl_lds[i] = static_cast<uint32_t>(table[i]);
     }
     __syncthreads();
@@ -361,12 +385,12 @@ prefill_kernel(const PrefillParams p)
     // fetches the next tile's first K operands. Every copy is unconditional (tiles past the end copy the last
     // tile again into a stage nobody reads any more), so the wait counts are exact.
     const uint32_t last = n_tiles - 1;
-    issue(0);
-    issue(min(1u, last));
-    issue(min(2u, last));
+    issue(first_tile);
+    issue(min(first_tile + 1, last));
+    issue(min(first_tile + 2, last));
     dma_wait<2 * PER_WAVE>();
     __syncthreads();
-    fetch_k(0, 0);
+    fetch_k((first_tile % kStages) * STAGE, 0);
     using MaskOn = std::integral_constant<bool, true>;
     using MaskOff = std::integral_constant<bool, false>;
     auto tile_iter = [&](uint32_t tile, auto mask_tag) {
@@ -383,29 +407,60 @@ prefill_kernel(const PrefillParams p)
     // branch in one: each loop body exists once, so the accumulators keep their registers. Every wave runs
     // n_tiles iterations in total (one barrier each), wherever its own boundary between the loops lies.
     const uint32_t first_masked = min(n_tiles, wave_min_vis / BN);
-    uint32_t tile = 0;
-    for (; tile < first_masked; tile++) {
-        tile_iter(tile, MaskOff{});
-    }
-    for (; tile < n_tiles; tile++) {
-        tile_iter(tile, MaskOn{});
+    uint32_t tile = first_tile;
+    if (m_first + wave * 32 < m_rows) {
+        for (; tile < first_masked; tile++) {
+            tile_iter(tile, MaskOff{});
+        }
+        for (; tile < n_tiles; tile++) {
+            tile_iter(tile, MaskOn{});
+        }
+    } else {
+        // none of the wave's 32 rows exists (the last M tile of a sequence; a decode row in a mixed batch
+        // fills 4 of 256): the wave only keeps copying its share and meeting the others at the barrier
+        for (; tile < n_tiles; tile++) {
+            dma_wait<PER_WAVE>();
+            __syncthreads();
+            issue(min(tile + 3, last));
+        }
     }
     dma_wait<0>();
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     if (m_valid) {
         // O^T lane layout: column = M row, register k of tile dt = element 32 dt + 8 (k / 4) + 4 half + k % 4
-        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        uint16_t *dst = p.out + static_cast<uint64_t>(tok) * p.out_tok_stride + static_cast<uint64_t>(head) * D;
+        const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head;
+        if (n_splits == 1) {
+            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            uint16_t *dst = p.out + static_cast<uint64_t>(tok) * p.out_tok_stride + static_cast<uint64_t>(head) * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
+            for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
-            for (int kg = 0; kg < 4; kg++) {
-                uint2 o;
-                o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
-                o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
-                *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
+                for (int kg = 0; kg < 4; kg++) {
+                    uint2 o;
+                    o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
+                    o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
+                    *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
+                }
             }
+        } else {
+            // this run's partial: a row that sees none of the run's positions leaves (-inf, 0, zeros)
+            const uint64_t slot = rh * p.max_splits + split;
+            float *dst = p.part_acc + slot * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                for (int kg = 0; kg < 4; kg++) {
+                    *reinterpret_cast<float4 *>(dst + dt * 32 + kg * 8 + half * 4) =
+                        make_float4(O[dt][kg * 4], O[dt][kg * 4 + 1], O[dt][kg * 4 + 2], O[dt][kg * 4 + 3]);
+                }
+            }
+            if (half == 0) {
+                *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run * kLog2e, l_tot);
+            }
+        }
+        if (half == 0 && split == 0 && p.part_cnt != nullptr) {
+            p.part_cnt[rh] = n_splits == 1 ? 0 : static_cast<int32_t>(n_splits);
         }
     }
 }
@@ -416,6 +471,38 @@ bool prefill_mfma_supported(const AttentionArgs &a)
 {
     return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size >= 4 &&
            (a.block_size & (a.block_size - 1)) == 0 && a.n_heads % a.n_kv_heads == 0;
+}
+
+// KV splits per M tile: with fewer workgroups than compute units, the split count that minimises
+// (rounds of workgroups over the chip) / splits, each split keeping at least kMinSplitTiles tiles of the
+// longest possible context.
+uint32_t prefill_mfma_pick_splits(uint32_t total_tokens, uint32_t group, uint32_t batch, uint32_t n_kv_heads,
+                                  uint32_t max_ctx)
+{
+    const uint64_t base = (static_cast<uint64_t>(ceil_div(total_tokens * group, static_cast<uint32_t>(kMTile))) + batch) *
+                          n_kv_heads;
+    const uint64_t n_cu = 256;
+    const uint32_t cap = min(64u, max_ctx / (kMinSplitTiles * BN));
+    if (base >= n_cu || cap <= 1) {
+        return 1;
+    }
+    uint32_t best = 1;
+    double best_cost = 1.0;   // base < n_cu: one round
+    for (uint32_t s = 2; s <= cap; s++) {
+        const double cost = static_cast<double>((base * s + n_cu - 1) / n_cu) / s;
+        if (cost < best_cost * 0.95) {
+            best = s;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+size_t prefill_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                    uint32_t batch, uint32_t max_ctx)
+{
+    const uint32_t splits = prefill_mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx);
+    return splits <= 1 ? 0 : partial_bytes(total_tokens, n_heads, head_dim, splits);
 }
 
 int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
@@ -440,6 +527,17 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.max_num_block = a.max_num_block;
     // upper bound on the number of M tiles: every sequence may end with a ragged one
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
+    p.n_heads = a.n_heads;
+    uint32_t splits = prefill_mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, a.max_num_block * a.block_size);
+    if (a.workspace == nullptr || a.workspace_bytes < partial_bytes(a.total_tokens, a.n_heads, a.head_dim, splits)) {
+        splits = 1;   // no scratch: every M tile walks its whole KV range
+    }
+    p.max_splits = splits;
+    const PartialBuffers pb = splits > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, splits)
+                                         : PartialBuffers{};
+    p.part_cnt = pb.cnt;
+    p.part_acc = pb.acc;
+    p.part_ml = pb.ml;
 
     const size_t lds = static_cast<size_t>(kStages) * STAGE + (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     const bool bf = a.dtype == XLITE_HIP_BF16;
@@ -456,14 +554,17 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     } else {
         n_wg = a.n_kv_heads * p.n_mtiles;
     }
-    dim3 grid(n_wg, 1, 1);
+    dim3 grid(n_wg, splits, 1);
     if (bf) {
         prefill_kernel<BF16><<<grid, kThreads, lds, stream>>>(p);
     } else {
         prefill_kernel<FP16><<<grid, kThreads, lds, stream>>>(p);
     }
     XL_LAUNCH_CHECK();
-    return XLITE_HIP_OK;
+    if (splits == 1) {
+        return XLITE_HIP_OK;
+    }
+    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, splits);
 }
 
 }  // namespace xlite

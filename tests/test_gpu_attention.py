@@ -165,6 +165,22 @@ def test_prefill_model_grid(rt, model, work):
     check(run_attention(rt, w), oracle_attention(w))
 
 
+SPLIT_WORK = [([3000], [100]), ([16384], [128]), ([2047, 1500, 0, 4000], [1, 1, 300, 1]), ([8191] * 4 + [0], [1] * 4 + [256]),
+              ([5000, 900], [257, 2])]
+
+
+@pytest.mark.parametrize("model", [(8, 2, 128, 128, torch.bfloat16), (32, 8, 128, 128, torch.bfloat16),
+                                   (16, 4, 128, 16, torch.float16), (28, 4, 128, 64, torch.bfloat16)])
+@pytest.mark.parametrize("work", SPLIT_WORK)
+def test_prefill_few_tiles_over_long_context(rt, model, work):
+    """Short chunks after a long cached context and decode rows mixed with a prefill: fewer M tiles than
+    compute units, so each tile's KV range is split over several workgroups and merged."""
+    nH, nKV, d, bs, dtype = model
+    clens, lens = work
+    w = generic_case(23, lens, clens, nH, nKV, d, bs, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 def test_prefill_rows_equal_decode_steps(rt):
     """Row r of a prefill chunk must match the same row issued alone as a decode step."""
     w = generic_case(22, [40], [200], 8, 2, 128, 128, torch.bfloat16)
