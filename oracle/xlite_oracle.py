@@ -21,6 +21,8 @@ piece of the reference (paths under /root/reference/):
   gather_sparse_kv_cache_ref  xlite/tests/kernels/gather_sparse_kv_cache.py:102-116
   mha_forward_ref      xlite/csrc/model.cpp:480-600 (composition of the pieces; the projections are fp32
                        matrix products rounded once)
+  mla_forward_ref      xlite/csrc/model.cpp:333-482 (composition of the MLA pieces; golden of the whole layer:
+                       xlite/tests/models/deepseek_v3.py:629-692)
   indexer_scores_ref   xlite/tests/kernels/indexer_scores.py:96-118 (golden) with the 16-bit rounding of
                        the per-head products of xlite/csrc/kernels/indexer_scores.h:214-217
   indexer_topk_ref     xlite/tests/kernels/indexer_topk.py:139-152
@@ -48,6 +50,9 @@ tests/test_oracle_pins.py):
       preservation, complex-multiply identity in fp64.
   mla_prepare_ref, qk_rms_norm_ref: composition of pinned pieces + RMSNorm closed forms (a vector of
       equal entries c normalises to sign(c) * w + b; scale invariance; per-vector Python loop).
+  mha_forward_ref, mla_forward_ref: compositions of pinned pieces; mla_forward_ref additionally against the
+      textbook model form (per-head keys and values from the whole token history, rope as a complex product,
+      no paging, no absorption) over a prefill and two decode steps.
   gather_*: brute-force Python loops.
   indexer_scores_ref: pure-Python triple loop in float (tiny case); one head with weight 1 reduces to
       q . k; with no intermediate rounding the weighted sum equals (sum_h w_h q_h) . k (linearity).
@@ -329,6 +334,34 @@ def mha_forward_ref(hidden, wqkv, wo, k_cache, v_cache, lens, cached_lens, block
                          torch.from_numpy(meta["block_tables"]).flatten(), n_heads, n_kv_heads, head_dim, block_size, batch,
                          meta["max_num_blocks"])
     return (attn.to(dt).float().reshape(hidden.shape[0], -1) @ wo.float()).to(dt)
+
+
+def mla_forward_ref(hidden, wqkv_a, q_norm, kv_norm, wq_b, wuk_t, wuv, wo, k_cache, pe_cache, lens, cached_lens,
+                    block_tables, freqs, n_heads, q_lora_rank, kv_lora_rank, nope_head_dim, rope_head_dim, v_head_dim,
+                    block_size, scale, norm_eps=1e-6):
+    """xlite/csrc/model.cpp:333-482 as a composition of the pieces above: metadata (prepare_attn_ref), QKV_A
+    projection, mla_prepare (in place on the caches), Q_B projection, rope_complex, mla_v2 (absorb einsum,
+    absorbed attention, W_UV einsum), output projection; every stage leaves its result in the activation
+    dtype, as the reference's tensors between operators do. `block_tables[i]` lists the blocks of sequence i."""
+    dt = hidden.dtype
+    T = hidden.shape[0]
+    meta = prepare_attn_ref(lens, cached_lens, block_tables, block_size)
+    pos = torch.tensor(meta["position"], dtype=torch.int64)
+    slots = torch.tensor(meta["slot_mapping"], dtype=torch.int32)
+    qkvc = (hidden.float() @ wqkv_a.float()).to(dt)
+    norm_qc = torch.empty(T, q_lora_rank, dtype=dt)
+    norm_kvc = torch.empty(T, kv_lora_rank, dtype=dt)
+    mla_prepare_ref(qkvc, q_norm, torch.zeros_like(q_norm), norm_qc, kv_norm, torch.zeros_like(kv_norm), norm_kvc, freqs,
+                    pos, q_lora_rank, kv_lora_rank, rope_head_dim, block_size, k_cache, pe_cache, slots, norm_eps)
+    q_with_qr = (norm_qc.float() @ wq_b.float()).to(dt)
+    q_pe = rope_complex_ref(n_heads, nope_head_dim + rope_head_dim, rope_head_dim, q_with_qr, freqs, pos)
+    batch = len(lens)
+    attn = mla_v2_ref(q_with_qr, q_pe.reshape(T, -1), k_cache, pe_cache, wuk_t, wuv,
+                      torch.tensor(meta["query_start_loc"], dtype=torch.int32), torch.tensor(list(lens), dtype=torch.int32),
+                      torch.tensor(list(cached_lens), dtype=torch.int32), torch.from_numpy(meta["block_tables"]).flatten(),
+                      n_heads, rope_head_dim, nope_head_dim, v_head_dim, kv_lora_rank, block_size, batch,
+                      meta["max_num_blocks"], scale)
+    return (attn.to(dt).float().reshape(T, -1) @ wo.float()).to(dt)
 
 
 # --------------------------------------------------------------------------

@@ -390,3 +390,55 @@ def test_qk_rms_norm_pins():
     full = O.qk_rms_norm_ref(x, torch.ones(nH * d).bfloat16(), None, torch.ones(nKV * d).bfloat16(), None, 1e-6,
                              nH * d, 1, nKV * d, 1, nH * d)
     torch.testing.assert_close(full[:, :nH * d].float().pow(2).mean(-1), torch.ones(5), rtol=2e-2, atol=0)
+
+
+def test_mla_forward_equals_the_naive_model_form():
+    """The layer composition (projection, norms, rope, absorbed attention over the paged cache, output
+    projection) must equal the textbook model form of xlite/tests/models/deepseek_v3.py:656-674: per-head keys
+    k = [W_UK kv | k_pe], values v = W_UV^T kv, rope as a complex product, recomputed here from the whole
+    token history in float32 with no paging, no absorption and no cache."""
+    g = torch.Generator().manual_seed(31)
+    H, ql, kvl, nope, rope, vd, hid, bs = 3, 12, 8, 6, 4, 5, 10, 4
+    scale = (nope + rope) ** -0.5
+    r = lambda *s: torch.randn(*s, generator=g)
+    wa, wqb, wuk_t, wuv, wo = r(hid, ql + kvl + rope) * 0.3, r(ql, H * (nope + rope)) * 0.3, r(H, nope, kvl), r(H, kvl, vd), r(H * vd, hid)
+    qn, kn = 1 + 0.1 * r(ql), 1 + 0.1 * r(kvl)
+    ang = torch.outer(torch.arange(64).float(), 1.0 / (100.0 ** (torch.arange(0, rope, 2).float() / rope)))
+    freqs = torch.polar(torch.ones_like(ang), ang)                     # complex64 [max_pos, rope / 2]
+    prompts = [7, 2, 9]
+    tables = [[5, 1, 9], [0, 7, 3], [2, 8, 4]]
+    kc, pc = torch.zeros(10, bs, kvl), torch.zeros(10, bs, rope)
+    history = [torch.zeros(0, hid) for _ in prompts]
+    cached = [0] * len(prompts)
+
+    def rms(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+
+    def crope(x, pos):                                                  # interleaved pairs -> complex product
+        xc = torch.view_as_complex(x.reshape(*x.shape[:-1], -1, 2).contiguous()) * freqs[pos].reshape(len(pos), *([1] * (x.dim() - 2)), -1)
+        return torch.view_as_real(xc).flatten(-2)
+
+    for step in range(3):
+        lens = prompts if step == 0 else [1] * len(prompts)
+        hidden = r(sum(lens), hid)
+        got = O.mla_forward_ref(hidden, wa, qn, kn, wqb, wuk_t, wuv, wo, kc, pc, lens, cached, tables, freqs, H, ql, kvl,
+                                nope, rope, vd, bs, scale)
+        off = 0
+        for i, n in enumerate(lens):
+            history[i] = torch.cat([history[i], hidden[off:off + n]])
+            x = history[i]
+            L = x.shape[0]
+            pos = torch.arange(L)
+            a = x @ wa
+            q = (rms(a[:, :ql], qn) @ wqb).view(L, H, nope + rope)
+            q_pe = crope(q[..., nope:], pos)
+            kv = rms(a[:, ql:ql + kvl], kn)
+            k_pe = crope(a[:, ql + kvl:], pos)
+            k_nope = torch.einsum("tc,hdc->thd", kv, wuk_t)
+            v = torch.einsum("tc,hcv->thv", kv, wuv)
+            s = (torch.einsum("shd,thd->hst", q[..., :nope], k_nope) + torch.einsum("shr,tr->hst", q_pe, k_pe)) * scale
+            s = s + torch.full((L, L), float("-inf")).triu(1)
+            o = torch.einsum("hst,thv->shv", torch.softmax(s, -1), v).reshape(L, -1) @ wo
+            assert torch.allclose(got[off:off + n], o[L - n:], atol=2e-4, rtol=2e-4), "step %d sequence %d" % (step, i)
+            off += n
+        cached = [c + l for c, l in zip(cached, lens)]
