@@ -31,7 +31,8 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
         const uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);
-        return decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile));
+        return std::max(decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile)),
+                        prefill_mfma_workspace_bytes(total_tokens, n_heads, n_kv_heads, head_dim, batch, max_ctx));
     }
     const uint32_t splits =
         mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx, 64);
@@ -74,7 +75,12 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
             return launch_decode_mfma(s, a);
         }
-        // block sizes that are not a multiple of 32, or more than 16 query heads per kv head
+        // more than 16 query heads per kv head, or a small block size: the prefill kernel takes the rows of a
+        // sequence as one (ragged) M tile and splits the KV range
+        if (kv_dtype == XLITE_HIP_KV_SAME && prefill_mfma_supported(a)) {
+            return launch_prefill_mfma(s, a);
+        }
+        // block sizes that are not a multiple of 16 nor a power of two, int8 caches of such shapes
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
         uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);

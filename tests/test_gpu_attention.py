@@ -103,6 +103,18 @@ def test_decode_special_cases(rt):
         check(run_attention(rt, w), oracle_attention(w))
 
 
+@pytest.mark.parametrize("model", [(64, 2, 128, 128, torch.bfloat16), (64, 1, 128, 64, torch.float16), (40, 2, 128, 16, torch.bfloat16),
+                                   (32, 8, 128, 8, torch.bfloat16), (8, 2, 128, 4, torch.bfloat16)])
+@pytest.mark.parametrize("work", DECODE_WORK)
+def test_decode_wide_groups_and_small_blocks(rt, model, work):
+    """More than 16 query heads per kv head, and power-of-two block sizes below 16: decode batches the
+    streaming prefill kernel serves (a sequence's rows are one ragged M tile, the KV range is split)."""
+    nH, nKV, d, bs, dtype = model
+    clens, lens = work
+    w = generic_case(15, lens, clens, nH, nKV, d, bs, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 def test_decode_int8_kv(rt):
     ctx = [129, 4100, 640, 17, 2048, 9000]
     w = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=True)
