@@ -123,6 +123,29 @@ class Runtime:
         torch.cuda.current_stream(self.device).synchronize()
 
 
+class ModelAttnMeta:
+    """Host lists describing one step, as in xlite._C.ModelAttnMeta (xlite/csrc/_C.cpp:1988-1993): the metadata
+    builder derives positions, slots and the dense block table from them."""
+
+    def __init__(self):
+        self.lens: List[int] = []
+        self.cached_lens: List[int] = []
+        self.is_prefills: List[bool] = []          # deprecated in the reference; ignored
+        self.block_tables: List[List[int]] = []
+
+
+class AttnMeta:
+    """The vLLM-compatible form, as in xlite._C.AttnMeta (xlite/csrc/_C.cpp:1995-2001): host block tables, and
+    the positions taken from the caller's tensor instead of being derived (xlite/csrc/_C.cpp:666-677)."""
+
+    def __init__(self):
+        self.lens: List[int] = []
+        self.cached_lens: List[int] = []
+        self.is_prefills: List[bool] = []
+        self.block_tables_cpu: List[List[int]] = []
+        self.positions: Optional[torch.Tensor] = None
+
+
 def rope_and_cache(rt: Runtime, inout: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    position: torch.Tensor, cosin: torch.Tensor, slot_mapping: torch.Tensor, n_heads: int,
                    n_kv_heads: int, head_dim: int, rot_dim: int, block_size: int, is_neox: bool,

@@ -16,7 +16,7 @@ from . import _C, _lib
 
 
 @dataclass
-class AttnMeta:
+class StepMeta:
     """What `PrepareAttn` leaves on the device for one step (xlite/csrc/runtime.h:37-51)."""
     batch: int
     batched_tokens: int
@@ -31,9 +31,11 @@ class AttnMeta:
 
 
 def prepare_attn(lens: Sequence[int], cached_lens: Sequence[int], block_tables: Sequence[Sequence[int]],
-                 block_size: int, device) -> AttnMeta:
+                 block_size: int, device, positions: Optional[torch.Tensor] = None) -> StepMeta:
     """Host metadata of one step through the library's `xlite_hip_prepare_attn`, then one upload per array.
-    `block_tables[i]` lists the physical blocks of sequence i (at least ceil((len + cached) / block_size))."""
+    `block_tables[i]` lists the physical blocks of sequence i (at least ceil((len + cached) / block_size)).
+    `positions` (int64, one per token) replaces the derived positions, as the reference's version-1 metadata
+    does (xlite/csrc/runtime.cpp:535-548)."""
     lib = _lib.load()
     batch = len(lens)
     if batch == 0:
@@ -53,10 +55,26 @@ def prepare_attn(lens: Sequence[int], cached_lens: Sequence[int], block_tables: 
         block_size, ctypes.c_void_p(qsl.data_ptr()), ctypes.c_void_p(pos.data_ptr()), ctypes.c_void_p(slots.data_ptr()),
         ctypes.c_void_p(dense.data_ptr()), cap, ctypes.byref(mnb), ctypes.byref(bt), ctypes.byref(dec)))
     up = lambda t: t.to(device, non_blocking=False)
-    return AttnMeta(batch=batch, batched_tokens=int(bt.value), max_num_blocks=int(mnb.value), is_decode=bool(dec.value),
+    if positions is not None:
+        if positions.dtype != torch.int64 or positions.numel() < T:
+            raise RuntimeError("prepare_attn: positions must hold one int64 per token")
+        pos = positions.reshape(-1)[:T]
+    return StepMeta(batch=batch, batched_tokens=int(bt.value), max_num_blocks=int(mnb.value), is_decode=bool(dec.value),
                     query_start_loc=up(qsl), lens=up(torch.tensor([int(x) for x in lens], dtype=torch.int32)),
                     cached_lens=up(torch.tensor([int(x) for x in cached_lens], dtype=torch.int32)),
                     block_tables=up(dense[: batch * int(mnb.value)].contiguous()), position=up(pos), slot_mapping=up(slots))
+
+
+def prepare_attn_meta(meta, block_size: int, device) -> StepMeta:
+    """`prepare_attn` from one of the reference's metadata objects: `_C.ModelAttnMeta` (positions derived) or
+    `_C.AttnMeta` (vLLM form: `block_tables_cpu` and the caller's `positions` tensor)."""
+    if isinstance(meta, _C.ModelAttnMeta):
+        return prepare_attn(meta.lens, meta.cached_lens, meta.block_tables, block_size, device)
+    if isinstance(meta, _C.AttnMeta):
+        if meta.positions is None:
+            raise RuntimeError("prepare_attn: AttnMeta.positions is not set")
+        return prepare_attn(meta.lens, meta.cached_lens, meta.block_tables_cpu, block_size, device, positions=meta.positions)
+    raise RuntimeError("prepare_attn: invalid attnMeta version: " + type(meta).__name__)
 
 
 @dataclass
@@ -81,7 +99,7 @@ class MhaLayer:
         if cfg.qk_norm and (q_norm is None or k_norm is None):
             raise RuntimeError("MhaLayer: qk_norm needs q_norm and k_norm")
 
-    def forward(self, rt: _C.Runtime, hidden: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, meta: AttnMeta,
+    def forward(self, rt: _C.Runtime, hidden: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, meta: StepMeta,
                 cosin: torch.Tensor) -> torch.Tensor:
         c = self.cfg
         qkv = torch.matmul(hidden, self.wqkv)

@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 from . import _C
-from .mha import AttnMeta
+from .mha import StepMeta
 
 
 @dataclass
@@ -49,7 +49,7 @@ class MlaLayer:
             raise RuntimeError("MlaLayer: wuv must be [n_heads, kv_lora_rank, v_head_dim]")
 
     def forward(self, rt: _C.Runtime, hidden: torch.Tensor, k_cache: torch.Tensor, pe_cache: torch.Tensor,
-                meta: AttnMeta, freqs: torch.Tensor, topk_indices: Optional[torch.Tensor] = None,
+                meta: StepMeta, freqs: torch.Tensor, topk_indices: Optional[torch.Tensor] = None,
                 top_k: int = 0) -> torch.Tensor:
         c = self.cfg
         T = hidden.shape[0]

@@ -109,3 +109,30 @@ def test_operators_refuse_cpu_tensors_and_bad_arguments():
         _C.einsum_mht_htd_mhd(FakeRt(), x, x, x, 1, 1, 16, 32, True)
     with pytest.raises(RuntimeError, match="single GPU"):
         _C.Runtime(0, 0, tp_size=2)
+
+
+def test_prepare_attn_accepts_the_reference_metadata_objects():
+    """`ModelAttnMeta` (positions derived) and the vLLM form `AttnMeta` (host block tables, caller's positions:
+    xlite/csrc/_C.cpp:666-677, xlite/csrc/runtime.cpp:535-548) through the host-side builder, on CPU tensors."""
+    import torch
+    from gvirt_amd import _C
+    from gvirt_amd.mha import prepare_attn_meta
+    lens, clens, rows, bs = [3, 1, 5], [5, 9, 0], [[7, 2], [4, 9, 1], [3, 8]], 4
+    want = O.prepare_attn_ref(lens, clens, rows, bs)
+    m0 = _C.ModelAttnMeta()
+    m0.lens, m0.cached_lens, m0.block_tables = lens, clens, rows
+    a = prepare_attn_meta(m0, bs, "cpu")
+    assert a.batch == 3 and a.batched_tokens == 9 and not a.is_decode and a.max_num_blocks == want["max_num_blocks"]
+    assert a.position.tolist() == list(want["position"]) and a.slot_mapping.tolist() == list(want["slot_mapping"])
+    assert a.query_start_loc.tolist() == list(want["query_start_loc"])
+    assert a.block_tables.tolist() == want["block_tables"].flatten().tolist()
+    m1 = _C.AttnMeta()
+    m1.lens, m1.cached_lens, m1.block_tables_cpu = lens, clens, rows
+    m1.positions = torch.arange(100, 109, dtype=torch.int64)
+    b = prepare_attn_meta(m1, bs, "cpu")
+    assert b.position.tolist() == list(range(100, 109)) and b.slot_mapping.tolist() == a.slot_mapping.tolist()
+    m1.positions = None
+    with pytest.raises(RuntimeError):
+        prepare_attn_meta(m1, bs, "cpu")
+    with pytest.raises(RuntimeError):
+        prepare_attn_meta(object(), bs, "cpu")
