@@ -75,12 +75,12 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
             return launch_decode_mfma(s, a);
         }
-        // more than 16 query heads per kv head, or a small block size: the prefill kernel takes the rows of a
-        // sequence as one (ragged) M tile and splits the KV range
+        // more than 16 query heads per kv head, or a block size that is not a multiple of 16: the prefill
+        // kernel takes the rows of a sequence as one (ragged) M tile and splits the KV range
         if (kv_dtype == XLITE_HIP_KV_SAME && prefill_mfma_supported(a)) {
             return launch_prefill_mfma(s, a);
         }
-        // block sizes that are not a multiple of 16 nor a power of two, int8 caches of such shapes
+        // head_dim 64 or block sizes that are not a multiple of 4 at such shapes, int8 caches with wide groups
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);
         uint32_t tile = decode_pick_tile(batch, n_kv_heads, block_size, max_num_block, zdim);

@@ -78,8 +78,8 @@ struct PrefillParams {
     uint32_t group;            // query heads per kv head
     uint32_t n_kv_heads;
     uint32_t batch;
-    uint32_t block_size;       // a power of two
-    uint32_t block_shift;
+    uint32_t block_size;       // a multiple of 4
+    uint32_t block_magic;      // floor(2^32 / block_size) + 1: position / block_size == mulhi(position, magic)
     uint32_t max_num_block;
     uint32_t n_mtiles;         // grid.x
     uint32_t max_splits;       // grid.y: KV splits per M tile (1: none, results are final)
@@ -181,8 +181,8 @@ prefill_kernel(const PrefillParams p)
     const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const uint32_t row_bytes = p.n_kv_heads * ROWB;
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE);
-    for (uint32_t i = ((first_tile * BN) >> p.block_shift) + threadIdx.x;
-         i <= (min(n_tiles * BN, range_end) - 1) >> p.block_shift; i += kThreads) {
+    for (uint32_t i = __umulhi(first_tile * BN, p.block_magic) + threadIdx.x;
+         i <= __umulhi(min(n_tiles * BN, range_end) - 1, p.block_magic); i += kThreads) {
         tbl_lds[i] = static_cast<uint32_t>(table[i]);
     }
     __syncthreads();
@@ -263,9 +263,9 @@ prefill_kernel(const PrefillParams p)
             }
             // block-table entries come from LDS (copied there once): a vector load here would have to be
             // awaited together with every copy issued before it
-            const uint32_t blk = t >> p.block_shift, off = t & (p.block_size - 1);
+            const uint32_t blk = __umulhi(t, p.block_magic), off = t - blk * p.block_size;
             const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk]);
-            const uint64_t row0 = (static_cast<uint64_t>(phys) << p.block_shift) + off;
+            const uint64_t row0 = static_cast<uint64_t>(phys) * p.block_size + off;
             const char *kb = reinterpret_cast<const char *>(p.k_cache) + row0 * row_bytes + kvh * ROWB;
             const char *vb = reinterpret_cast<const char *>(p.v_cache) + row0 * row_bytes + kvh * ROWB;
             dma_1k(st + pos * ROWB, voff, kb);
@@ -469,8 +469,10 @@ prefill_kernel(const PrefillParams p)
 
 bool prefill_mfma_supported(const AttentionArgs &a)
 {
-    return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size >= 4 &&
-           (a.block_size & (a.block_size - 1)) == 0 && a.n_heads % a.n_kv_heads == 0;
+    // the division by the block size is a multiply-high, exact while position * block_size < 2^32
+    return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size >= 4 && a.block_size % 4 == 0 &&
+           static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32) &&
+           a.n_heads % a.n_kv_heads == 0;
 }
 
 // KV splits per M tile: with fewer workgroups than compute units, the split count that minimises
@@ -523,7 +525,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.n_kv_heads = a.n_kv_heads;
     p.batch = a.batch;
     p.block_size = a.block_size;
-    p.block_shift = static_cast<uint32_t>(__builtin_ctz(a.block_size));
+    p.block_magic = static_cast<uint32_t>((1ull << 32) / a.block_size) + 1;
     p.max_num_block = a.max_num_block;
     // upper bound on the number of M tiles: every sequence may end with a ragged one
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
