@@ -59,6 +59,9 @@ int launch_merge(hipStream_t stream, int dtype, void *out, const PartialBuffers 
 // 2 (c0 + s) after that (meta = segments, c0, first flag per row); acc holds O / l in the 16-bit activation type.
 int launch_merge_mla(hipStream_t stream, int dtype, void *out, const uint16_t *acc, const float *ml, const int32_t *meta,
                      uint32_t rows, uint32_t n_heads, uint32_t dv);
+// The same slot scheme with fp32 partials (O, maximum in the log2 domain, normaliser), [slot][head][dv].
+int launch_merge_meta(hipStream_t stream, int dtype, void *out, const float *acc, const float *ml, const int32_t *meta,
+                      uint32_t rows, uint32_t n_heads, uint32_t dv);
 
 // decode_attention.hip
 bool decode_supported(uint32_t head_dim);
@@ -77,6 +80,12 @@ void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, 
                       uint32_t *tile_tokens, uint32_t *n_sub, uint32_t *max_slots);
 size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim, uint32_t max_slots);
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
+struct DecodeDmaPlan {
+    uint32_t max_chunks;   // bound on the number of chunks, hence of partial slots (two per chunk)
+    size_t meta_bytes, ml_bytes, acc_bytes;
+};
+bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, uint32_t batch, int kv_dtype);
+size_t decode_dma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t block_size, uint32_t max_num_block);
 
 // mla_decode.hip
 struct MlaDecodeParams {

@@ -84,6 +84,9 @@ struct DecodeMfmaParams {
     uint32_t tile_tokens;  // multiple of kStep * n_sub
     uint32_t n_sub;        // sub-ranges of a tile handled by different waves (kv heads < 8)
     uint32_t max_slots;    // max tiles * n_sub
+    // decode_dma_kernel only: its partials sit in per-chunk slots, [slot][head][D] and [slot][head][2]
+    int32_t *part_meta;    // [token] int4: segments to merge (0: final), first chunk, first-segment flag
+    uint32_t batch;
 };
 
 // 8 cache elements (uint4 = 16-bit, uint2 = int8) -> 8 x 16-bit in a uint4
@@ -523,6 +526,19 @@ __device__ __forceinline__ void dma_wait()
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
+// Work split of decode_dma_kernel: every sequence owns ceil(limit / 16) steps, limit its visible range; the
+// sequences' steps laid end to end are cut into equal chunks, one per workgroup (the lengths live in device
+// memory, so every workgroup computes the prefix sums itself), so that ragged batches keep every compute unit
+// equally busy. A chunk that crosses a sequence boundary runs as several segments. Only a chunk's first and
+// last segment can be parts of sequences that continue in other chunks: chunk c owns the partial slots 2c
+// (its first segment) and 2c + 1 (its last, when that is another one); a sequence cut into n segments that
+// starts in chunk c0 finds them at 2 c0 (+ 1 unless it is that chunk's first segment), 2 (c0 + 1), ...
+// and its meta entry (n, c0, first flag) tells the merge kernel so. Sequences inside one chunk are final.
+constexpr uint32_t kDmaTblCap = 1024;    // block-table entries staged per segment
+constexpr uint32_t kDmaSeqCap = 4096;    // sequences whose prefix sums fit in LDS (with 2^28 steps in all)
+constexpr uint32_t kDmaMinChunk = 16;    // steps: no chunk below 256 positions
+constexpr uint32_t kDmaMaxWorkgroups = 512;   // grid bound the partial slots are sized for (one workgroup per compute unit)
+
 template <typename T>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_dma_kernel(const DecodeMfmaParams p)
@@ -537,13 +553,13 @@ decode_dma_kernel(const DecodeMfmaParams p)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE);
+    uint32_t *wave_tot = tbl_lds + kDmaTblCap;   // kWaves entries
+    uint32_t *pref = wave_tot + kWaves;          // batch + 1 exclusive prefix sums of the step counts
     const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
         static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t tile = blockIdx.x;
-    const uint32_t seq = blockIdx.y;
     const uint32_t col = lane & 15;
     const uint32_t jq = lane >> 4;
 
@@ -570,29 +586,133 @@ decode_dma_kernel(const DecodeMfmaParams p)
         c_voff[i] = (lane >> 4) * HEADB + (((lane & 15u) ^ swizzle<D>(2 * wave + i)) << 4);
     }
 
-    const int32_t qlen = p.lens[seq];
-    const int32_t clen = p.cached_lens[seq];
-    const int32_t qstart = p.query_start_loc[seq];
-    const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t row_bytes = p.n_kv_heads * HEADB;
+    const uint32_t B = p.batch;
 
-    for (int32_t r = 0; r < qlen; r++) {
-        const uint32_t tok = static_cast<uint32_t>(qstart + r);
-        const uint32_t limit = static_cast<uint32_t>(clen + r + 1);
-        const uint32_t n_tiles = ceil_div(limit, p.tile_tokens);
-        if (tile >= n_tiles) {
-            continue;
+    // what is the same in every lane, said so: the copies take scalar addresses
+    auto uni = [](uint32_t x) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(x))); };
+    // ---- exclusive prefix sums of the sequences' step counts. Up to 64 sequences: every wave keeps them in
+    // its lanes (lane = sequence), nothing goes through LDS. More: thread t owns `ipt` consecutive sequences
+    // and the sums land in LDS, each entry packed with its sequence's (limit - 1) % 16.
+    const bool in_lanes = B <= 64;
+    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_tok = 0, total;
+    auto steps_of = [&](uint32_t i, uint32_t *limit) {
+        const int32_t ql = p.lens[i];
+        *limit = ql > 0 ? static_cast<uint32_t>(p.cached_lens[i] + 1) : 0u;   // the visible range of the sequence's row
+        if (ql <= 0 && blockIdx.x == 0) {
+            reinterpret_cast<int4 *>(p.part_meta)[p.query_start_loc[i]] = make_int4(0, 0, 0, 0);   // nothing to merge
         }
-        const uint32_t t0 = tile * p.tile_tokens;
-        const uint32_t t1 = min(limit, t0 + p.tile_tokens);
-        const bool single = n_tiles == 1;
+        return ceil_div(*limit, static_cast<uint32_t>(kStep));
+    };
+    if (in_lanes) {
+        if (lane < B) {
+            ln_tok = static_cast<uint32_t>(p.query_start_loc[lane]);
+            ln_steps = steps_of(lane, &ln_limit);
+        }
+        uint32_t incl = ln_steps;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d);
+            incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
+        }
+        ln_pref = incl - ln_steps;
+        total = uni(__shfl(incl, 63));
+    } else {
+        const uint32_t ipt = ceil_div(B, static_cast<uint32_t>(kWaves * 64));
+        const uint32_t i0 = min(B, threadIdx.x * ipt), i1 = min(B, i0 + ipt);
+        uint32_t mine = 0, limit;
+        for (uint32_t i = i0; i < i1; i++) {
+            mine += steps_of(i, &limit);
+        }
+        uint32_t incl = mine;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d);
+            incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
+        }
+        if (lane == 63) {
+            wave_tot[wave] = incl;
+        }
+        __syncthreads();
+        uint32_t before = 0;
+        for (uint32_t w = 0; w < wave; w++) {
+            before += wave_tot[w];
+        }
+        uint32_t run = before + incl - mine;
+        for (uint32_t i = i0; i < i1; i++) {
+            const uint32_t n = steps_of(i, &limit);
+            pref[i] = (run << 4) | ((limit - 1) & 15u);
+            run += n;
+        }
+        if (threadIdx.x == kWaves * 64 - 1) {
+            pref[B] = (before + incl) << 4;
+        }
+        __syncthreads();
+        total = uni(pref[B]) >> 4;
+    }
+    if (total == 0) {
+        return;
+    }
+    // first step, step count and visible range of sequence i
+    auto seq_info = [&](uint32_t i, uint32_t *first, uint32_t *n, uint32_t *limit) {
+        if (in_lanes) {
+            *first = uni(__shfl(ln_pref, static_cast<int>(i)));
+            *n = uni(__shfl(ln_steps, static_cast<int>(i)));
+            *limit = uni(__shfl(ln_limit, static_cast<int>(i)));
+        } else {
+            const uint32_t a = uni(pref[i]), b = uni(pref[i + 1]);
+            *first = a >> 4;
+            *n = (b >> 4) - *first;
+            *limit = *n == 0 ? 0u : (*n - 1) * kStep + (a & 15u) + 1;
+        }
+    };
+    // the sequence that holds step `start`: the last one whose prefix is <= start
+    auto seq_of = [&](uint32_t start) -> uint32_t {
+        if (in_lanes) {
+            const uint64_t mask = __ballot(lane < B && ln_pref <= start);
+            return static_cast<uint32_t>(__builtin_popcountll(mask)) - 1;
+        }
+        uint32_t lo = 0, hi = B;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if ((uni(pref[mid]) >> 4) <= start) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        return lo;
+    };
+    uint32_t chunk = max(ceil_div(total, gridDim.x), kDmaMinChunk);
+    chunk = min(chunk, (kDmaTblCap - 2) * p.block_size / kStep);
+    const uint32_t n_chunks = ceil_div(total, chunk);
+
+    // one segment: positions [t0, t1) of sequence `seq`
+    auto run_segment = [&](uint32_t seq_, uint32_t t0_, uint32_t t1_, bool whole, uint32_t pslot_, bool first_piece, int4 meta) {
+        const uint32_t seq = uni(seq_), t0 = uni(t0_), t1 = uni(t1_), pslot = uni(pslot_);
+        const uint32_t tok = in_lanes ? uni(__shfl(ln_tok, static_cast<int>(seq))) : static_cast<uint32_t>(p.query_start_loc[seq]);
+        const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
         const uint32_t n_steps = ceil_div(t1 - t0, kStep);
         const uint32_t blk0 = t0 / p.block_size;
+        // the query rows of the first pass travel together with the block-table entries
+        uint4 qreg[KS];
+        auto load_q = [&](uint32_t kv0) {
+            const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
+                                   static_cast<uint64_t>((kv0 + wave) * p.group + col) * D;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8) : make_uint4(0, 0, 0, 0);
+            }
+        };
+        load_q(0);
         {
             const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
             for (uint32_t i = threadIdx.x; i < nblk; i += kWaves * 64) {
                 tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
+            }
+            if (first_piece && threadIdx.x == 0) {
+                reinterpret_cast<int4 *>(p.part_meta)[tok] = meta;
             }
             __syncthreads();
         }
@@ -601,18 +721,13 @@ decode_dma_kernel(const DecodeMfmaParams p)
             const uint32_t kvh = kv0 + wave;
             const uint32_t head0 = kvh * p.group;
 
-            uint4 qreg[KS];
-            {
-                const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride + static_cast<uint64_t>(head0 + col) * D;
+            if (kv0 > 0) {
+                load_q(kv0);
+            }
+            // complete these loads before any copy is issued: memory operations finish in order
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8) : make_uint4(0, 0, 0, 0);
-                }
-                // complete these loads before any copy is issued: memory operations finish in order
-#pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
-                }
+            for (int ks = 0; ks < KS; ks++) {
+                asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
             }
             f32x4_t O[MT];
 #pragma unroll
@@ -714,7 +829,7 @@ decode_dma_kernel(const DecodeMfmaParams p)
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
             if (col < g_valid) {
-                if (single) {
+                if (whole) {
                     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
                     uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
 #pragma unroll
@@ -725,7 +840,7 @@ decode_dma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<uint2 *>(dst + mt * 16 + jq * 4) = o;
                     }
                 } else {
-                    const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * p.max_slots + tile;
+                    const uint64_t slot = static_cast<uint64_t>(pslot) * p.n_heads + head0 + col;
                     float *dst = p.part_acc + slot * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
@@ -735,23 +850,42 @@ decode_dma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
                     }
                 }
-                if (jq == 0 && tile == 0 && p.part_cnt != nullptr) {
-                    p.part_cnt[static_cast<uint64_t>(tok) * p.n_heads + head0 + col] = single ? 0 : static_cast<int32_t>(n_tiles);
-                }
             }
+        }
+    };
+
+    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const uint32_t start = c * chunk, end = min(total, start + chunk);
+        uint32_t seq = seq_of(start), pos = start;
+        while (pos < end) {
+            uint32_t first, n, limit;
+            seq_info(seq, &first, &n, &limit);
+            if (n == 0) {
+                seq++;
+                continue;
+            }
+            const uint32_t a = pos - first, b = min(n, a + (end - pos));
+            const bool whole = a == 0 && b == n;
+            const bool first_seg = pos == start;
+            const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
+            const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
+            run_segment(seq, a * kStep, min(limit, b * kStep), whole, 2 * c + (first_seg ? 0u : 1u), a == 0, meta);
+            pos += b - a;
+            seq++;
         }
     }
 }
 
 template <typename T>
-int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
+int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
-    const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) + (p.tile_tokens / kStep + 2) * sizeof(uint32_t);
+    const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
+                       (kDmaTblCap + kWaves + p.batch + 1) * sizeof(uint32_t);
     auto kernel = decode_dma_kernel<T>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
     }
-    dim3 grid(p.max_slots, batch, 1);
+    dim3 grid(n_workgroups, 1, 1);
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
@@ -813,8 +947,79 @@ size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint
     return max_slots > 1 ? partial_bytes(total_tokens, n_heads, head_dim, max_slots) : 0;
 }
 
+// decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8, a batch whose prefix sums fit in LDS
+bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, uint32_t batch, int kv_dtype)
+{
+    return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0 && batch <= kDmaSeqCap;
+}
+
+// The chunk the kernel really uses is the batch's total step count over the number of workgroups, which the
+// host cannot know (the lengths live in device memory); it is never below kDmaMinChunk steps nor above what
+// the block-table staging holds, which bounds the number of chunks and hence of partial slots (two per chunk).
+void decode_dma_plan(uint32_t batch, uint32_t n_heads, uint32_t block_size, uint32_t max_num_block, DecodeDmaPlan *pl)
+{
+    const uint64_t max_steps = ceil_div(max_num_block * block_size, static_cast<uint32_t>(kStep));
+    const uint64_t chunk_cap = static_cast<uint64_t>(kDmaTblCap - 2) * block_size / kStep;
+    const uint64_t by_cap = (static_cast<uint64_t>(batch) * max_steps + chunk_cap - 1) / chunk_cap;
+    pl->max_chunks = static_cast<uint32_t>(by_cap > kDmaMaxWorkgroups ? by_cap : kDmaMaxWorkgroups);
+    pl->meta_bytes = ((static_cast<size_t>(batch) * sizeof(int4) + 255) / 256) * 256;
+    pl->ml_bytes = static_cast<size_t>(2) * pl->max_chunks * n_heads * 2 * sizeof(float);
+    pl->acc_bytes = static_cast<size_t>(2) * pl->max_chunks * n_heads * 128 * sizeof(float);
+}
+
+size_t decode_dma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t block_size, uint32_t max_num_block)
+{
+    DecodeDmaPlan pl{};
+    decode_dma_plan(batch, n_heads, block_size, max_num_block, &pl);
+    return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
+}
+
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
 {
+    if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.batch, a.kv_dtype)) {
+        DecodeDmaPlan pl{};
+        decode_dma_plan(a.batch, a.n_heads, a.block_size, a.max_num_block, &pl);
+        thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
+        int dev = 0;
+        XL_HIP(hipGetDevice(&dev));
+        if (dev != cu_dev) {
+            XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+            cu_dev = dev;
+        }
+        const uint32_t n_workgroups = min(static_cast<uint32_t>(n_cu), kDmaMaxWorkgroups);
+        const size_t need = pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
+        if (a.workspace == nullptr || a.workspace_bytes < need) {
+            return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
+                                                        " bytes, have " + std::to_string(a.workspace_bytes));
+        }
+        char *ws = static_cast<char *>(a.workspace);
+        DecodeMfmaParams p{};
+        p.q = static_cast<const uint16_t *>(a.qkv);
+        p.k_cache = a.k_cache;
+        p.v_cache = a.v_cache;
+        p.out = static_cast<uint16_t *>(a.output);
+        p.query_start_loc = a.query_start_loc;
+        p.lens = a.lens;
+        p.cached_lens = a.cached_lens;
+        p.block_tables = a.block_tables;
+        p.part_meta = reinterpret_cast<int32_t *>(ws);
+        p.part_ml = reinterpret_cast<float *>(ws + pl.meta_bytes);
+        p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
+        p.q_row_stride = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
+        p.n_heads = a.n_heads;
+        p.n_kv_heads = a.n_kv_heads;
+        p.group = a.n_heads / a.n_kv_heads;
+        p.block_size = a.block_size;
+        p.max_num_block = a.max_num_block;
+        p.batch = a.batch;
+        const int rc = a.dtype == XLITE_HIP_BF16 ? launch_dma<BF16>(stream, p, n_workgroups)
+                                                 : launch_dma<FP16>(stream, p, n_workgroups);
+        if (rc != XLITE_HIP_OK) {
+            return rc;
+        }
+        return launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens,
+                                 a.n_heads, a.head_dim);
+    }
     uint32_t tile, n_sub, max_slots;
     decode_mfma_plan(a.batch, a.n_kv_heads, a.block_size, a.max_num_block, &tile, &n_sub, &max_slots);
     const size_t need = decode_mfma_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, max_slots);
@@ -851,9 +1056,7 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
     const bool bf = a.dtype == XLITE_HIP_BF16;
     int rc;
-    if (a.head_dim == 128 && !kv8 && a.n_kv_heads % kWaves == 0) {
-        rc = bf ? launch_dma<BF16>(stream, p, a.batch) : launch_dma<FP16>(stream, p, a.batch);
-    } else if (a.head_dim == 128) {
+    if (a.head_dim == 128) {
         if (bf) {
             rc = kv8 ? launch_one<BF16, 128, true>(stream, p, a.batch) : launch_one<BF16, 128, false>(stream, p, a.batch);
         } else {

@@ -168,6 +168,85 @@ merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_a
     }
 }
 
+// The balanced GQA decode kernel's partials: fp32 (O, maximum in the log2 domain, normaliser) in the same
+// per-chunk slots as above, [slot][head][dv]. A wave owns one (row, head); four columns per lane.
+template <typename T>
+__global__ void __launch_bounds__(256)
+merge_meta_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc, const float *__restrict__ part_ml,
+                  const int4 *__restrict__ meta, uint32_t rows, uint32_t n_heads, uint32_t dv)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (rh >= static_cast<uint64_t>(rows) * n_heads) {
+        return;
+    }
+    const uint32_t row = static_cast<uint32_t>(rh / n_heads), head = static_cast<uint32_t>(rh % n_heads);
+    const int4 mt = meta[row];
+    const uint32_t n = static_cast<uint32_t>(mt.x);
+    if (n == 0) {
+        return;  // the producer wrote the final value itself
+    }
+    const uint32_t c0 = static_cast<uint32_t>(mt.y), first_flag = static_cast<uint32_t>(mt.z);
+    auto slot_of = [&](uint32_t s) -> uint64_t {
+        const uint32_t ps = s == 0 ? 2 * c0 + (1 - first_flag) : 2 * (c0 + s);
+        return static_cast<uint64_t>(ps) * n_heads + head;
+    };
+    float mm = -INFINITY;
+    for (uint32_t s = lane; s < n; s += 64) {
+        mm = fmaxf(mm, part_ml[slot_of(s) * 2]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        mm = fmaxf(mm, __shfl_xor(mm, d));
+    }
+    const float ms = mm == -INFINITY ? 0.f : mm;
+    for (uint32_t cc = 0; cc < dv / 4; cc += 64) {
+        const uint32_t c = cc + lane;
+        const bool c_ok = c < dv / 4;   // idle lanes still take part in the exchanges
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float lsum = 0.f;
+        for (uint32_t s0 = 0; s0 < n; s0 += 64) {
+            const uint32_t cnt = min(64u, n - s0);
+            float w_lane = 0.f, l_lane = 0.f;
+            if (lane < cnt) {
+                const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
+                w_lane = fast_exp2(ml.x - ms);
+                l_lane = ml.y * w_lane;
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                l_lane += __shfl_xor(l_lane, d);
+            }
+            lsum += l_lane;
+            for (uint32_t j = 0; j < cnt; j += 4) {
+                float4 x[4];
+                float w[4];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    const uint32_t idx = min(j + u, cnt - 1);
+                    x[u] = c_ok ? *reinterpret_cast<const float4 *>(part_acc + slot_of(s0 + idx) * dv + c * 4)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+                    w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    acc.x += x[u].x * w[u];
+                    acc.y += x[u].y * w[u];
+                    acc.z += x[u].z * w[u];
+                    acc.w += x[u].w * w[u];
+                }
+            }
+        }
+        if (c_ok) {
+            const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+            uint2 o;
+            o.x = T::pack(acc.x * inv, acc.y * inv);
+            o.y = T::pack(acc.z * inv, acc.w * inv);
+            *reinterpret_cast<uint2 *>(out + rh * dv + c * 4) = o;
+        }
+    }
+}
+
 }  // namespace
 
 size_t partial_bytes(uint32_t rows, uint32_t n_heads, uint32_t dv, uint32_t max_slots)
@@ -221,6 +300,24 @@ int launch_merge_mla(hipStream_t stream, int dtype, void *out, const uint16_t *a
         merge_mla_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
     } else {
         merge_mla_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
+int launch_merge_meta(hipStream_t stream, int dtype, void *out, const float *acc, const float *ml, const int32_t *meta,
+                      uint32_t rows, uint32_t n_heads, uint32_t dv)
+{
+    if (rows == 0) {
+        return XLITE_HIP_OK;
+    }
+    const uint64_t total_rh = static_cast<uint64_t>(rows) * n_heads;
+    const dim3 grid(static_cast<uint32_t>((total_rh + 3) / 4), 1, 1);
+    const int4 *m4 = reinterpret_cast<const int4 *>(meta);
+    if (dtype == XLITE_HIP_BF16) {
+        merge_meta_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
+    } else {
+        merge_meta_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

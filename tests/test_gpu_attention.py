@@ -116,6 +116,23 @@ def test_decode_wide_groups_and_small_blocks(rt, model, work):
     check(run_attention(rt, w), oracle_attention(w))
 
 
+@pytest.mark.parametrize("model,batch,lo,hi,long_ones", [((32, 8, 128, 128, torch.bfloat16), 100, 1, 3000, [9000, 5000]),
+                                                        ((32, 8, 128, 128, torch.bfloat16), 700, 1, 200, [2500]),
+                                                        ((16, 8, 128, 16, torch.float16), 70, 1, 900, []),
+                                                        ((64, 16, 128, 64, torch.bfloat16), 40, 100, 2000, [])])
+def test_decode_ragged_batches_balanced_split(rt, model, batch, lo, hi, long_ones):
+    """Ragged decode batches on the shapes of the streaming decode kernel: the sequences' steps are cut into
+    equal chunks across workgroups, so chunks hold whole short sequences, tails and heads of long ones; more
+    than 64 sequences take the prefix sums through LDS, more than 512 several sequences per thread."""
+    nH, nKV, d, bs, dtype = model
+    rng = np.random.default_rng(batch)
+    clens = [int(x) for x in rng.integers(lo, hi, size=batch)]
+    for i, v in enumerate(long_ones):
+        clens[(7 * i + 3) % batch] = v
+    w = generic_case(16, [1] * batch, clens, nH, nKV, d, bs, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 def test_decode_int8_kv(rt):
     ctx = [129, 4100, 640, 17, 2048, 9000]
     w = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=True)
