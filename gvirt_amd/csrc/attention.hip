@@ -24,12 +24,7 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
     const uint32_t max_ctx = max_num_block * block_size;
     if (is_decode_batch(total_tokens, batch)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
-            uint32_t tile, n_sub, max_slots;
-            decode_mfma_plan(batch, n_kv_heads, block_size, max_num_block, &tile, &n_sub, &max_slots);
-            // a 16-bit cache may go to the balanced kernel, an int8 cache of the same shape does not
-            const size_t dma = decode_dma_supported(n_kv_heads, head_dim, batch, XLITE_HIP_KV_SAME)
-                                   ? decode_dma_workspace_bytes(batch, n_heads, block_size, max_num_block) : 0;
-            return std::max(dma, decode_mfma_workspace_bytes(total_tokens, n_heads, head_dim, max_slots));
+            return decode_mfma_workspace_for(batch, total_tokens, n_heads, n_kv_heads, head_dim, block_size, max_num_block);
         }
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);

@@ -124,6 +124,171 @@ __device__ __forceinline__ uint32_t swizzle(uint32_t row)
     return ((rr & (CH / 2 - 1)) << 1) | ((rr / (CH / 2)) & 1);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Work split of the decode kernels: every sequence owns ceil(limit / 16) steps, limit its visible range;
+// the sequences' steps laid end to end are cut into equal chunks, one per workgroup (the lengths live in
+// device memory, so every workgroup computes the prefix sums itself), so that ragged batches keep every
+// compute unit equally busy. A chunk that crosses a sequence boundary runs as several segments. Only a
+// chunk's first and last segment can be parts of sequences that continue in other chunks: chunk c owns the
+// partial slots 2c (its first segment) and 2c + 1 (its last, when that is another one); a sequence cut into
+// n segments that starts in chunk c0 finds them at 2 c0 (+ 1 unless it is that chunk's first segment),
+// 2 (c0 + 1), ... and its meta entry (n, c0, first flag) tells the merge kernel so. Sequences inside one
+// chunk are final.
+// ---------------------------------------------------------------------------------------------------
+constexpr uint32_t kSplitTblCap = 1024;         // block-table entries staged per segment
+constexpr uint32_t kSplitSeqCap = 4096;         // sequences whose prefix sums fit in LDS (with 2^28 steps in all)
+constexpr uint32_t kSplitMinChunk = 16;         // steps: no chunk below 256 positions
+constexpr uint32_t kSplitMaxWorkgroups = 512;   // grid bound the partial slots are sized for (one workgroup per compute unit)
+constexpr uint32_t kSplitLdsWords = kSplitTblCap + kWaves;   // + batch + 1
+
+// what is the same in every lane, said so: scalar address arithmetic follows
+__device__ __forceinline__ uint32_t uni(uint32_t x)
+{
+    return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(x)));
+}
+
+struct DecodeSplit {
+    const DecodeMfmaParams &p;
+    uint32_t *wave_tot, *pref;   // LDS: kWaves words, batch + 1 words
+    uint32_t lane, wave, B;
+    bool in_lanes;
+    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_tok = 0, total = 0, chunk = 0, n_chunks = 0;
+
+    __device__ __forceinline__ DecodeSplit(const DecodeMfmaParams &params, uint32_t *lds, uint32_t lane_, uint32_t wave_)
+        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_), B(params.batch), in_lanes(params.batch <= 64)
+    {
+    }
+    __device__ __forceinline__ uint32_t steps_of(uint32_t i, uint32_t *limit) const
+    {
+        const int32_t ql = p.lens[i];
+        *limit = ql > 0 ? static_cast<uint32_t>(p.cached_lens[i] + 1) : 0u;   // the visible range of the sequence's row
+        if (ql <= 0 && blockIdx.x == 0) {
+            reinterpret_cast<int4 *>(p.part_meta)[p.query_start_loc[i]] = make_int4(0, 0, 0, 0);   // nothing to merge
+        }
+        return ceil_div(*limit, static_cast<uint32_t>(kStep));
+    }
+    // Exclusive prefix sums of the step counts. Up to 64 sequences: every wave keeps them in its lanes
+    // (lane = sequence), nothing goes through LDS. More: thread t owns `ipt` consecutive sequences and the
+    // sums land in LDS, each entry packed with its sequence's (limit - 1) % 16. Contains barriers in the
+    // second case: every thread of the workgroup calls it.
+    __device__ __forceinline__ void scan()
+    {
+        if (in_lanes) {
+            if (lane < B) {
+                ln_tok = static_cast<uint32_t>(p.query_start_loc[lane]);
+                ln_steps = steps_of(lane, &ln_limit);
+            }
+            uint32_t incl = ln_steps;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(incl, d);
+                incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
+            }
+            ln_pref = incl - ln_steps;
+            total = uni(__shfl(incl, 63));
+        } else {
+            const uint32_t ipt = ceil_div(B, static_cast<uint32_t>(kWaves * 64));
+            const uint32_t i0 = min(B, threadIdx.x * ipt), i1 = min(B, i0 + ipt);
+            uint32_t mine = 0, limit;
+            for (uint32_t i = i0; i < i1; i++) {
+                mine += steps_of(i, &limit);
+            }
+            uint32_t incl = mine;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(incl, d);
+                incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
+            }
+            if (lane == 63) {
+                wave_tot[wave] = incl;
+            }
+            __syncthreads();
+            uint32_t before = 0;
+            for (uint32_t w = 0; w < wave; w++) {
+                before += wave_tot[w];
+            }
+            uint32_t run = before + incl - mine;
+            for (uint32_t i = i0; i < i1; i++) {
+                const uint32_t n = steps_of(i, &limit);
+                pref[i] = (run << 4) | ((limit - 1) & 15u);
+                run += n;
+            }
+            if (threadIdx.x == kWaves * 64 - 1) {
+                pref[B] = (before + incl) << 4;
+            }
+            __syncthreads();
+            total = uni(pref[B]) >> 4;
+        }
+        if (total != 0) {
+            chunk = max(ceil_div(total, gridDim.x), kSplitMinChunk);
+            chunk = min(chunk, (kSplitTblCap - 2) * p.block_size / kStep);
+            n_chunks = ceil_div(total, chunk);
+        }
+    }
+    // first step, step count and visible range of sequence i
+    __device__ __forceinline__ void seq_info(uint32_t i, uint32_t *first, uint32_t *n, uint32_t *limit) const
+    {
+        if (in_lanes) {
+            *first = uni(__shfl(ln_pref, static_cast<int>(i)));
+            *n = uni(__shfl(ln_steps, static_cast<int>(i)));
+            *limit = uni(__shfl(ln_limit, static_cast<int>(i)));
+        } else {
+            const uint32_t a = uni(pref[i]), b = uni(pref[i + 1]);
+            *first = a >> 4;
+            *n = (b >> 4) - *first;
+            *limit = *n == 0 ? 0u : (*n - 1) * kStep + (a & 15u) + 1;
+        }
+    }
+    // the sequence that holds step `start`: the last one whose prefix is <= start
+    __device__ __forceinline__ uint32_t seq_of(uint32_t start) const
+    {
+        if (in_lanes) {
+            const uint64_t mask = __ballot(lane < B && ln_pref <= start);
+            return static_cast<uint32_t>(__builtin_popcountll(mask)) - 1;
+        }
+        uint32_t lo = 0, hi = B;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if ((uni(pref[mid]) >> 4) <= start) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        return lo;
+    }
+    __device__ __forceinline__ uint32_t tok_of(uint32_t seq) const
+    {
+        return in_lanes ? uni(__shfl(ln_tok, static_cast<int>(seq))) : static_cast<uint32_t>(p.query_start_loc[seq]);
+    }
+    // segment(seq, tok, t0, t1, whole, partial slot, first piece of its sequence, meta of the sequence)
+    template <typename F>
+    __device__ __forceinline__ void for_each_segment(F &&segment) const
+    {
+        for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+            const uint32_t start = c * chunk, end = min(total, start + chunk);
+            uint32_t seq = seq_of(start), pos = start;
+            while (pos < end) {
+                uint32_t first, n, limit;
+                seq_info(seq, &first, &n, &limit);
+                if (n == 0) {
+                    seq++;
+                    continue;
+                }
+                const uint32_t a = pos - first, b = min(n, a + (end - pos));
+                const bool whole = a == 0 && b == n;
+                const bool first_seg = pos == start;
+                const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
+                const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
+                segment(uni(seq), tok_of(seq), uni(a * kStep), uni(min(limit, b * kStep)), whole,
+                        uni(2 * c + (first_seg ? 0u : 1u)), a == 0, meta);
+                pos += b - a;
+                seq++;
+            }
+        }
+    }
+};
+
 template <typename T, int D, bool KV8, bool MULTI_SUB>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_mfma_kernel(const DecodeMfmaParams p)
@@ -143,8 +308,6 @@ decode_mfma_kernel(const DecodeMfmaParams p)
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t tile = blockIdx.x;
-    const uint32_t seq = blockIdx.y;
     // LDS: two stages; in a stage one region per (kv head, sub range) pair of the pass = per
     // computing wave, K tile then V tile. int8 caches: behind the stages, the scales of the two
     // stages [stage][K | V][region][16 positions]
@@ -154,6 +317,10 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     // loop must not be a vector memory load, whose completion can only be awaited together with
     // every cache load issued before it (that would drain the prefetch pipeline at every step)
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE_BYTES + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0));
+    // Two ways to hand out work. One sub range per tile (kv heads >= 8): the balanced split of DecodeSplit,
+    // partials in per-chunk slots. Several sub ranges (fewer kv heads, the waves of a kv head share a tile):
+    // one workgroup per (sequence, tile of p.tile_tokens positions), partials at [token][head][tile][sub].
+    constexpr bool BALANCED = !MULTI_SUB;
 
     // ---- compute roles -------------------------------------------------------------------------------
     const uint32_t col = lane & 15;       // MFMA column = query head inside the group
@@ -200,26 +367,17 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     const float *s_src = threadIdx.x < 128 ? p.k_scale : p.v_scale;
     const uint32_t s_dst = (threadIdx.x < 128 ? 0 : kWaves * kStep) + (s_sub * kvw + s_kvl) * kStep + s_pos;
 
-    const int32_t qlen = p.lens[seq];
-    const int32_t clen = p.cached_lens[seq];
-    const int32_t qstart = p.query_start_loc[seq];
-    const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const gvec_t *kc = static_cast<const gvec_t *>(p.k_cache);
     const gvec_t *vc = static_cast<const gvec_t *>(p.v_cache);
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
-    const uint32_t sub_len = p.tile_tokens / p.n_sub;
     const uint32_t my_kvl = wave & (kvw - 1), my_sub = wave >> kvw_shift;
 
-    for (int32_t r = 0; r < qlen; r++) {
-        const uint32_t tok = static_cast<uint32_t>(qstart + r);
-        const uint32_t limit = static_cast<uint32_t>(clen + r + 1);
-        const uint32_t n_tiles = ceil_div(limit, p.tile_tokens);
-        if (tile >= n_tiles) {
-            continue;
-        }
-        const uint32_t t0 = tile * p.tile_tokens;
-        const uint32_t t1 = min(limit, t0 + p.tile_tokens);
-        const bool single = n_tiles == 1 && p.n_sub == 1;
+    // one segment: positions [t0, t1) of the row `tok` of sequence `seq`. `single`: the result is final.
+    // Otherwise head h's partial goes to slot slot_base + h * slot_head_stride (+ the wave's sub range).
+    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool single, uint64_t slot_base,
+                           uint32_t slot_head_stride, int32_t cnt_value, bool write_meta, int4 meta) {
+        const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
+        const uint32_t sub_len = BALANCED ? t1 - t0 : p.tile_tokens / p.n_sub;
         // every sub range runs the same number of steps (the first one is never shorter than the others)
         const uint32_t n_steps = ceil_div(min(t1 - t0, sub_len), kStep);
         const uint32_t ta = min(t1, t0 + my_sub * sub_len);   // this wave's range
@@ -229,6 +387,9 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
             for (uint32_t i = threadIdx.x; i < nblk; i += NT) {
                 tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
+            }
+            if (BALANCED && write_meta && threadIdx.x == 0) {
+                reinterpret_cast<int4 *>(p.part_meta)[tok] = meta;
             }
             __syncthreads();
         }
@@ -485,7 +646,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<uint2 *>(dst + mt * 16 + jq * 4) = o;
                     }
                 } else {
-                    const uint64_t slot = (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * p.max_slots + tile * p.n_sub + my_sub;
+                    const uint64_t slot = slot_base + static_cast<uint64_t>(head0 + col) * slot_head_stride + my_sub;
                     float *dst = p.part_acc + slot * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
@@ -496,10 +657,41 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                     }
                 }
                 // every workgroup of the row stores the same count: no ordering needed
-                if (jq == 0 && tile == 0 && my_sub == 0 && p.part_cnt != nullptr) {
-                    p.part_cnt[static_cast<uint64_t>(tok) * p.n_heads + head0 + col] = single ? 0 : static_cast<int32_t>(n_tiles * p.n_sub);
+                if (!BALANCED && jq == 0 && cnt_value >= 0 && my_sub == 0 && p.part_cnt != nullptr) {
+                    p.part_cnt[static_cast<uint64_t>(tok) * p.n_heads + head0 + col] = cnt_value;
                 }
             }
+        }
+        __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
+    };
+
+    if constexpr (BALANCED) {
+        DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
+        split.scan();
+        if (split.total == 0) {
+            return;
+        }
+        split.for_each_segment([&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool whole, uint32_t pslot,
+                                   bool first_piece, int4 meta) {
+            run_segment(seq, tok, t0, t1, whole, static_cast<uint64_t>(pslot) * p.n_heads, 1u, -1, first_piece, meta);
+        });
+    } else {
+        const uint32_t tile = blockIdx.x;
+        const uint32_t seq = blockIdx.y;
+        const int32_t qlen = p.lens[seq];
+        const int32_t clen = p.cached_lens[seq];
+        const int32_t qstart = p.query_start_loc[seq];
+        for (int32_t r = 0; r < qlen; r++) {
+            const uint32_t tok = static_cast<uint32_t>(qstart + r);
+            const uint32_t limit = static_cast<uint32_t>(clen + r + 1);
+            const uint32_t n_tiles = ceil_div(limit, p.tile_tokens);
+            if (tile >= n_tiles) {
+                continue;
+            }
+            const uint32_t t0 = tile * p.tile_tokens;
+            run_segment(seq, tok, t0, min(limit, t0 + p.tile_tokens), false,
+                        static_cast<uint64_t>(tok) * p.n_heads * p.max_slots + tile * p.n_sub, p.max_slots,
+                        tile == 0 ? static_cast<int32_t>(n_tiles * p.n_sub) : -1, false, make_int4(0, 0, 0, 0));
         }
     }
 }
@@ -526,19 +718,6 @@ __device__ __forceinline__ void dma_wait()
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-// Work split of decode_dma_kernel: every sequence owns ceil(limit / 16) steps, limit its visible range; the
-// sequences' steps laid end to end are cut into equal chunks, one per workgroup (the lengths live in device
-// memory, so every workgroup computes the prefix sums itself), so that ragged batches keep every compute unit
-// equally busy. A chunk that crosses a sequence boundary runs as several segments. Only a chunk's first and
-// last segment can be parts of sequences that continue in other chunks: chunk c owns the partial slots 2c
-// (its first segment) and 2c + 1 (its last, when that is another one); a sequence cut into n segments that
-// starts in chunk c0 finds them at 2 c0 (+ 1 unless it is that chunk's first segment), 2 (c0 + 1), ...
-// and its meta entry (n, c0, first flag) tells the merge kernel so. Sequences inside one chunk are final.
-constexpr uint32_t kDmaTblCap = 1024;    // block-table entries staged per segment
-constexpr uint32_t kDmaSeqCap = 4096;    // sequences whose prefix sums fit in LDS (with 2^28 steps in all)
-constexpr uint32_t kDmaMinChunk = 16;    // steps: no chunk below 256 positions
-constexpr uint32_t kDmaMaxWorkgroups = 512;   // grid bound the partial slots are sized for (one workgroup per compute unit)
-
 template <typename T>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_dma_kernel(const DecodeMfmaParams p)
@@ -553,8 +732,6 @@ decode_dma_kernel(const DecodeMfmaParams p)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE);
-    uint32_t *wave_tot = tbl_lds + kDmaTblCap;   // kWaves entries
-    uint32_t *pref = wave_tot + kWaves;          // batch + 1 exclusive prefix sums of the step counts
     const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
         static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
 
@@ -588,110 +765,16 @@ decode_dma_kernel(const DecodeMfmaParams p)
 
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t row_bytes = p.n_kv_heads * HEADB;
-    const uint32_t B = p.batch;
 
-    // what is the same in every lane, said so: the copies take scalar addresses
-    auto uni = [](uint32_t x) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(x))); };
-    // ---- exclusive prefix sums of the sequences' step counts. Up to 64 sequences: every wave keeps them in
-    // its lanes (lane = sequence), nothing goes through LDS. More: thread t owns `ipt` consecutive sequences
-    // and the sums land in LDS, each entry packed with its sequence's (limit - 1) % 16.
-    const bool in_lanes = B <= 64;
-    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_tok = 0, total;
-    auto steps_of = [&](uint32_t i, uint32_t *limit) {
-        const int32_t ql = p.lens[i];
-        *limit = ql > 0 ? static_cast<uint32_t>(p.cached_lens[i] + 1) : 0u;   // the visible range of the sequence's row
-        if (ql <= 0 && blockIdx.x == 0) {
-            reinterpret_cast<int4 *>(p.part_meta)[p.query_start_loc[i]] = make_int4(0, 0, 0, 0);   // nothing to merge
-        }
-        return ceil_div(*limit, static_cast<uint32_t>(kStep));
-    };
-    if (in_lanes) {
-        if (lane < B) {
-            ln_tok = static_cast<uint32_t>(p.query_start_loc[lane]);
-            ln_steps = steps_of(lane, &ln_limit);
-        }
-        uint32_t incl = ln_steps;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t up = __shfl_up(incl, d);
-            incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
-        }
-        ln_pref = incl - ln_steps;
-        total = uni(__shfl(incl, 63));
-    } else {
-        const uint32_t ipt = ceil_div(B, static_cast<uint32_t>(kWaves * 64));
-        const uint32_t i0 = min(B, threadIdx.x * ipt), i1 = min(B, i0 + ipt);
-        uint32_t mine = 0, limit;
-        for (uint32_t i = i0; i < i1; i++) {
-            mine += steps_of(i, &limit);
-        }
-        uint32_t incl = mine;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t up = __shfl_up(incl, d);
-            incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
-        }
-        if (lane == 63) {
-            wave_tot[wave] = incl;
-        }
-        __syncthreads();
-        uint32_t before = 0;
-        for (uint32_t w = 0; w < wave; w++) {
-            before += wave_tot[w];
-        }
-        uint32_t run = before + incl - mine;
-        for (uint32_t i = i0; i < i1; i++) {
-            const uint32_t n = steps_of(i, &limit);
-            pref[i] = (run << 4) | ((limit - 1) & 15u);
-            run += n;
-        }
-        if (threadIdx.x == kWaves * 64 - 1) {
-            pref[B] = (before + incl) << 4;
-        }
-        __syncthreads();
-        total = uni(pref[B]) >> 4;
-    }
-    if (total == 0) {
+    DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
+    split.scan();
+    if (split.total == 0) {
         return;
     }
-    // first step, step count and visible range of sequence i
-    auto seq_info = [&](uint32_t i, uint32_t *first, uint32_t *n, uint32_t *limit) {
-        if (in_lanes) {
-            *first = uni(__shfl(ln_pref, static_cast<int>(i)));
-            *n = uni(__shfl(ln_steps, static_cast<int>(i)));
-            *limit = uni(__shfl(ln_limit, static_cast<int>(i)));
-        } else {
-            const uint32_t a = uni(pref[i]), b = uni(pref[i + 1]);
-            *first = a >> 4;
-            *n = (b >> 4) - *first;
-            *limit = *n == 0 ? 0u : (*n - 1) * kStep + (a & 15u) + 1;
-        }
-    };
-    // the sequence that holds step `start`: the last one whose prefix is <= start
-    auto seq_of = [&](uint32_t start) -> uint32_t {
-        if (in_lanes) {
-            const uint64_t mask = __ballot(lane < B && ln_pref <= start);
-            return static_cast<uint32_t>(__builtin_popcountll(mask)) - 1;
-        }
-        uint32_t lo = 0, hi = B;
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if ((uni(pref[mid]) >> 4) <= start) {
-                lo = mid;
-            } else {
-                hi = mid;
-            }
-        }
-        return lo;
-    };
-    uint32_t chunk = max(ceil_div(total, gridDim.x), kDmaMinChunk);
-    chunk = min(chunk, (kDmaTblCap - 2) * p.block_size / kStep);
-    const uint32_t n_chunks = ceil_div(total, chunk);
 
     // one segment: positions [t0, t1) of sequence `seq`
-    auto run_segment = [&](uint32_t seq_, uint32_t t0_, uint32_t t1_, bool whole, uint32_t pslot_, bool first_piece, int4 meta) {
-        const uint32_t seq = uni(seq_), t0 = uni(t0_), t1 = uni(t1_), pslot = uni(pslot_);
-        const uint32_t tok = in_lanes ? uni(__shfl(ln_tok, static_cast<int>(seq))) : static_cast<uint32_t>(p.query_start_loc[seq]);
+    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool whole, uint32_t pslot, bool first_piece,
+                           int4 meta) {
         const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
         const uint32_t n_steps = ceil_div(t1 - t0, kStep);
         const uint32_t blk0 = t0 / p.block_size;
@@ -854,33 +937,14 @@ decode_dma_kernel(const DecodeMfmaParams p)
         }
     };
 
-    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const uint32_t start = c * chunk, end = min(total, start + chunk);
-        uint32_t seq = seq_of(start), pos = start;
-        while (pos < end) {
-            uint32_t first, n, limit;
-            seq_info(seq, &first, &n, &limit);
-            if (n == 0) {
-                seq++;
-                continue;
-            }
-            const uint32_t a = pos - first, b = min(n, a + (end - pos));
-            const bool whole = a == 0 && b == n;
-            const bool first_seg = pos == start;
-            const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
-            const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
-            run_segment(seq, a * kStep, min(limit, b * kStep), whole, 2 * c + (first_seg ? 0u : 1u), a == 0, meta);
-            pos += b - a;
-            seq++;
-        }
-    }
+    split.for_each_segment(run_segment);
 }
 
 template <typename T>
 int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
-                       (kDmaTblCap + kWaves + p.batch + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + p.batch + 1) * sizeof(uint32_t);
     auto kernel = decode_dma_kernel<T>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
@@ -891,28 +955,29 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
     return XLITE_HIP_OK;
 }
 
+// `grid_x`: the number of workgroups of the balanced split (one sub range), tiles per sequence otherwise
 template <typename T, int D, bool KV8, bool MULTI_SUB>
-int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
+int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
-                       (p.tile_tokens / kStep + 2) * sizeof(uint32_t);
+                       (MULTI_SUB ? p.tile_tokens / kStep + 2 : kSplitLdsWords + p.batch + 1) * sizeof(uint32_t);
     auto kernel = decode_mfma_kernel<T, D, KV8, MULTI_SUB>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
             return rc;
         }
     }
-    dim3 grid(ceil_div(p.max_slots, p.n_sub), batch, 1);
+    dim3 grid(grid_x, MULTI_SUB ? p.batch : 1, 1);
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
 }
 
 template <typename T, int D, bool KV8>
-int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t batch)
+int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
-    return p.n_sub > 1 ? launch_inst<T, D, KV8, true>(stream, p, batch)
-                       : launch_inst<T, D, KV8, false>(stream, p, batch);
+    return p.n_sub > 1 ? launch_inst<T, D, KV8, true>(stream, p, grid_x)
+                       : launch_inst<T, D, KV8, false>(stream, p, grid_x);
 }
 
 }  // namespace
@@ -921,8 +986,9 @@ bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_
                            uint32_t total_tokens)
 {
     const uint32_t group = n_heads / n_kv_heads;
-    (void)total_tokens;
-    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16;
+    // one row per sequence; the balanced split (kv heads >= 8) keeps the batch's prefix sums in LDS
+    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16 &&
+           (n_kv_heads < kWaves || total_tokens <= kSplitSeqCap);
 }
 
 void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, uint32_t max_num_block,
@@ -947,88 +1013,45 @@ size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint
     return max_slots > 1 ? partial_bytes(total_tokens, n_heads, head_dim, max_slots) : 0;
 }
 
-// decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8, a batch whose prefix sums fit in LDS
-bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, uint32_t batch, int kv_dtype)
+// decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8
+bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
 {
-    return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0 && batch <= kDmaSeqCap;
+    return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0;
 }
 
 // The chunk the kernel really uses is the batch's total step count over the number of workgroups, which the
-// host cannot know (the lengths live in device memory); it is never below kDmaMinChunk steps nor above what
+// host cannot know (the lengths live in device memory); it is never below kSplitMinChunk steps nor above what
 // the block-table staging holds, which bounds the number of chunks and hence of partial slots (two per chunk).
-void decode_dma_plan(uint32_t batch, uint32_t n_heads, uint32_t block_size, uint32_t max_num_block, DecodeDmaPlan *pl)
+void decode_split_plan(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint32_t block_size, uint32_t max_num_block,
+                       DecodeSplitPlan *pl)
 {
     const uint64_t max_steps = ceil_div(max_num_block * block_size, static_cast<uint32_t>(kStep));
-    const uint64_t chunk_cap = static_cast<uint64_t>(kDmaTblCap - 2) * block_size / kStep;
+    const uint64_t chunk_cap = static_cast<uint64_t>(kSplitTblCap - 2) * block_size / kStep;
     const uint64_t by_cap = (static_cast<uint64_t>(batch) * max_steps + chunk_cap - 1) / chunk_cap;
-    pl->max_chunks = static_cast<uint32_t>(by_cap > kDmaMaxWorkgroups ? by_cap : kDmaMaxWorkgroups);
+    pl->max_chunks = static_cast<uint32_t>(by_cap > kSplitMaxWorkgroups ? by_cap : kSplitMaxWorkgroups);
     pl->meta_bytes = ((static_cast<size_t>(batch) * sizeof(int4) + 255) / 256) * 256;
     pl->ml_bytes = static_cast<size_t>(2) * pl->max_chunks * n_heads * 2 * sizeof(float);
-    pl->acc_bytes = static_cast<size_t>(2) * pl->max_chunks * n_heads * 128 * sizeof(float);
+    pl->acc_bytes = static_cast<size_t>(2) * pl->max_chunks * n_heads * head_dim * sizeof(float);
 }
 
-size_t decode_dma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t block_size, uint32_t max_num_block)
+// what launch_decode_mfma needs for this shape: per-chunk slots (kv heads >= 8) or per-tile slots
+size_t decode_mfma_workspace_for(uint32_t batch, uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                                 uint32_t head_dim, uint32_t block_size, uint32_t max_num_block)
 {
-    DecodeDmaPlan pl{};
-    decode_dma_plan(batch, n_heads, block_size, max_num_block, &pl);
-    return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
+    if (n_kv_heads >= kWaves) {
+        DecodeSplitPlan pl{};
+        decode_split_plan(batch, n_heads, head_dim, block_size, max_num_block, &pl);
+        return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
+    }
+    uint32_t tile, n_sub, max_slots;
+    decode_mfma_plan(batch, n_kv_heads, block_size, max_num_block, &tile, &n_sub, &max_slots);
+    return decode_mfma_workspace_bytes(total_tokens, n_heads, head_dim, max_slots);
 }
 
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
 {
-    if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.batch, a.kv_dtype)) {
-        DecodeDmaPlan pl{};
-        decode_dma_plan(a.batch, a.n_heads, a.block_size, a.max_num_block, &pl);
-        thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
-        int dev = 0;
-        XL_HIP(hipGetDevice(&dev));
-        if (dev != cu_dev) {
-            XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-            cu_dev = dev;
-        }
-        const uint32_t n_workgroups = min(static_cast<uint32_t>(n_cu), kDmaMaxWorkgroups);
-        const size_t need = pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
-        if (a.workspace == nullptr || a.workspace_bytes < need) {
-            return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
-                                                        " bytes, have " + std::to_string(a.workspace_bytes));
-        }
-        char *ws = static_cast<char *>(a.workspace);
-        DecodeMfmaParams p{};
-        p.q = static_cast<const uint16_t *>(a.qkv);
-        p.k_cache = a.k_cache;
-        p.v_cache = a.v_cache;
-        p.out = static_cast<uint16_t *>(a.output);
-        p.query_start_loc = a.query_start_loc;
-        p.lens = a.lens;
-        p.cached_lens = a.cached_lens;
-        p.block_tables = a.block_tables;
-        p.part_meta = reinterpret_cast<int32_t *>(ws);
-        p.part_ml = reinterpret_cast<float *>(ws + pl.meta_bytes);
-        p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
-        p.q_row_stride = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
-        p.n_heads = a.n_heads;
-        p.n_kv_heads = a.n_kv_heads;
-        p.group = a.n_heads / a.n_kv_heads;
-        p.block_size = a.block_size;
-        p.max_num_block = a.max_num_block;
-        p.batch = a.batch;
-        const int rc = a.dtype == XLITE_HIP_BF16 ? launch_dma<BF16>(stream, p, n_workgroups)
-                                                 : launch_dma<FP16>(stream, p, n_workgroups);
-        if (rc != XLITE_HIP_OK) {
-            return rc;
-        }
-        return launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens,
-                                 a.n_heads, a.head_dim);
-    }
-    uint32_t tile, n_sub, max_slots;
-    decode_mfma_plan(a.batch, a.n_kv_heads, a.block_size, a.max_num_block, &tile, &n_sub, &max_slots);
-    const size_t need = decode_mfma_workspace_bytes(a.total_tokens, a.n_heads, a.head_dim, max_slots);
-    if (max_slots > 1 && (a.workspace == nullptr || a.workspace_bytes < need)) {
-        return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
-                                                    " bytes, have " + std::to_string(a.workspace_bytes));
-    }
-    const PartialBuffers pb = max_slots > 1 ? carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_slots)
-                                            : PartialBuffers{};
+    const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
+    const bool bf = a.dtype == XLITE_HIP_BF16;
     DecodeMfmaParams p{};
     p.q = static_cast<const uint16_t *>(a.qkv);
     p.k_cache = a.k_cache;
@@ -1040,37 +1063,73 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     p.lens = a.lens;
     p.cached_lens = a.cached_lens;
     p.block_tables = a.block_tables;
-    p.part_cnt = pb.cnt;
-    p.part_acc = pb.acc;
-    p.part_ml = pb.ml;
     p.q_row_stride = (a.n_heads + 2 * a.n_kv_heads) * a.head_dim;
     p.n_heads = a.n_heads;
     p.n_kv_heads = a.n_kv_heads;
     p.group = a.n_heads / a.n_kv_heads;
     p.block_size = a.block_size;
     p.max_num_block = a.max_num_block;
-    p.tile_tokens = tile;
-    p.n_sub = n_sub;
-    p.max_slots = max_slots;
+    p.batch = a.batch;
+    const size_t need = decode_mfma_workspace_for(a.batch, a.total_tokens, a.n_heads, a.n_kv_heads, a.head_dim, a.block_size,
+                                                  a.max_num_block);
+    if (need > 0 && (a.workspace == nullptr || a.workspace_bytes < need)) {
+        return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
+                                                    " bytes, have " + std::to_string(a.workspace_bytes));
+    }
+    uint32_t grid_x;
+    const bool balanced = a.n_kv_heads >= kWaves;
+    PartialBuffers pb{};
+    if (balanced) {
+        DecodeSplitPlan pl{};
+        decode_split_plan(a.batch, a.n_heads, a.head_dim, a.block_size, a.max_num_block, &pl);
+        thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
+        int dev = 0;
+        XL_HIP(hipGetDevice(&dev));
+        if (dev != cu_dev) {
+            XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+            cu_dev = dev;
+        }
+        grid_x = min(static_cast<uint32_t>(n_cu), kSplitMaxWorkgroups);
+        char *ws = static_cast<char *>(a.workspace);
+        p.part_meta = reinterpret_cast<int32_t *>(ws);
+        p.part_ml = reinterpret_cast<float *>(ws + pl.meta_bytes);
+        p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
+        p.n_sub = 1;
+    } else {
+        uint32_t tile, n_sub, max_slots;
+        decode_mfma_plan(a.batch, a.n_kv_heads, a.block_size, a.max_num_block, &tile, &n_sub, &max_slots);
+        pb = carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_slots);
+        p.part_cnt = pb.cnt;
+        p.part_acc = pb.acc;
+        p.part_ml = pb.ml;
+        p.tile_tokens = tile;
+        p.n_sub = n_sub;
+        p.max_slots = max_slots;
+        grid_x = ceil_div(max_slots, n_sub);
+    }
 
-    const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
-    const bool bf = a.dtype == XLITE_HIP_BF16;
     int rc;
-    if (a.head_dim == 128) {
+    if (balanced && decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+        rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
+    } else if (a.head_dim == 128) {
         if (bf) {
-            rc = kv8 ? launch_one<BF16, 128, true>(stream, p, a.batch) : launch_one<BF16, 128, false>(stream, p, a.batch);
+            rc = kv8 ? launch_one<BF16, 128, true>(stream, p, grid_x) : launch_one<BF16, 128, false>(stream, p, grid_x);
         } else {
-            rc = kv8 ? launch_one<FP16, 128, true>(stream, p, a.batch) : launch_one<FP16, 128, false>(stream, p, a.batch);
+            rc = kv8 ? launch_one<FP16, 128, true>(stream, p, grid_x) : launch_one<FP16, 128, false>(stream, p, grid_x);
         }
     } else if (bf) {
-        rc = kv8 ? launch_one<BF16, 64, true>(stream, p, a.batch) : launch_one<BF16, 64, false>(stream, p, a.batch);
+        rc = kv8 ? launch_one<BF16, 64, true>(stream, p, grid_x) : launch_one<BF16, 64, false>(stream, p, grid_x);
     } else {
-        rc = kv8 ? launch_one<FP16, 64, true>(stream, p, a.batch) : launch_one<FP16, 64, false>(stream, p, a.batch);
+        rc = kv8 ? launch_one<FP16, 64, true>(stream, p, grid_x) : launch_one<FP16, 64, false>(stream, p, grid_x);
     }
-    if (rc != XLITE_HIP_OK || max_slots == 1) {
+    if (rc != XLITE_HIP_OK) {
         return rc;
     }
-    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, max_slots);
+    if (balanced) {
+        return launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens, a.n_heads,
+                                 a.head_dim);
+    }
+    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, p.max_slots);
 }
 
 }  // namespace xlite
