@@ -79,8 +79,9 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  *
  * workspace   device scratch of at least xlite_hip_attention_workspace_bytes()
  *             (split-KV partial results; contents need no initialisation and
- *             are not preserved). With a smaller or NULL workspace the call
- *             still works but splits the KV axis less, or not at all.
+ *             are not preserved). Decode batches need all of it
+ *             (XLITE_HIP_ENOSPC otherwise); a prefill batch given less, or
+ *             NULL, still works but does not split the KV axis.
  * ---------------------------------------------------------------------- */
 
 size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
