@@ -158,7 +158,7 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
-        "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_mfma_kernel (+ merge_kernel)", "achieved": round(achieved, 2),
+        "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_mfma_kernel (+ merge_meta_kernel)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name.split()[0]),
                      "algorithmic_bytes_per_launch": int(alg_bytes)},

@@ -24,7 +24,7 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
     const uint32_t max_ctx = max_num_block * block_size;
     if (is_decode_batch(total_tokens, batch)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
-            return decode_mfma_workspace_for(batch, total_tokens, n_heads, n_kv_heads, head_dim, block_size, max_num_block);
+            return decode_mfma_workspace_bytes(batch, n_heads, head_dim, block_size, max_num_block);
         }
         uint32_t g_kernel, head_chunks, nkv_wg, zdim;
         decode_geometry(n_heads, n_kv_heads, head_dim, &g_kernel, &head_chunks, &nkv_wg, &zdim);

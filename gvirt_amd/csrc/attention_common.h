@@ -76,16 +76,13 @@ int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_toke
 // decode_mfma.hip
 bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
                            uint32_t total_tokens);
-void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, uint32_t max_num_block,
-                      uint32_t *tile_tokens, uint32_t *n_sub, uint32_t *max_slots);
-size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim, uint32_t max_slots);
-int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
 struct DecodeSplitPlan {
     uint32_t max_chunks;   // bound on the number of chunks, hence of partial slots (two per chunk)
     size_t meta_bytes, ml_bytes, acc_bytes;
 };
-size_t decode_mfma_workspace_for(uint32_t batch, uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
-                                 uint32_t head_dim, uint32_t block_size, uint32_t max_num_block);
+size_t decode_mfma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint32_t block_size,
+                                   uint32_t max_num_block);
+int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
 
 // mla_decode.hip
 struct MlaDecodeParams {

@@ -74,18 +74,14 @@ struct DecodeMfmaParams {
     const int32_t *lens;
     const int32_t *cached_lens;
     const int32_t *block_tables;
-    int32_t *part_cnt; // [token][head] number of partial slots (0: final value stored directly)
-    float *part_acc;   // [token][head][slot][D]
-    float *part_ml;    // [token][head][slot][2]
+    int32_t *part_meta;    // [token] int4: segments to merge (0: final), first chunk, first-segment flag
+    float *part_acc;       // [slot][head][D]; chunk c of the work split owns slots 2c and 2c + 1
+    float *part_ml;        // [slot][head][2]: maximum (log2 domain), normaliser
     uint32_t q_row_stride;
     uint32_t n_heads, n_kv_heads, group;
     uint32_t block_size;
     uint32_t max_num_block;
-    uint32_t tile_tokens;  // multiple of kStep * n_sub
-    uint32_t n_sub;        // sub-ranges of a tile handled by different waves (kv heads < 8)
-    uint32_t max_slots;    // max tiles * n_sub
-    // decode_dma_kernel only: its partials sit in per-chunk slots, [slot][head][D] and [slot][head][2]
-    int32_t *part_meta;    // [token] int4: segments to merge (0: final), first chunk, first-segment flag
+    uint32_t n_sub;        // sub ranges of a segment handled by different waves (kv heads < 8)
     uint32_t batch;
 };
 
@@ -154,8 +150,11 @@ struct DecodeSplit {
     bool in_lanes;
     uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_tok = 0, total = 0, chunk = 0, n_chunks = 0;
 
-    __device__ __forceinline__ DecodeSplit(const DecodeMfmaParams &params, uint32_t *lds, uint32_t lane_, uint32_t wave_)
-        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_), B(params.batch), in_lanes(params.batch <= 64)
+    // `lanes_ok`: a kernel short of registers keeps the sums in LDS whatever the batch
+    __device__ __forceinline__ DecodeSplit(const DecodeMfmaParams &params, uint32_t *lds, uint32_t lane_, uint32_t wave_,
+                                           bool lanes_ok = true)
+        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_), B(params.batch),
+          in_lanes(lanes_ok && params.batch <= 64)
     {
     }
     __device__ __forceinline__ uint32_t steps_of(uint32_t i, uint32_t *limit) const
@@ -317,10 +316,6 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     // loop must not be a vector memory load, whose completion can only be awaited together with
     // every cache load issued before it (that would drain the prefetch pipeline at every step)
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE_BYTES + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0));
-    // Two ways to hand out work. One sub range per tile (kv heads >= 8): the balanced split of DecodeSplit,
-    // partials in per-chunk slots. Several sub ranges (fewer kv heads, the waves of a kv head share a tile):
-    // one workgroup per (sequence, tile of p.tile_tokens positions), partials at [token][head][tile][sub].
-    constexpr bool BALANCED = !MULTI_SUB;
 
     // ---- compute roles -------------------------------------------------------------------------------
     const uint32_t col = lane & 15;       // MFMA column = query head inside the group
@@ -372,12 +367,13 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t my_kvl = wave & (kvw - 1), my_sub = wave >> kvw_shift;
 
-    // one segment: positions [t0, t1) of the row `tok` of sequence `seq`. `single`: the result is final.
-    // Otherwise head h's partial goes to slot slot_base + h * slot_head_stride (+ the wave's sub range).
-    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool single, uint64_t slot_base,
-                           uint32_t slot_head_stride, int32_t cnt_value, bool write_meta, int4 meta) {
+    // one segment: positions [t0, t1) of the row `tok` of sequence `seq`. `single`: the result is final;
+    // otherwise it goes to partial slot `pslot`. With fewer than 8 kv heads the waves of a kv head take equal
+    // sub ranges of the segment and combine their results through LDS at its end.
+    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool single, uint32_t pslot, bool write_meta,
+                           int4 meta) {
         const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
-        const uint32_t sub_len = BALANCED ? t1 - t0 : p.tile_tokens / p.n_sub;
+        const uint32_t sub_len = ceil_div(ceil_div(t1 - t0, static_cast<uint32_t>(kStep)), p.n_sub) * kStep;
         // every sub range runs the same number of steps (the first one is never shorter than the others)
         const uint32_t n_steps = ceil_div(min(t1 - t0, sub_len), kStep);
         const uint32_t ta = min(t1, t0 + my_sub * sub_len);   // this wave's range
@@ -388,7 +384,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             for (uint32_t i = threadIdx.x; i < nblk; i += NT) {
                 tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
             }
-            if (BALANCED && write_meta && threadIdx.x == 0) {
+            if (write_meta && threadIdx.x == 0) {
                 reinterpret_cast<int4 *>(p.part_meta)[tok] = meta;
             }
             __syncthreads();
@@ -633,7 +629,45 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             // ---- this wave's result for (kv head, sub range) -----------------------------------------------
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
-            if (kv_ok && col < g_valid) {
+            if constexpr (MULTI_SUB) {
+                // the sub ranges of a kv head meet in its first wave: (m, l, O) of the others through the stage
+                // memory, which nobody reads any more (every wave has passed the loop's last barrier)
+                constexpr int XS = D + 4;   // floats per (wave, column): O, then m and l
+                float *xch = reinterpret_cast<float *>(smem);
+                if (my_sub != 0) {
+                    float *dst = xch + (wave * 16 + col) * XS;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
+                    }
+                    if (jq == 0) {
+                        dst[D] = m_run;
+                        dst[D + 1] = l_tot;
+                    }
+                }
+                __syncthreads();
+                if (my_sub == 0) {
+                    for (uint32_t sub = 1; sub < p.n_sub; sub++) {
+                        const float *src = xch + ((sub * kvw + my_kvl) * 16 + col) * XS;
+                        const float m2 = src[D], l2 = src[D + 1];
+                        const float m_new = fmaxf(m_run, m2);
+                        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                        const float a1 = fast_exp2(m_run - m_safe), a2 = fast_exp2(m2 - m_safe);
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++) {
+                            const float4 o2 = *reinterpret_cast<const float4 *>(src + mt * 16 + jq * 4);
+                            O[mt][0] = O[mt][0] * a1 + o2.x * a2;
+                            O[mt][1] = O[mt][1] * a1 + o2.y * a2;
+                            O[mt][2] = O[mt][2] * a1 + o2.z * a2;
+                            O[mt][3] = O[mt][3] * a1 + o2.w * a2;
+                        }
+                        l_tot = l_tot * a1 + l2 * a2;
+                        m_run = m_new;
+                    }
+                }
+                __syncthreads();   // the next pass refills the stages
+            }
+            if (kv_ok && col < g_valid && my_sub == 0) {
                 // O^T lane layout: column = head `col`, rows 16 mt + 4 jq + e
                 if (single) {
                     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -646,7 +680,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<uint2 *>(dst + mt * 16 + jq * 4) = o;
                     }
                 } else {
-                    const uint64_t slot = slot_base + static_cast<uint64_t>(head0 + col) * slot_head_stride + my_sub;
+                    const uint64_t slot = static_cast<uint64_t>(pslot) * p.n_heads + head0 + col;
                     float *dst = p.part_acc + slot * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
@@ -656,44 +690,17 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
                     }
                 }
-                // every workgroup of the row stores the same count: no ordering needed
-                if (!BALANCED && jq == 0 && cnt_value >= 0 && my_sub == 0 && p.part_cnt != nullptr) {
-                    p.part_cnt[static_cast<uint64_t>(tok) * p.n_heads + head0 + col] = cnt_value;
-                }
             }
         }
         __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
     };
 
-    if constexpr (BALANCED) {
-        DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
-        split.scan();
-        if (split.total == 0) {
-            return;
-        }
-        split.for_each_segment([&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool whole, uint32_t pslot,
-                                   bool first_piece, int4 meta) {
-            run_segment(seq, tok, t0, t1, whole, static_cast<uint64_t>(pslot) * p.n_heads, 1u, -1, first_piece, meta);
-        });
-    } else {
-        const uint32_t tile = blockIdx.x;
-        const uint32_t seq = blockIdx.y;
-        const int32_t qlen = p.lens[seq];
-        const int32_t clen = p.cached_lens[seq];
-        const int32_t qstart = p.query_start_loc[seq];
-        for (int32_t r = 0; r < qlen; r++) {
-            const uint32_t tok = static_cast<uint32_t>(qstart + r);
-            const uint32_t limit = static_cast<uint32_t>(clen + r + 1);
-            const uint32_t n_tiles = ceil_div(limit, p.tile_tokens);
-            if (tile >= n_tiles) {
-                continue;
-            }
-            const uint32_t t0 = tile * p.tile_tokens;
-            run_segment(seq, tok, t0, min(limit, t0 + p.tile_tokens), false,
-                        static_cast<uint64_t>(tok) * p.n_heads * p.max_slots + tile * p.n_sub, p.max_slots,
-                        tile == 0 ? static_cast<int32_t>(n_tiles * p.n_sub) : -1, false, make_int4(0, 0, 0, 0));
-        }
+    DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave, !(MULTI_SUB && D == 128));
+    split.scan();
+    if (split.total == 0) {
+        return;
     }
+    split.for_each_segment(run_segment);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -955,19 +962,18 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
     return XLITE_HIP_OK;
 }
 
-// `grid_x`: the number of workgroups of the balanced split (one sub range), tiles per sequence otherwise
 template <typename T, int D, bool KV8, bool MULTI_SUB>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
-                       (MULTI_SUB ? p.tile_tokens / kStep + 2 : kSplitLdsWords + p.batch + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + p.batch + 1) * sizeof(uint32_t);
     auto kernel = decode_mfma_kernel<T, D, KV8, MULTI_SUB>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
             return rc;
         }
     }
-    dim3 grid(grid_x, MULTI_SUB ? p.batch : 1, 1);
+    dim3 grid(grid_x, 1, 1);
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
@@ -986,31 +992,9 @@ bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_
                            uint32_t total_tokens)
 {
     const uint32_t group = n_heads / n_kv_heads;
-    // one row per sequence; the balanced split (kv heads >= 8) keeps the batch's prefix sums in LDS
-    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16 &&
-           (n_kv_heads < kWaves || total_tokens <= kSplitSeqCap);
-}
-
-void decode_mfma_plan(uint32_t batch, uint32_t n_kv_heads, uint32_t block_size, uint32_t max_num_block,
-                      uint32_t *tile_tokens, uint32_t *n_sub, uint32_t *max_slots)
-{
-    const uint32_t subs = n_kv_heads >= kWaves ? 1 : kWaves / n_kv_heads;
-    const uint64_t max_ctx = static_cast<uint64_t>(max_num_block) * block_size;
-    const uint64_t quantum = static_cast<uint64_t>(kStep) * subs;
-    // about one workgroup per compute unit if every sequence were as long as its block table
-    // allows, but never tiles above 1024 positions (ragged batches balance through many tiles)
-    // nor below 256 (the fp32 partials must stay a small fraction of the KV bytes)
-    uint64_t tile = max_ctx * batch / 256;
-    tile = tile > 1024 ? 1024 : (tile < 256 ? 256 : tile);
-    tile = (tile + quantum - 1) / quantum * quantum;
-    *tile_tokens = static_cast<uint32_t>(tile);
-    *n_sub = subs;
-    *max_slots = static_cast<uint32_t>((max_ctx + tile - 1) / tile) * subs;
-}
-
-size_t decode_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t head_dim, uint32_t max_slots)
-{
-    return max_slots > 1 ? partial_bytes(total_tokens, n_heads, head_dim, max_slots) : 0;
+    // one row per sequence; the work split keeps the batch's prefix sums in LDS
+    (void)n_kv_heads;
+    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16 && total_tokens <= kSplitSeqCap;
 }
 
 // decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8
@@ -1034,18 +1018,12 @@ void decode_split_plan(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint
     pl->acc_bytes = static_cast<size_t>(2) * pl->max_chunks * n_heads * head_dim * sizeof(float);
 }
 
-// what launch_decode_mfma needs for this shape: per-chunk slots (kv heads >= 8) or per-tile slots
-size_t decode_mfma_workspace_for(uint32_t batch, uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
-                                 uint32_t head_dim, uint32_t block_size, uint32_t max_num_block)
+size_t decode_mfma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint32_t block_size,
+                                   uint32_t max_num_block)
 {
-    if (n_kv_heads >= kWaves) {
-        DecodeSplitPlan pl{};
-        decode_split_plan(batch, n_heads, head_dim, block_size, max_num_block, &pl);
-        return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
-    }
-    uint32_t tile, n_sub, max_slots;
-    decode_mfma_plan(batch, n_kv_heads, block_size, max_num_block, &tile, &n_sub, &max_slots);
-    return decode_mfma_workspace_bytes(total_tokens, n_heads, head_dim, max_slots);
+    DecodeSplitPlan pl{};
+    decode_split_plan(batch, n_heads, head_dim, block_size, max_num_block, &pl);
+    return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
 }
 
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
@@ -1070,46 +1048,29 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     p.block_size = a.block_size;
     p.max_num_block = a.max_num_block;
     p.batch = a.batch;
-    const size_t need = decode_mfma_workspace_for(a.batch, a.total_tokens, a.n_heads, a.n_kv_heads, a.head_dim, a.block_size,
-                                                  a.max_num_block);
-    if (need > 0 && (a.workspace == nullptr || a.workspace_bytes < need)) {
+    DecodeSplitPlan pl{};
+    decode_split_plan(a.batch, a.n_heads, a.head_dim, a.block_size, a.max_num_block, &pl);
+    const size_t need = pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
+    if (a.workspace == nullptr || a.workspace_bytes < need) {
         return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +
                                                     " bytes, have " + std::to_string(a.workspace_bytes));
     }
-    uint32_t grid_x;
-    const bool balanced = a.n_kv_heads >= kWaves;
-    PartialBuffers pb{};
-    if (balanced) {
-        DecodeSplitPlan pl{};
-        decode_split_plan(a.batch, a.n_heads, a.head_dim, a.block_size, a.max_num_block, &pl);
-        thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
-        int dev = 0;
-        XL_HIP(hipGetDevice(&dev));
-        if (dev != cu_dev) {
-            XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-            cu_dev = dev;
-        }
-        grid_x = min(static_cast<uint32_t>(n_cu), kSplitMaxWorkgroups);
-        char *ws = static_cast<char *>(a.workspace);
-        p.part_meta = reinterpret_cast<int32_t *>(ws);
-        p.part_ml = reinterpret_cast<float *>(ws + pl.meta_bytes);
-        p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
-        p.n_sub = 1;
-    } else {
-        uint32_t tile, n_sub, max_slots;
-        decode_mfma_plan(a.batch, a.n_kv_heads, a.block_size, a.max_num_block, &tile, &n_sub, &max_slots);
-        pb = carve_partials(a.workspace, a.total_tokens, a.n_heads, a.head_dim, max_slots);
-        p.part_cnt = pb.cnt;
-        p.part_acc = pb.acc;
-        p.part_ml = pb.ml;
-        p.tile_tokens = tile;
-        p.n_sub = n_sub;
-        p.max_slots = max_slots;
-        grid_x = ceil_div(max_slots, n_sub);
+    thread_local int cu_dev = -1, n_cu = 0;   // the compute-unit count of the device this thread last used
+    int dev = 0;
+    XL_HIP(hipGetDevice(&dev));
+    if (dev != cu_dev) {
+        XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+        cu_dev = dev;
     }
+    const uint32_t grid_x = min(static_cast<uint32_t>(n_cu), kSplitMaxWorkgroups);
+    char *ws = static_cast<char *>(a.workspace);
+    p.part_meta = reinterpret_cast<int32_t *>(ws);
+    p.part_ml = reinterpret_cast<float *>(ws + pl.meta_bytes);
+    p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
+    p.n_sub = a.n_kv_heads >= kWaves ? 1 : kWaves / a.n_kv_heads;
 
     int rc;
-    if (balanced && decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+    if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
         rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
     } else if (a.head_dim == 128) {
         if (bf) {
@@ -1125,11 +1086,8 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     if (rc != XLITE_HIP_OK) {
         return rc;
     }
-    if (balanced) {
-        return launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens, a.n_heads,
-                                 a.head_dim);
-    }
-    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, p.max_slots);
+    return launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens, a.n_heads,
+                             a.head_dim);
 }
 
 }  // namespace xlite

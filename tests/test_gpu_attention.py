@@ -119,11 +119,15 @@ def test_decode_wide_groups_and_small_blocks(rt, model, work):
 @pytest.mark.parametrize("model,batch,lo,hi,long_ones", [((32, 8, 128, 128, torch.bfloat16), 100, 1, 3000, [9000, 5000]),
                                                         ((32, 8, 128, 128, torch.bfloat16), 700, 1, 200, [2500]),
                                                         ((16, 8, 128, 16, torch.float16), 70, 1, 900, []),
-                                                        ((64, 16, 128, 64, torch.bfloat16), 40, 100, 2000, [])])
+                                                        ((64, 16, 128, 64, torch.bfloat16), 40, 100, 2000, []),
+                                                        ((14, 2, 64, 128, torch.bfloat16), 100, 1, 1500, [7000]),
+                                                        ((28, 4, 128, 128, torch.float16), 70, 1, 2000, [6000, 33]),
+                                                        ((4, 1, 128, 16, torch.bfloat16), 30, 1, 700, [])])
 def test_decode_ragged_batches_balanced_split(rt, model, batch, lo, hi, long_ones):
     """Ragged decode batches on the shapes of the streaming decode kernel: the sequences' steps are cut into
     equal chunks across workgroups, so chunks hold whole short sequences, tails and heads of long ones; more
-    than 64 sequences take the prefix sums through LDS, more than 512 several sequences per thread."""
+    than 64 sequences take the prefix sums through LDS, more than 512 several sequences per thread. With fewer
+    than 8 kv heads the waves of a kv head share a segment and combine their parts inside the workgroup."""
     nH, nKV, d, bs, dtype = model
     rng = np.random.default_rng(batch)
     clens = [int(x) for x in rng.integers(lo, hi, size=batch)]
@@ -141,6 +145,13 @@ def test_decode_int8_kv(rt):
     # and against the unquantised cache the error stays within the int8 budget as well
     w16 = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=False)
     check(got, oracle_attention(w16), max_abs=MAX_ABS_INT8, mean_abs=1e-2)
+
+
+def test_decode_int8_kv_ragged_batch(rt):
+    rng = np.random.default_rng(3)
+    ctx = [int(x) for x in np.exp(rng.uniform(np.log(16), np.log(6000), 90))]
+    w = W.gqa_decode(W.LLAMA3_8B, ctx, 78, int8_kv=True)
+    check(run_attention(rt, w), oracle_attention(w), max_abs=MAX_ABS_INT8)
 
 
 def test_config2_llama3_8b_decode_sampled(rt):
