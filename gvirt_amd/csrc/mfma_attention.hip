@@ -111,18 +111,27 @@ mfma_attention_kernel(const MfmaParams p)
     const uint32_t kvh = blockIdx.z;
     const uint32_t G = p.rows_per_pos;
 
-    // ---- locate the M tile: tiles are numbered sequence by sequence ---------------------------
-    uint32_t seq = 0, mt = blockIdx.y;
-    int32_t qlen = 0;
-    for (; seq < p.batch; seq++) {
-        qlen = p.lens[seq];
-        const uint32_t tiles = ceil_div(static_cast<uint32_t>(qlen > 0 ? qlen : 0) * G, kMTile);
-        if (mt < tiles) {
-            break;
+    // ---- locate the M tile. Sequence i owns the tile ids from floor(query_start_loc[i] * G / 128) + i up to
+    // the next sequence's first one: at least its ceil(lens[i] * G / 128) tiles (the surplus ids are empty),
+    // and a formula of the prefix sums the caller provides, so the owner is found by bisection.
+    auto first_id = [&](uint32_t i) {
+        return static_cast<uint32_t>((static_cast<uint64_t>(p.query_start_loc[i]) * G) / kMTile) + i;
+    };
+    uint32_t seq = 0;
+    {
+        uint32_t hi = p.batch;   // first_id(seq) <= blockIdx.y < first_id(hi); first_id(0) == 0
+        while (hi - seq > 1) {
+            const uint32_t mid = (seq + hi) >> 1;
+            if (first_id(mid) <= blockIdx.y) {
+                seq = mid;
+            } else {
+                hi = mid;
+            }
         }
-        mt -= tiles;
     }
-    if (seq >= p.batch) {
+    const uint32_t mt = blockIdx.y - first_id(seq);
+    const int32_t qlen = p.lens[seq];
+    if (qlen <= 0 || mt >= ceil_div(static_cast<uint32_t>(qlen) * G, kMTile)) {
         return;
     }
     const int32_t clen = p.cached_lens[seq];

@@ -142,18 +142,29 @@ prefill_kernel(const PrefillParams p)
             return;
         }
     }
-    // ---- locate the M tile: tiles are numbered sequence by sequence; the grid runs them backwards ----
-    uint32_t seq = 0, mt = p.n_mtiles - 1 - mt_fwd;
-    int32_t qlen = 0;
-    for (; seq < p.batch; seq++) {
-        qlen = p.lens[seq];
-        const uint32_t tiles = ceil_div(static_cast<uint32_t>(qlen > 0 ? qlen : 0) * G, static_cast<uint32_t>(kMTile));
-        if (mt < tiles) {
-            break;
+    // ---- locate the M tile; the grid runs the tile ids backwards. Sequence i owns the ids from
+    // floor(query_start_loc[i] * G / 256) + i up to the next sequence's first one: at least its
+    // ceil(lens[i] * G / 256) tiles (the surplus ids are empty), and a formula of the prefix sums the caller
+    // provides, so the owner of an id is found by bisection, not by a walk over the batch.
+    const uint32_t tid = p.n_mtiles - 1 - mt_fwd;
+    auto first_id = [&](uint32_t i) {
+        return static_cast<uint32_t>((static_cast<uint64_t>(p.query_start_loc[i]) * G) / kMTile) + i;
+    };
+    uint32_t seq = 0;
+    {
+        uint32_t hi = p.batch;   // first_id(seq) <= tid < first_id(hi); first_id(0) == 0
+        while (hi - seq > 1) {
+            const uint32_t mid = (seq + hi) >> 1;
+            if (first_id(mid) <= tid) {
+                seq = mid;
+            } else {
+                hi = mid;
+            }
         }
-        mt -= tiles;
     }
-    if (seq >= p.batch) {
+    const uint32_t mt = tid - first_id(seq);
+    const int32_t qlen = p.lens[seq];
+    if (qlen <= 0 || mt >= ceil_div(static_cast<uint32_t>(qlen) * G, static_cast<uint32_t>(kMTile))) {
         return;
     }
     const int32_t clen = p.cached_lens[seq];
@@ -527,7 +538,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.block_size = a.block_size;
     p.block_magic = static_cast<uint32_t>((1ull << 32) / a.block_size) + 1;
     p.max_num_block = a.max_num_block;
-    // upper bound on the number of M tiles: every sequence may end with a ragged one
+    // tile ids: every sequence may end with a ragged tile (see the kernel's numbering)
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
     p.n_heads = a.n_heads;
     uint32_t splits = prefill_mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, a.max_num_block * a.block_size);
