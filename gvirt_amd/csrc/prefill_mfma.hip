@@ -1,4 +1,4 @@
-// Chunked causal prefill over the paged GQA cache on the matrix cores (head_dim 128, 16-bit cache).
+// Chunked causal prefill over the paged GQA cache on the matrix cores (head_dim 128 or 64, 16-bit cache).
 //
 // Workgroup = 8 wavefronts (two per SIMD: while one waits for LDS or does its softmax on the vector
 // ALU, the other keeps the matrix pipe busy) = 256 "M rows" of one kv head, an M row being one
@@ -10,7 +10,8 @@
 // = four consecutive positions of the kv head = 1 KiB of LDS) into a ring of four 32 KiB stages; V
 // stays row major and is transposed on the way out of LDS, so no transposing stores are needed. The
 // 16-byte chunks of a row are XOR-swizzled by the position (the lane chooses which global chunk lands
-// in its LDS slot) so that both read shapes are bank-conflict free.
+// in its LDS slot) so that both read shapes are bank-conflict free. With head_dim 64 a 256-byte bank
+// window holds two positions, a copy instruction eight, and the pattern is a function of the window.
 // M tiles are numbered sequence by sequence and launched last-first: the tiles with the longest
 // visible range start first. When there are fewer M tiles than compute units (a short chunk after a
 // long cached context, decode rows mixed into the batch), grid.y splits every tile's visible range into
@@ -31,16 +32,9 @@ constexpr int kWaves = 8;
 constexpr int kXcds = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kMTile = kWaves * 32;
-constexpr int D = 128;
 constexpr int BN = 64;                    // positions per KV tile
-constexpr int ROWB = D * 2;               // 256: bytes of one (position, kv head) row
-constexpr int KBYTES = BN * ROWB;         // 16 KiB
-constexpr int STAGE = 2 * KBYTES;         // K tile, then V tile
 constexpr int kStages = 4;
-constexpr int KS = D / 16;                // k-steps of the QK product
 constexpr int NT = BN / 32;               // 32-position sub tiles
-constexpr int DT = D / 32;                // 32-row tiles of O^T
-constexpr int PER_WAVE = 2 * BN / 4 / kWaves;   // copies per wave and tile (4)
 constexpr uint32_t kMinSplitTiles = 8;          // a KV split walks at least 512 positions
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
@@ -93,6 +87,20 @@ struct PrefillParams {
 // 16 rows that one ds_read_b128 pass touches get 16 different chunk slots, and the 4 rows that one
 // transposing pass touches get 4 different 64-byte groups.
 __device__ __forceinline__ uint32_t swz(uint32_t row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// head_dim 64: pattern of bank window `win` (two positions of 128 bytes; the upper half of the 16 chunk slots
+// belongs to the odd position, so only the low three bits move). Eight consecutive windows get eight
+// different values, neighbours differ in bit 2 (the 64-byte group a transposing pass reads).
+__device__ __forceinline__ uint32_t swz64(uint32_t win) { return ((win & 1) << 2) | ((win >> 1) & 3); }
+// byte offset inside a K or V tile of 16-byte chunk `chunk` of position `pos`
+template <int D>
+__device__ __forceinline__ uint32_t tile_off(uint32_t pos, uint32_t chunk)
+{
+    if constexpr (D == 128) {
+        return pos * 256 + ((chunk ^ swz(pos)) << 4);
+    } else {
+        return (pos >> 1) * 256 + (((((pos & 1) << 3) | chunk) ^ swz64(pos >> 1)) << 4);
+    }
+}
 
 // One wave-wide copy of 1 KiB from global memory into LDS at `lds_addr` + 16 * lane. The compiler sees
 // neither the LDS write nor the memory counter: completion is awaited with dma_wait.
@@ -107,10 +115,18 @@ __device__ __forceinline__ void dma_wait()
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-template <typename T>
+template <typename T, int D>
 __global__ void __launch_bounds__(kThreads, 1)
 prefill_kernel(const PrefillParams p)
 {
+    constexpr int ROWB = D * 2;               // bytes of one (position, kv head) row
+    constexpr int KBYTES = BN * ROWB;         // 16 KiB (8 KiB for head_dim 64)
+    constexpr int STAGE = 2 * KBYTES;         // K tile, then V tile
+    constexpr int KS = D / 16;                // k-steps of the QK product
+    constexpr int DT = D / 32;                // 32-row tiles of O^T
+    constexpr int PPC = 1024 / ROWB;          // positions per copy instruction (4 or 8)
+    constexpr int CPT = BN / PPC / kWaves;    // copies per wave, tile and tensor (2 or 1)
+    constexpr int PER_WAVE = 2 * CPT;         // copies per wave and tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
         static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
@@ -234,9 +250,10 @@ prefill_kernel(const PrefillParams p)
     float m_run = -INFINITY, l_run = 0.f;
 
     // ---- read roles ------------------------------------------------------------------------------------
-    // K rows as the A operand: row = position nt * 32 + col, chunk 2 ks + half
-    const uint32_t kx = (half ^ swz(col)) << 4;           // swz(col + 32) == swz(col)
-    const uint32_t k_row = col * ROWB;
+    // K rows as the A operand: row = position nt * 32 + col, chunk 2 ks + half. The pattern of position
+    // col + 32 is that of col, so one XOR term serves both sub tiles.
+    const uint32_t kx = D == 128 ? (half ^ swz(col)) << 4 : ((((col & 1) << 3) | half) ^ swz64(col >> 1)) << 4;
+    const uint32_t k_row = D == 128 ? col * 256 : (col >> 1) * 256;
     // transposed V: 16-lane group g covers columns 16 (g % 2) .. +16 of a 32-column tile for the
     // positions of half g / 2; lane 4 j' + q points at elements [4 q, +4) of position 4 half + j' (+8 for
     // the second read of a 16-position k-step)
@@ -245,32 +262,47 @@ prefill_kernel(const PrefillParams p)
         const uint32_t g = lane >> 4, jp = (lane & 15) >> 2, q = lane & 3;
         const uint32_t y = 2 * (g & 1) + (q >> 1);
         const uint32_t pos = 4 * (g >> 1) + jp;
-        vr_off = KBYTES + pos * ROWB + ((y ^ swz(pos)) << 4) + ((q & 1) << 3);
+        vr_off = KBYTES + tile_off<D>(pos, y) + ((q & 1) << 3);
     }
-    // ---- copy role: wave w moves positions 8w .. 8w+7 of the tile, four per copy, for K and for V.
-    // Lane = (position inside the four) * 16 + chunk slot; the slot receives chunk slot ^ pattern(position).
-    uint32_t c_voff[2];
+    // ---- copy role: wave w moves positions 8w .. 8w+7 of the tile, for K and for V: two copies of four
+    // positions (head_dim 128) or one of eight. A copy fills 1 KiB of LDS, lane l the 16 bytes at 16 l: bank
+    // window l / 16 of the copy, chunk slot l % 16; the slot receives the (position, chunk) whose pattern
+    // maps there. copy_src: that position (relative to the copy's first) and its chunk.
+    auto copy_src = [&](uint32_t first_pos, uint32_t *rel, uint32_t *chunk) {
+        if constexpr (D == 128) {
+            *rel = lane >> 4;
+            *chunk = (lane & 15u) ^ swz(first_pos + (lane >> 4));
+        } else {
+            const uint32_t c16 = (lane & 15u) ^ swz64((first_pos >> 1) + (lane >> 4));
+            *rel = 2 * (lane >> 4) + (c16 >> 3);
+            *chunk = c16 & 7u;
+        }
+    };
+    uint32_t c_voff[CPT];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t pos = 8 * wave + 4 * i + (lane >> 4);
-        c_voff[i] = (lane >> 4) * row_bytes + (((lane & 15u) ^ swz(pos)) << 4);
+    for (int i = 0; i < CPT; i++) {
+        uint32_t rel, chunk;
+        copy_src(PPC * (CPT * wave + i), &rel, &chunk);
+        c_voff[i] = rel * row_bytes + (chunk << 4);
     }
 
-    // copies of KV tile `tile` into stage tile % 3. Four consecutive positions share one block
-    // (block_size % 4 == 0). Positions at or beyond the end of the range re-read the last valid one
+    // copies of KV tile `tile` into stage tile % 4. The positions of a copy share one block (block_size a
+    // multiple of the four or eight). Positions at or beyond the end of the range re-read the last valid one
     // (finite values; their probabilities are masked to zero).
     auto issue = [&](uint32_t tile) {
         const uint32_t st = smem_addr + (tile % kStages) * STAGE;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const uint32_t pos = 8 * wave + 4 * i;
+        for (int i = 0; i < CPT; i++) {
+            const uint32_t pos = PPC * (CPT * wave + i);
             uint32_t t = tile * BN + pos;
             uint32_t voff = c_voff[i];
-            if (t + 3 >= range_end) {   // uniform; only the last tile
+            if (t + PPC - 1 >= range_end) {   // uniform; only the last tile
                 const uint32_t lim = range_end - 1;
-                const uint32_t tl = min(t + (lane >> 4), lim);
-                t = min(t, lim) & ~3u;
-                voff = (tl - t) * row_bytes + (((lane & 15u) ^ swz(pos + (lane >> 4))) << 4);
+                uint32_t rel, chunk;
+                copy_src(pos, &rel, &chunk);
+                const uint32_t tl = min(t + rel, lim);
+                t = min(t, lim) & ~static_cast<uint32_t>(PPC - 1);
+                voff = (tl - t) * row_bytes + (chunk << 4);
             }
             // block-table entries come from LDS (copied there once): a vector load here would have to be
             // awaited together with every copy issued before it
@@ -481,7 +513,9 @@ prefill_kernel(const PrefillParams p)
 bool prefill_mfma_supported(const AttentionArgs &a)
 {
     // the division by the block size is a multiply-high, exact while position * block_size < 2^32
-    return a.head_dim == D && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size >= 4 && a.block_size % 4 == 0 &&
+    // the positions of one copy instruction (1 KiB: four rows of head_dim 128, eight of head_dim 64) share a block
+    const uint32_t per_copy = a.head_dim == 128 ? 4 : 8;
+    return (a.head_dim == 128 || a.head_dim == 64) && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size % per_copy == 0 &&
            static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32) &&
            a.n_heads % a.n_kv_heads == 0;
 }
@@ -552,11 +586,16 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.part_acc = pb.acc;
     p.part_ml = pb.ml;
 
-    const size_t lds = static_cast<size_t>(kStages) * STAGE + (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
+    const size_t lds = static_cast<size_t>(kStages) * 2 * BN * a.head_dim * 2 +
+                       (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     const bool bf = a.dtype == XLITE_HIP_BF16;
     XL_REQUIRE(lds <= 160 * 1024, "block table too long for the prefill kernel");
-    if (const int rc = ensure_dynamic_lds(bf ? reinterpret_cast<const void *>(prefill_kernel<BF16>)
-                                             : reinterpret_cast<const void *>(prefill_kernel<FP16>), lds)) {
+    const void *kernel = a.head_dim == 128
+                             ? (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 128>)
+                                   : reinterpret_cast<const void *>(prefill_kernel<FP16, 128>))
+                             : (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 64>)
+                                   : reinterpret_cast<const void *>(prefill_kernel<FP16, 64>));
+    if (const int rc = ensure_dynamic_lds(kernel, lds)) {
         return rc;
     }
     uint32_t n_wg;
@@ -568,10 +607,16 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
         n_wg = a.n_kv_heads * p.n_mtiles;
     }
     dim3 grid(n_wg, splits, 1);
-    if (bf) {
-        prefill_kernel<BF16><<<grid, kThreads, lds, stream>>>(p);
+    if (a.head_dim == 128) {
+        if (bf) {
+            prefill_kernel<BF16, 128><<<grid, kThreads, lds, stream>>>(p);
+        } else {
+            prefill_kernel<FP16, 128><<<grid, kThreads, lds, stream>>>(p);
+        }
+    } else if (bf) {
+        prefill_kernel<BF16, 64><<<grid, kThreads, lds, stream>>>(p);
     } else {
-        prefill_kernel<FP16><<<grid, kThreads, lds, stream>>>(p);
+        prefill_kernel<FP16, 64><<<grid, kThreads, lds, stream>>>(p);
     }
     XL_LAUNCH_CHECK();
     if (splits == 1) {

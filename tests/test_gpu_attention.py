@@ -105,7 +105,8 @@ def test_decode_special_cases(rt):
 
 @pytest.mark.parametrize("model", [(64, 2, 128, 128, torch.bfloat16), (64, 1, 128, 64, torch.float16), (40, 2, 128, 16, torch.bfloat16),
                                    (32, 8, 128, 8, torch.bfloat16), (8, 2, 128, 4, torch.bfloat16),
-                                   (48, 2, 128, 48, torch.bfloat16), (8, 2, 128, 20, torch.bfloat16)])
+                                   (48, 2, 128, 48, torch.bfloat16), (8, 2, 128, 20, torch.bfloat16),
+                                   (40, 2, 64, 128, torch.bfloat16), (6, 2, 64, 8, torch.float16)])
 @pytest.mark.parametrize("work", DECODE_WORK)
 def test_decode_wide_groups_and_small_blocks(rt, model, work):
     """More than 16 query heads per kv head, and block sizes that are not a multiple of 16: decode batches the
@@ -212,7 +213,8 @@ SPLIT_WORK = [([3000], [100]), ([16384], [128]), ([2047, 1500, 0, 4000], [1, 1, 
 
 @pytest.mark.parametrize("model", [(8, 2, 128, 128, torch.bfloat16), (32, 8, 128, 128, torch.bfloat16),
                                    (16, 4, 128, 16, torch.float16), (28, 4, 128, 64, torch.bfloat16),
-                                   (8, 2, 128, 48, torch.bfloat16), (6, 2, 128, 12, torch.float16)])
+                                   (8, 2, 128, 48, torch.bfloat16), (6, 2, 128, 12, torch.float16),
+                                   (14, 2, 64, 128, torch.bfloat16), (8, 8, 64, 8, torch.float16), (12, 4, 64, 24, torch.bfloat16)])
 @pytest.mark.parametrize("work", SPLIT_WORK)
 def test_prefill_few_tiles_over_long_context(rt, model, work):
     """Short chunks after a long cached context and decode rows mixed with a prefill: fewer M tiles than
