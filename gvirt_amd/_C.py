@@ -471,6 +471,63 @@ def rope_complex(rt: Runtime, n_local_heads: int, step_dim: int, rope_dim: int, 
     rt.finish()
 
 
+def rope_complex_and_cache(rt: Runtime, n_local_heads: int, step_dim: int, rope_dim: int, offset: int, vdim: int,
+                           input_with_r: torch.Tensor, freqs: torch.Tensor, position: torch.Tensor,
+                           output: Optional[torch.Tensor] = None, out_step_dim: int = 0, out_offset: int = 0,
+                           block_size: int = 0, cache: Optional[torch.Tensor] = None,
+                           slot_mapping: Optional[torch.Tensor] = None) -> None:
+    """The general interleaved-pair rope (no Python binding in the reference; XliteOpRopeComplex and
+    XliteOpRopeComplexAndCache, xlite/csrc/op.cpp:1106-1150): the rope_dim columns from `offset` of every head,
+    to `output` (which may be the input) or, with a cache, the vdim columns from `offset` to cache[slot]."""
+    _dev("input_with_r", input_with_r)
+    _dev("position", position, torch.int64)
+    dt = _act_dtype("rope_complex_and_cache", input_with_r)
+    f = _freqs_f32(freqs, rope_dim)
+    T = input_with_r.shape[0]
+    _req(input_with_r.numel() == T * n_local_heads * step_dim, "rope_complex_and_cache: input shape mismatch")
+    _req(position.numel() >= T, "rope_complex_and_cache: position too short")
+    if cache is not None:
+        _dev("cache", cache, input_with_r.dtype)
+        _dev("slot_mapping", slot_mapping, torch.int32)
+        _req(block_size > 0 and cache.numel() % (block_size * vdim) == 0, "rope_complex_and_cache: cache shape mismatch")
+        _req(slot_mapping.numel() >= T, "rope_complex_and_cache: slot_mapping too short")
+    else:
+        _dev("output", output, input_with_r.dtype)
+        _req(output.numel() == T * n_local_heads * out_step_dim, "rope_complex_and_cache: output shape mismatch")
+    _lib.check(rt._lib.xlite_hip_rope_complex_and_cache(
+        rt.stream(), T, n_local_heads, step_dim, rope_dim, offset, vdim, _ptr(input_with_r), _ptr(output), out_step_dim,
+        out_offset, _ptr(f), _ptr(position), block_size if cache is not None else 0, _ptr(cache), _ptr(slot_mapping), dt))
+    rt.finish()
+
+
+def layernorm(rt: Runtime, in_: torch.Tensor, norm: torch.Tensor, norm_bias: torch.Tensor, out: torch.Tensor,
+              norm_eps: float, norm_dim: int) -> None:
+    """LayerNorm over the first norm_dim columns of every row (xlite/csrc/_C.cpp:1122-1133)."""
+    for n, t in (("in_", in_), ("norm", norm), ("norm_bias", norm_bias), ("out", out)):
+        _dev(n, t)
+    dt = _act_dtype("layernorm", in_, norm, norm_bias, out)
+    _req(in_.dim() == 2 and out.dim() == 2 and in_.shape[0] == out.shape[0], "layernorm: [rows, columns] tensors expected")
+    _req(norm.numel() >= norm_dim and norm_bias.numel() >= norm_dim, "layernorm: weight / bias shorter than norm_dim")
+    _lib.check(rt._lib.xlite_hip_layernorm(rt.stream(), _ptr(in_), _ptr(norm), _ptr(norm_bias), _ptr(out), in_.shape[0],
+                                           in_.shape[1], out.shape[1], norm_dim, float(norm_eps), dt))
+    rt.finish()
+
+
+def muls(rt: Runtime, input: torch.Tensor, scale: float, output: torch.Tensor, calc_offset: int = 0,
+         calc_num: int = 0xFFFFFFFF) -> None:
+    """output = input * scale (xlite/csrc/_C.cpp:1660-1667); `calc_offset` / `calc_num` restrict it to a column
+    range of every row, the form the model runner calls (xlite/csrc/model.cpp:316)."""
+    _dev("input", input)
+    _dev("output", output)
+    dt = _act_dtype("muls", input, output)
+    _req(input.shape == output.shape, "muls: shape mismatch")
+    rows = input.shape[0] if input.dim() >= 2 else 1
+    row_len = input.numel() // max(rows, 1)
+    _lib.check(rt._lib.xlite_hip_muls(rt.stream(), _ptr(input), _ptr(output), rows, row_len, calc_offset,
+                                      min(calc_num, 0xFFFFFFFF), float(scale), dt))
+    rt.finish()
+
+
 def mla_prepare(rt: Runtime, attn_qkvc: torch.Tensor, q_norm: torch.Tensor, q_norm_bias: torch.Tensor,
                 attn_norm_qc: torch.Tensor, kv_norm: torch.Tensor, kv_norm_bias: torch.Tensor,
                 attn_norm_kvc: torch.Tensor, freqs: torch.Tensor, position: torch.Tensor, q_lora_rank: int,

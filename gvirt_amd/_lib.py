@@ -32,6 +32,9 @@ SIGNATURES = {
     "xlite_hip_indexer_scores": (_i32, [_vp] * 9 + [_u32] * 6 + [_i32]),
     "xlite_hip_indexer_topk_workspace_bytes": (_sz, [_u32] * 3),
     "xlite_hip_indexer_topk": (_i32, [_vp] * 10 + [_u32] * 7 + [_i32, _vp, _sz]),
+    "xlite_hip_layernorm": (_i32, [_vp] * 5 + [_u32] * 4 + [_f32, _i32]),
+    "xlite_hip_muls": (_i32, [_vp] * 3 + [_u32] * 4 + [_f32, _i32]),
+    "xlite_hip_rope_complex_and_cache": (_i32, [_vp] + [_u32] * 6 + [_vp, _vp, _u32, _u32, _vp, _vp, _u32, _vp, _vp, _i32]),
 }
 
 _lib = None

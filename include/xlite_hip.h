@@ -160,6 +160,46 @@ int xlite_hip_qk_rms_norm(void *stream, const void *in, void *out, const void *q
                           uint32_t k_start_offset, float norm_eps, int dtype);
 
 /* ------------------------------------------------------------------------
+ * layernorm — replaces XliteOpLayerNorm (xlite/csrc/op.cpp:607-628) as bound by
+ * `layernorm` (xlite/csrc/_C.cpp:1122-1133): LayerNorm with weight and bias over the
+ * first norm_dim columns of every row, fp32 arithmetic, biased variance, one rounding;
+ * rows of `in` are in_stride elements apart, rows of `out` out_stride (`out` may be `in`).
+ * In the MLA layer it normalises the index key (xlite/csrc/model.cpp:291-292).
+ * ---------------------------------------------------------------------- */
+int xlite_hip_layernorm(void *stream, const void *in, const void *norm, const void *norm_bias, void *out,
+                        uint32_t num_rows, uint32_t in_stride, uint32_t out_stride, uint32_t norm_dim,
+                        float norm_eps, int dtype);
+
+/* ------------------------------------------------------------------------
+ * muls — replaces XliteOpMuls (xlite/csrc/op.cpp:1644-1680), bound as `muls`
+ * (xlite/csrc/_C.cpp:1660-1667): output[r][calc_offset + i] = input[r][calc_offset + i] * scale
+ * for i < calc_num (clipped to the row), fp32 product rounded once; other columns are not
+ * written. The MLA layer scales the indexer's head weights with it (xlite/csrc/model.cpp:316).
+ * ---------------------------------------------------------------------- */
+int xlite_hip_muls(void *stream, const void *input, void *output, uint32_t num_rows, uint32_t row_len,
+                   uint32_t calc_offset, uint32_t calc_num, float scale, int dtype);
+
+/* ------------------------------------------------------------------------
+ * rope_complex_and_cache — the general form of the interleaved-pair rope kernel
+ * (xlite/csrc/kernels/rope_complex_and_cache.h:12-241) behind XliteOpRopeComplex
+ * (xlite/csrc/op.cpp:1106-1126) and XliteOpRopeComplexAndCache (:1128-1150).
+ * Of every head's step_dim columns the rope_dim columns from `offset` are rotated by
+ * freqs[position[t]] (fp32 cos, sin pairs) and leave de-interleaved [re... | im...].
+ *  cache == NULL: written to output[t][head * out_step_dim + out_offset ...]; `output`
+ *    may be `input` (the in-place call on the indexer's query, xlite/csrc/model.cpp:311-313);
+ *  cache != NULL (one head, block_size > 0): the vdim columns from `offset` - the rotated
+ *    ones, then the rest unchanged - go to cache[slot / block_size][slot % block_size]
+ *    ([num_blocks, block_size, vdim]) and nothing else is written (the index key cache,
+ *    xlite/csrc/model.cpp:295-297).
+ * xlite_hip_rope_complex is the case offset = step_dim - rope_dim, out_step_dim = rope_dim.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_rope_complex_and_cache(void *stream, uint32_t num_tokens, uint32_t n_local_heads,
+                                     uint32_t step_dim, uint32_t rope_dim, uint32_t offset, uint32_t vdim,
+                                     const void *input, void *output, uint32_t out_step_dim,
+                                     uint32_t out_offset, const float *freqs, const int64_t *position,
+                                     uint32_t block_size, void *cache, const int32_t *slot_mapping, int dtype);
+
+/* ------------------------------------------------------------------------
  * gather_sparse_kv_cache — replaces XliteOpGatherSparseKVCache
  * (xlite/csrc/op.cpp:1060-1084) + kernel gather_sparse_kv_cache.h:15-134.
  * dense[b, i] = paged[block_tables[b*max_num_blocks + tok / block_size], tok % block_size]

@@ -29,6 +29,10 @@ piece of the reference (paths under /root/reference/):
   rope_complex_ref     xlite/tests/kernels/rope_complex.py:31-41 with the fp32 operation order of
                        xlite/csrc/kernels/rope_complex_and_cache.h:165-205
   mla_prepare_ref      xlite/tests/kernels/mla_prepare.py:27-45,90-109
+  layernorm_ref        xlite/tests/kernels/layernorm.py:22-23; muls_ref xlite/tests/kernels/muls.py:23
+  rope_complex_and_cache_ref  xlite/csrc/kernels/rope_complex_and_cache.h:12-241 (any column offset; cache form)
+  indexer_forward_ref  xlite/csrc/model.cpp:285-330 (composition; golden of the whole indexer:
+                       xlite/tests/models/deepseek_v3.py:543-568)
   qk_rms_norm_ref      xlite/csrc/kernels/qk_rms_norm.h:32-54 over rmsnorm_ref
                        (xlite/tests/kernels/rmsnorm.py:24-30)
   einsum_ref           xlite/tests/kernels/einsum_mht_mhd.py:44
@@ -53,6 +57,10 @@ tests/test_oracle_pins.py):
   mha_forward_ref, mla_forward_ref: compositions of pinned pieces; mla_forward_ref additionally against the
       textbook model form (per-head keys and values from the whole token history, rope as a complex product,
       no paging, no absorption) over a prefill and two decode steps.
+  layernorm_ref: torch.nn.functional.layer_norm; a constant row normalises to the bias. muls_ref: exact
+      for power-of-two scales. rope_complex_and_cache_ref: equals rope_complex_ref on the last columns; complex
+      product in fp64; the cache form against a Python loop. indexer_forward_ref: the textbook indexer (fp32,
+      no cache, no paging; the golden's orthogonal rotate_activation cancels in q . k) selects the same sets.
   gather_*: brute-force Python loops.
   indexer_scores_ref: pure-Python triple loop in float (tiny case); one head with weight 1 reduces to
       q . k; with no intermediate rounding the weighted sum equals (sum_h w_h q_h) . k (linearity).
@@ -338,11 +346,15 @@ def mha_forward_ref(hidden, wqkv, wo, k_cache, v_cache, lens, cached_lens, block
 
 def mla_forward_ref(hidden, wqkv_a, q_norm, kv_norm, wq_b, wuk_t, wuv, wo, k_cache, pe_cache, lens, cached_lens,
                     block_tables, freqs, n_heads, q_lora_rank, kv_lora_rank, nope_head_dim, rope_head_dim, v_head_dim,
-                    block_size, scale, norm_eps=1e-6):
+                    block_size, scale, norm_eps=1e-6, indexer=None, index_k_cache=None, topk_override=None):
     """xlite/csrc/model.cpp:333-482 as a composition of the pieces above: metadata (prepare_attn_ref), QKV_A
     projection, mla_prepare (in place on the caches), Q_B projection, rope_complex, mla_v2 (absorb einsum,
     absorbed attention, W_UV einsum), output projection; every stage leaves its result in the activation
-    dtype, as the reference's tensors between operators do. `block_tables[i]` lists the blocks of sequence i."""
+    dtype, as the reference's tensors between operators do. `block_tables[i]` lists the blocks of sequence i.
+    `indexer`: dict with wk_weights_proj, k_norm, k_norm_bias, wq_b, index_n_heads, index_head_dim, index_topk -
+    the DSA branch (indexer_forward_ref) then masks the attention with its position lists; `index_k_cache` is
+    written in place. `topk_override` [T, index_topk] replaces the lists the branch selected (to check the
+    attention on lists chosen elsewhere). Returns the output, and with an indexer (output, lists or None)."""
     dt = hidden.dtype
     T = hidden.shape[0]
     meta = prepare_attn_ref(lens, cached_lens, block_tables, block_size)
@@ -353,15 +365,32 @@ def mla_forward_ref(hidden, wqkv_a, q_norm, kv_norm, wq_b, wuk_t, wuv, wo, k_cac
     norm_kvc = torch.empty(T, kv_lora_rank, dtype=dt)
     mla_prepare_ref(qkvc, q_norm, torch.zeros_like(q_norm), norm_qc, kv_norm, torch.zeros_like(kv_norm), norm_kvc, freqs,
                     pos, q_lora_rank, kv_lora_rank, rope_head_dim, block_size, k_cache, pe_cache, slots, norm_eps)
+    batch = len(lens)
+    qsl = torch.tensor(meta["query_start_loc"], dtype=torch.int32)
+    lens_t, clens_t = torch.tensor(list(lens), dtype=torch.int32), torch.tensor(list(cached_lens), dtype=torch.int32)
+    tables = torch.from_numpy(meta["block_tables"]).flatten()
+    topk_indices, top_k = None, 0
+    if indexer is not None:
+        res = indexer_forward_ref(hidden, norm_qc, indexer["wk_weights_proj"], indexer["k_norm"], indexer["k_norm_bias"],
+                                  indexer["wq_b"], index_k_cache, freqs, pos, slots, qsl, lens_t, clens_t, tables,
+                                  indexer["index_n_heads"], indexer["index_head_dim"], rope_head_dim, indexer["index_topk"],
+                                  block_size, batch, meta["max_num_blocks"], norm_eps)
+        if res is not None:
+            top_k = indexer["index_topk"]
+            topk_indices = torch.full((T, top_k), -1, dtype=torch.int32)
+            for i in range(batch):
+                for r, row in enumerate(res[1][i]):
+                    topk_indices[int(qsl[i]) + r, :len(row)] = torch.tensor(row, dtype=torch.int32)
+    own_lists = topk_indices
+    if topk_indices is not None and topk_override is not None:
+        topk_indices = topk_override
     q_with_qr = (norm_qc.float() @ wq_b.float()).to(dt)
     q_pe = rope_complex_ref(n_heads, nope_head_dim + rope_head_dim, rope_head_dim, q_with_qr, freqs, pos)
-    batch = len(lens)
-    attn = mla_v2_ref(q_with_qr, q_pe.reshape(T, -1), k_cache, pe_cache, wuk_t, wuv,
-                      torch.tensor(meta["query_start_loc"], dtype=torch.int32), torch.tensor(list(lens), dtype=torch.int32),
-                      torch.tensor(list(cached_lens), dtype=torch.int32), torch.from_numpy(meta["block_tables"]).flatten(),
+    attn = mla_v2_ref(q_with_qr, q_pe.reshape(T, -1), k_cache, pe_cache, wuk_t, wuv, qsl, lens_t, clens_t, tables,
                       n_heads, rope_head_dim, nope_head_dim, v_head_dim, kv_lora_rank, block_size, batch,
-                      meta["max_num_blocks"], scale)
-    return (attn.to(dt).float().reshape(T, -1) @ wo.float()).to(dt)
+                      meta["max_num_blocks"], scale, topk_indices, top_k)
+    out = (attn.to(dt).float().reshape(T, -1) @ wo.float()).to(dt)
+    return out if indexer is None else (out, own_lists)
 
 
 # --------------------------------------------------------------------------
@@ -460,6 +489,70 @@ def qk_rms_norm_ref(qkv, q_norm, q_norm_bias, k_norm, k_norm_bias, norm_eps, q_n
     ks = qkv[:, k_start_offset:k_end].reshape(T, k_cnt_per_token, k_norm_dim)
     out[:, k_start_offset:k_end] = rmsnorm_ref(ks, k_norm, zk, norm_eps).reshape(T, -1)
     return out
+
+
+def layernorm_ref(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, norm_dim: int) -> torch.Tensor:
+    """xlite/tests/kernels/layernorm.py:22-23 over the first norm_dim columns of every row (the launcher's
+    defaults, xlite/csrc/op.cpp:607-628): fp32, biased variance, one rounding. Returns those columns."""
+    xf = x[:, :norm_dim].float()
+    mean = xf.mean(-1, keepdim=True)
+    var = (xf - mean).pow(2).mean(-1, keepdim=True)
+    y = (xf - mean) * torch.rsqrt(var + eps) * weight[:norm_dim].float() + bias[:norm_dim].float()
+    return y.to(x.dtype)
+
+
+def muls_ref(x: torch.Tensor, scale: float, calc_offset: int = 0, calc_num: Optional[int] = None) -> torch.Tensor:
+    """xlite/tests/kernels/muls.py:23 restricted to a column range (xlite/csrc/op.cpp:1644-1680): a new tensor."""
+    out = x.clone()
+    end = x.shape[1] if calc_num is None else min(x.shape[1], calc_offset + calc_num)
+    out[:, calc_offset:end] = (x[:, calc_offset:end].float() * scale).to(x.dtype)
+    return out
+
+
+def rope_complex_and_cache_ref(n_local_heads, step_dim, rope_dim, offset, vdim, input_with_r, freqs, position,
+                               block_size=0, cache=None, slot_mapping=None):
+    """xlite/csrc/kernels/rope_complex_and_cache.h:12-241: the rope_dim columns from `offset` of every head,
+    rotated and de-interleaved. Without a cache: returns them [T, heads, rope_dim]. With a cache (one head):
+    writes the vdim columns from `offset` (rotated part, then the rest unchanged) to cache[slot], in place."""
+    T = input_with_r.shape[0]
+    dt = input_with_r.dtype
+    rows = input_with_r.view(T, n_local_heads, step_dim)
+    cos, sin = _freqs_as_cos_sin(freqs)
+    pos = position.view(-1).long()
+    y = _rope_interleaved(rows[..., offset:offset + rope_dim].float(), cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)).to(dt)
+    if cache is None:
+        return y
+    assert n_local_heads == 1
+    cv = cache.view(-1, block_size, vdim)
+    slots = slot_mapping.view(-1).long() & 0xFFFFFFFF
+    for t in range(T):
+        cv[slots[t] // block_size, slots[t] % block_size, :rope_dim] = y[t, 0]
+        cv[slots[t] // block_size, slots[t] % block_size, rope_dim:] = rows[t, 0, offset + rope_dim:offset + vdim]
+    return None
+
+
+def indexer_forward_ref(hidden, norm_qc, wk_weights_proj, k_norm, k_norm_bias, wq_b, index_k_cache, freqs, position,
+                        slot_mapping, query_start_loc, lens, cached_lens, block_tables, index_n_heads, index_head_dim,
+                        rope_head_dim, index_topk, block_size, batch, max_num_blocks, norm_eps):
+    """xlite/csrc/model.cpp:285-330 as a composition: index key projection, LayerNorm, rope into the index key
+    cache (in place), index query projection, rope, head weights times (heads * head_dim)^-0.5, scores, top-k.
+    Returns (score rows per sequence, position lists per sequence), or None when no sequence can exceed
+    index_topk."""
+    dt = hidden.dtype
+    T = hidden.shape[0]
+    kw = (hidden.float() @ wk_weights_proj.float()).to(dt)
+    kw[:, :index_head_dim] = layernorm_ref(kw, k_norm, k_norm_bias, norm_eps, index_head_dim)
+    rope_complex_and_cache_ref(1, index_head_dim + index_n_heads, rope_head_dim, 0, index_head_dim, kw, freqs, position,
+                               block_size, index_k_cache, slot_mapping)
+    if max_num_blocks * block_size <= index_topk:
+        return None
+    q = (norm_qc.float() @ wq_b.float()).to(dt).view(T, index_n_heads, index_head_dim).clone()
+    q[..., :rope_head_dim] = rope_complex_and_cache_ref(index_n_heads, index_head_dim, rope_head_dim, 0, 0,
+                                                         q.reshape(T, -1), freqs, position)
+    kw = muls_ref(kw, (index_n_heads * index_head_dim) ** -0.5, index_head_dim, index_n_heads)
+    scores = indexer_scores_ref(q.reshape(T, -1), index_k_cache, kw, query_start_loc, lens, cached_lens, block_tables,
+                                index_n_heads, index_head_dim, block_size, batch, max_num_blocks)
+    return scores, indexer_topk_ref(scores, index_topk)
 
 
 def mla_prepare_ref(attn_qkvc, q_norm, q_norm_bias, attn_norm_qc, kv_norm, kv_norm_bias,

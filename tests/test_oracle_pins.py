@@ -442,3 +442,90 @@ def test_mla_forward_equals_the_naive_model_form():
             assert torch.allclose(got[off:off + n], o[L - n:], atol=2e-4, rtol=2e-4), "step %d sequence %d" % (step, i)
             off += n
         cached = [c + l for c, l in zip(cached, lens)]
+
+
+def test_layernorm_muls_and_general_rope_pins():
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(5, 40, generator=g)
+    w, b = torch.randn(24, generator=g), torch.randn(24, generator=g)
+    # library routine on the normalised columns; a constant row normalises to the bias
+    want = torch.nn.functional.layer_norm(x[:, :24], (24,), w, b, 1e-6)
+    assert torch.allclose(O.layernorm_ref(x, w, b, 1e-6, 24), want, atol=1e-6, rtol=1e-5)
+    assert torch.allclose(O.layernorm_ref(torch.full((2, 30), 3.25), w, b, 1e-6, 24), b.expand(2, 24), atol=1e-5)
+    # muls: exact for a power of two, other columns untouched
+    xb = torch.randn(4, 16, generator=g).bfloat16()
+    y = O.muls_ref(xb, 0.5, 4, 8)
+    assert torch.equal(y[:, 4:12].float(), xb[:, 4:12].float() * 0.5) and torch.equal(y[:, :4], xb[:, :4]) and torch.equal(y[:, 12:], xb[:, 12:])
+    # the general rope: on the last columns it is rope_complex_ref; at offset 0 it is the complex product
+    T, H, step, rope = 6, 3, 20, 8
+    inp = torch.randn(T, H * step, generator=g).bfloat16()
+    ang = torch.randn(32, rope // 2, generator=g)
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    pos = torch.randint(0, 32, (T,), generator=g)
+    a = O.rope_complex_and_cache_ref(H, step, rope, step - rope, 0, inp, freqs, pos)
+    assert torch.equal(a, O.rope_complex_ref(H, step, rope, inp, freqs, pos))
+    z = torch.view_as_complex(inp.view(T, H, step)[..., :rope].double().reshape(T, H, rope // 2, 2)) * freqs[pos].to(torch.complex128).unsqueeze(1)
+    got = O.rope_complex_and_cache_ref(H, step, rope, 0, 0, inp, freqs, pos).double()
+    assert torch.allclose(got[..., :rope // 2], z.real, atol=2e-2, rtol=1e-2) and torch.allclose(got[..., rope // 2:], z.imag, atol=2e-2, rtol=1e-2)
+    # the cache form: rotated columns, then the rest of the vdim columns unchanged, at the slot; nothing else
+    bs, vdim = 4, 12
+    one = torch.randn(T, step, generator=g).bfloat16()
+    cache = torch.full((3, bs, vdim), 9.0).bfloat16()
+    slots = torch.tensor([5, 0, 11, 7, 2, 9], dtype=torch.int32)
+    O.rope_complex_and_cache_ref(1, step, rope, 2, vdim, one, freqs, pos, bs, cache, slots)
+    rot = O.rope_complex_and_cache_ref(1, step, rope, 2, 0, one, freqs, pos)
+    flat = cache.view(-1, vdim)
+    for t in range(T):
+        assert torch.equal(flat[slots[t], :rope], rot[t, 0]) and torch.equal(flat[slots[t], rope:], one[t, 2 + rope:2 + vdim])
+    untouched = [i for i in range(3 * bs) if i not in slots.tolist()]
+    assert bool((flat[untouched] == 9.0).all())
+
+
+def test_indexer_forward_selects_the_textbook_sets():
+    """The indexer composition (projection, LayerNorm, rope into the paged index cache, query projection, rope,
+    scaled head weights, scores, top-k) against the textbook form of xlite/tests/models/deepseek_v3.py:543-568
+    recomputed from the whole token history in float32 without cache or paging (its rotate_activation is an
+    orthogonal map applied to q and k alike and cancels in q . k; the kernel path ranks every position of the
+    sequence for every row, so the comparison runs on decode rows, where the golden has no mask either)."""
+    g = torch.Generator().manual_seed(43)
+    hid, ql, nH, D, rope, bs, topk = 12, 10, 4, 16, 8, 4, 6
+    r = lambda *s: torch.randn(*s, generator=g)
+    wkw, kn, kb, wqb = r(hid, D + nH) * 0.4, 1 + 0.1 * r(D), 0.1 * r(D), r(ql, nH * D) * 0.4
+    ang = torch.outer(torch.arange(64).float(), 1.0 / (50.0 ** (torch.arange(0, rope, 2).float() / rope)))
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    tables = [[4, 1, 7, 2], [0, 6, 3, 5]]
+    cache = torch.zeros(8, bs, D)
+    prompts = [9, 13]
+    hist_x = [torch.zeros(0, hid), torch.zeros(0, hid)]
+    cached = [0, 0]
+
+    def crope(x, pos):
+        xc = torch.view_as_complex(x.reshape(*x.shape[:-1], -1, 2).contiguous()) * freqs[pos].reshape(len(pos), *([1] * (x.dim() - 2)), -1)
+        return torch.view_as_real(xc).flatten(-2)
+
+    for step in range(3):
+        lens = prompts if step == 0 else [1, 1]
+        hidden, qc = r(sum(lens), hid), r(sum(lens), ql)
+        meta = O.prepare_attn_ref(lens, cached, tables, bs)
+        res = O.indexer_forward_ref(hidden, qc, wkw, kn, kb, wqb, cache, freqs, torch.tensor(meta["position"]),
+                                    torch.tensor(meta["slot_mapping"], dtype=torch.int32),
+                                    torch.tensor(meta["query_start_loc"], dtype=torch.int32), torch.tensor(lens, dtype=torch.int32),
+                                    torch.tensor(cached, dtype=torch.int32), torch.from_numpy(meta["block_tables"]).flatten(), nH, D,
+                                    rope, topk, bs, 2, meta["max_num_blocks"], 1e-6)
+        off = 0
+        for i, n in enumerate(lens):
+            hist_x[i] = torch.cat([hist_x[i], hidden[off:off + n]])
+            if step > 0:
+                L = hist_x[i].shape[0]
+                kwf = hist_x[i] @ wkw
+                k = torch.nn.functional.layer_norm(kwf[:, :D], (D,), kn, kb, 1e-6)
+                k = torch.cat([crope(k[:, :rope], torch.arange(L)), k[:, rope:]], -1)
+                q = (qc[off:off + 1] @ wqb).view(1, nH, D)
+                q = torch.cat([crope(q[..., :rope], torch.tensor([L - 1])), q[..., rope:]], -1)
+                weights = kwf[L - 1:, D:] * nH ** -0.5
+                index_score = torch.einsum("sht,sh->st", torch.einsum("shd,td->sht", q, k) * D ** -0.5, weights)
+                want = sorted(index_score[0].topk(min(topk, L))[1].tolist())
+                assert res[1][i][0] == want, "step %d sequence %d" % (step, i)
+                assert torch.allclose(res[0][i][0], index_score[0], atol=1e-4, rtol=1e-4)
+            off += n
+        cached = [c + l for c, l in zip(cached, lens)]
