@@ -25,7 +25,8 @@ namespace {
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 constexpr int kWavesPerWg = 4;
 constexpr int kRange = 256;          // positions per wave
-constexpr int kSelThreads = 256;
+constexpr int kSelThreads = 1024;
+constexpr uint32_t kSelStage = 24576;   // scores of a row kept in LDS between the passes (48 KiB)
 
 template <typename T>
 struct Mma;
@@ -198,7 +199,8 @@ __device__ __forceinline__ uint32_t order_key(uint16_t bits)
     return (bits & 0x8000u) ? (~static_cast<uint32_t>(bits) & 0xffffu) : (static_cast<uint32_t>(bits) | 0x8000u);
 }
 
-// One workgroup per query row.
+// One workgroup per query row. The row is read from memory once: its first kSelStage scores stay in LDS for
+// the three passes (a longer row's remainder is re-read).
 __global__ void __launch_bounds__(kSelThreads)
 indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__restrict__ indices,
                       int32_t *__restrict__ topk_indices, const int32_t *__restrict__ query_start_loc,
@@ -207,6 +209,7 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
 {
     __shared__ uint32_t hist[256];
     __shared__ uint32_t wave_cnt[2][kSelThreads / 64];
+    __shared__ __attribute__((aligned(16))) uint16_t staged[kSelStage];
     __shared__ uint32_t sel[4];
     const uint32_t t = blockIdx.x;
     uint32_t seq = 0, n = 0;
@@ -223,9 +226,16 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
     }
     // ---- the k-th largest key: high byte, then low byte. Threads read eight keys (16 bytes) at a time.
     const uint32_t n8 = ld_scores % 8 == 0 ? n & ~7u : 0u;   // vector loads need 16-byte aligned rows
+    const uint32_t n_st = min(n8, kSelStage);                // scores [0, n_st) are served from LDS
+    for (uint32_t j = threadIdx.x * 8; j < n_st; j += kSelThreads * 8) {
+        *reinterpret_cast<uint4 *>(staged + j) = *reinterpret_cast<const uint4 *>(row + j);
+    }
+    // (the first pass's barrier orders these stores before any read)
     uint32_t prefix = 0, above = 0;   // keys whose high byte equals `prefix` are the candidates of pass 2
     for (int pass = 0; pass < 2; pass++) {
-        hist[threadIdx.x] = 0;
+        if (threadIdx.x < 256) {
+            hist[threadIdx.x] = 0;
+        }
         __syncthreads();
         auto count = [&](uint32_t key) {
             if (pass == 0) {
@@ -235,7 +245,7 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
             }
         };
         for (uint32_t j = threadIdx.x * 8; j < n8; j += kSelThreads * 8) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(row + j);
+            const uint4 v = j < n_st ? *reinterpret_cast<const uint4 *>(staged + j) : *reinterpret_cast<const uint4 *>(row + j);
             const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -282,7 +292,7 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
         const uint32_t j0 = base + threadIdx.x * 4;
         uint32_t key[4];
         if (j0 + 4 <= n8) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(row + j0);
+            const uint2 v = j0 < n_st ? *reinterpret_cast<const uint2 *>(staged + j0) : *reinterpret_cast<const uint2 *>(row + j0);
             key[0] = order_key(static_cast<uint16_t>(v.x & 0xffffu));
             key[1] = order_key(static_cast<uint16_t>(v.x >> 16));
             key[2] = order_key(static_cast<uint16_t>(v.y & 0xffffu));
