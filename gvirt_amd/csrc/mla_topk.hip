@@ -16,6 +16,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kMaxTopk = 2048;
 constexpr int kItems = kMaxTopk / kThreads;
+constexpr uint32_t kRun = 128;   // dense positions copied by one workgroup
 
 __global__ void __launch_bounds__(kThreads)
 topk_gather_kernel(const uint4 *__restrict__ k_cache, const uint4 *__restrict__ pe_cache,
@@ -100,7 +101,10 @@ topk_gather_kernel(const uint4 *__restrict__ k_cache, const uint4 *__restrict__ 
     // the dense rows: one 16-lane group per position
     const uint32_t group = threadIdx.x / 16, lane = threadIdx.x % 16;
     const int32_t *table = block_tables + static_cast<uint64_t>(seq) * max_num_blocks;
-    for (uint32_t i = group; i < count; i += kThreads / 16) {
+    // the row's dense positions are dealt to gridDim.y workgroups in runs of kRun (every one of them has
+    // compacted the list; a single workgroup per row copied 2.4 MB alone)
+    const uint32_t run0 = blockIdx.y * kRun;
+    for (uint32_t i = run0 + group; i < min(count, run0 + kRun); i += kThreads / 16) {
         const uint32_t tok = sel[i];
         const uint32_t phys = static_cast<uint32_t>(table[tok / block_size]);
         const uint64_t src = static_cast<uint64_t>(phys) * block_size + tok % block_size;
@@ -113,6 +117,9 @@ topk_gather_kernel(const uint4 *__restrict__ k_cache, const uint4 *__restrict__ 
         }
     }
     // the row as a dense "sequence" of one query: [query_start_loc | lens | cached_lens]
+    if (blockIdx.y != 0) {
+        return;
+    }
     if (threadIdx.x == 0) {
         meta[t] = static_cast<int32_t>(t);
         meta[total_tokens + t] = count > 0 ? 1 : 0;
@@ -154,7 +161,7 @@ int launch_mla_topk(hipStream_t stream, const MlaArgs &a)
     char *k_dense = ws + align256(3 * static_cast<size_t>(a.total_tokens) * sizeof(int32_t));
     char *pe_dense = k_dense + align256(static_cast<size_t>(a.total_tokens) * a.top_k * a.kv_lora_rank * 2);
 
-    topk_gather_kernel<<<a.total_tokens, kThreads, 0, stream>>>(
+    topk_gather_kernel<<<dim3(a.total_tokens, ceil_div(a.top_k, kRun), 1), kThreads, 0, stream>>>(
         static_cast<const uint4 *>(a.k_cache), static_cast<const uint4 *>(a.pe_cache), a.block_tables, a.topk_indices,
         a.query_start_loc, a.lens, a.cached_lens, reinterpret_cast<uint4 *>(k_dense), reinterpret_cast<uint4 *>(pe_dense),
         meta, static_cast<uint16_t *>(a.o_absorb), a.total_tokens, a.batch, a.top_k, a.block_size, a.max_num_blocks,
