@@ -110,6 +110,20 @@ extern "C" size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t 
                                                 uint32_t max_num_blocks, uint32_t top_k)
 {
     if (top_k > 0) {
+        MlaArgs a{};
+        a.total_tokens = total_tokens;
+        a.batch = batch;
+        a.n_heads = n_heads;
+        a.kv_lora_rank = kv_lora_rank;
+        a.rope_head_dim = rope_head_dim;
+        a.block_size = block_size;
+        a.max_num_blocks = max_num_blocks;
+        a.top_k = top_k;
+        static const int32_t dummy = 0;
+        a.block_tables = &dummy;
+        if (mla_decode_supported(a)) {
+            return mla_decode_workspace_bytes(a);   // the decode kernel reads the listed rows itself
+        }
         // the gathered per-row caches, then the dense attention over them (every row a sequence)
         return mla_topk_scratch_bytes(total_tokens, kv_lora_rank, rope_head_dim, top_k) +
                xlite_hip_mla_workspace_bytes(total_tokens, n_heads, kv_lora_rank, rope_head_dim, 1, total_tokens, top_k, 0);
@@ -162,11 +176,11 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
     MlaArgs a{q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks,
               0, scale, topk_indices, top_k, dtype, workspace, workspace_bytes};
-    if (top_k > 0) {
-        return launch_mla_topk(as_stream(stream), a);
-    }
     if (mla_decode_supported(a)) {
-        return launch_mla_decode(as_stream(stream), a);
+        return launch_mla_decode(as_stream(stream), a);   // with or without position lists
+    }
+    if (top_k > 0) {
+        return launch_mla_topk(as_stream(stream), a);      // other shapes: gather the listed rows, then dense
     }
     return launch_mfma_mla(as_stream(stream), a);
 }

@@ -106,6 +106,8 @@ struct MlaDecodeParams {
     uint32_t dense_len;
     uint32_t chunk_min_steps;
     float scale_log2e;
+    const int32_t *topk_indices;   // [total_rows][top_k] position lists (top_k == 0: none)
+    uint32_t top_k;
 };
 bool mla_decode_supported(const MlaArgs &a);
 size_t mla_decode_workspace_bytes(const MlaArgs &a);

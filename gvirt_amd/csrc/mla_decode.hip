@@ -75,17 +75,27 @@ __device__ __forceinline__ void dma_4x1k(uint32_t lds_addr, uint32_t v0, uint32_
                  "global_load_lds_dwordx4 %4, %5 offset:3072\n\t"
                  :: "s"(lds_addr), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(base) : "memory", "m0");
 }
+// the same copy with a 64-bit address per lane (rows gathered from anywhere in a cache of any size)
+__device__ __forceinline__ void dma_1k_ptr(uint32_t lds_addr, const void *lane_ptr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\t"
+                 :: "s"(lds_addr), "v"(lane_ptr) : "memory", "m0");
+}
 template <int N>
 __device__ __forceinline__ void dma_wait()
 {
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
+// LISTS: rows may come with position lists (p.top_k != 0); a separate instantiation, so that the plain kernel
+// keeps its register allocation.
+template <bool LISTS>
 __global__ void __launch_bounds__(kNT)
 mla_decode_kernel(const MlaDecodeParams p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE_BYTES);
+    uint32_t *mask_lds = tbl_lds + kTblCap;   // kTblCap / kStep + 2 words: valid positions of a listed row's steps
     const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
         static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
 
@@ -123,15 +133,41 @@ mla_decode_kernel(const MlaDecodeParams p)
     // ---- one (sequence, query row, range of steps) at a time
     // `n_slots`: segments the row is cut into; `pslot`: where this segment's partial goes when there are several;
     // `meta`: what the merge needs to find the row's partials (written with the row's first segment).
-    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t limit, uint32_t step_a, uint32_t step_b, uint32_t n_slots,
-                           uint32_t pslot, int4 meta) {
+    // `limit`: the row's length in positions - its causal range, or top_k entries of its position list when
+    // the range (`causal`) is longer than that (`listed`): then position j of the row is list entry j.
+    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t limit, uint32_t causal, uint32_t step_a, uint32_t step_b,
+                           uint32_t n_slots, uint32_t pslot, int4 meta) {
         const int32_t *table = dense ? nullptr : p.block_tables + static_cast<uint64_t>(seq) * p.max_num_blocks;
         const uint32_t t0 = step_a * kStep;
         const uint32_t t1 = min(limit, step_b * kStep);
         const uint32_t n_steps = step_b - step_a;
         const bool single = n_slots == 1;
-        const uint32_t blk0 = dense ? 0 : t0 / p.block_size;
-        if (!dense) {
+        const bool listed = LISTS && causal > p.top_k;
+        const uint32_t blk0 = dense || listed ? 0 : t0 / p.block_size;
+        if (listed) {
+            // cache row of every list entry of the segment (tbl_lds[i] for entry t0 + i) and, per step, the mask
+            // of its usable entries: inside the causal range, not a repeat of its predecessor. The others point
+            // at the row of position 0 and get probability zero.
+            const int32_t *list = p.topk_indices + static_cast<uint64_t>(tok) * p.top_k;
+            for (uint32_t base = 0; base < n_steps * kStep; base += kNT) {
+                const uint32_t i = base + threadIdx.x, j = t0 + i;
+                int32_t x = -1;
+                bool ok = false;
+                if (i < n_steps * kStep && j < t1) {
+                    x = list[j];
+                    ok = x >= 0 && static_cast<uint32_t>(x) < causal && (j == 0 || list[j - 1] != x);
+                }
+                const uint32_t pos = ok ? static_cast<uint32_t>(x) : 0u;
+                if (i < n_steps * kStep) {
+                    tbl_lds[i] = static_cast<uint32_t>(table[pos / p.block_size]) * p.block_size + pos % p.block_size;
+                }
+                const uint64_t m = __ballot(ok);
+                if (lane == 0 && base + wave * 64 < n_steps * kStep + 32) {
+                    mask_lds[(base >> 5) + 2 * wave] = static_cast<uint32_t>(m);
+                    mask_lds[(base >> 5) + 2 * wave + 1] = static_cast<uint32_t>(m >> 32);
+                }
+            }
+        } else if (!dense) {
             // block-table entries of the tile (lookups in the loop then cost an LDS read only)
             const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
             for (uint32_t i = threadIdx.x; i < nblk; i += kNT) {
@@ -203,8 +239,24 @@ mla_decode_kernel(const MlaDecodeParams p)
                 return c;
             };
             auto issue = [&](uint32_t step) {
-                const StepCopy c = plan(step);
                 const uint32_t r0 = 4 * wave;
+                if (listed) {
+                    const uint32_t stage = smem_addr + (step % kStages) * STAGE_BYTES;
+                    const uint32_t e0 = step * kStep;
+#pragma unroll
+                    for (uint32_t i = 0; i < 4; i++) {
+                        const uint64_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[e0 + r0 + i]);
+                        dma_1k(stage + (r0 + i) * KC_ROWB, kc_voff ^ (i << 5),
+                               reinterpret_cast<const char *>(p.k_cache) + phys * KC_ROWB);
+                    }
+                    if (wave < PE_WAVES) {
+                        const uint64_t phys = tbl_lds[e0 + pe_row];   // per lane: eight rotary rows per copy
+                        dma_1k_ptr(stage + KC_BYTES + wave * 1024,
+                                   reinterpret_cast<const char *>(p.pe_cache) + phys * PE_ROWB + pe_voff);
+                    }
+                    return;
+                }
+                const StepCopy c = plan(step);
                 if (c.last_pos == kStep - 1) {
                     dma_4x1k(c.stage + r0 * KC_ROWB, kc_voff, kc_voff ^ (1u << 5), kc_voff ^ (2u << 5),
                              kc_voff ^ (3u << 5), c.kb + r0 * KC_ROWB);
@@ -278,7 +330,18 @@ mla_decode_kernel(const MlaDecodeParams p)
                         S[mt][k] *= p.scale_log2e;
                     }
                 }
-                if (t + kStep > t1) {   // uniform: only a tile's last step has positions to mask
+                if (listed) {
+                    const uint32_t valid = __builtin_amdgcn_readfirstlane(mask_lds[step]) >> gi4;
+                    if (__builtin_amdgcn_readfirstlane(mask_lds[step]) != 0xffffffffu) {
+#pragma unroll
+                        for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+                            for (int k = 0; k < 4; k++) {
+                                S[mt][k] = ((valid >> (mt * 16 + k)) & 1u) ? S[mt][k] : -INFINITY;
+                            }
+                        }
+                    }
+                } else if (t + kStep > t1) {   // uniform: only a tile's last step has positions to mask
 #pragma unroll
                     for (int mt = 0; mt < 2; mt++) {
 #pragma unroll
@@ -464,13 +527,18 @@ mla_decode_kernel(const MlaDecodeParams p)
         }
         return seq < B && static_cast<int32_t>(t) >= p.query_start_loc[seq] ? seq : B;
     };
-    auto row_limit = [&](uint32_t t, uint32_t seq) -> uint32_t {
+    auto row_causal = [&](uint32_t t, uint32_t seq) -> uint32_t {
         if (seq >= B) {
             return 0;   // a row outside every sequence
         }
         const uint32_t clen = static_cast<uint32_t>(p.cached_lens[seq]);
         return dense ? min(clen + static_cast<uint32_t>(p.lens[seq]), p.dense_len)
                      : clen + (t - static_cast<uint32_t>(p.query_start_loc[seq])) + 1;
+    };
+    // positions the row walks: its causal range, or its list of top_k entries when the range is longer
+    auto row_limit = [&](uint32_t t, uint32_t seq) -> uint32_t {
+        const uint32_t causal = row_causal(t, seq);
+        return LISTS && causal > p.top_k ? p.top_k : causal;
     };
     for (uint32_t c = blockIdx.x;; c += gridDim.x) {
         // block-wide prefix sums of the rows' step counts (redone for every chunk: nothing of it stays in
@@ -512,6 +580,9 @@ mla_decode_kernel(const MlaDecodeParams p)
         total = __builtin_amdgcn_readfirstlane(total);
         uint32_t chunk = max(ceil_div(total, gridDim.x), p.chunk_min_steps);
         chunk = min(chunk, (kTblCap - 2) * p.block_size / kStep);
+        if (LISTS) {
+            chunk = min(chunk, static_cast<uint32_t>(kTblCap / kStep));   // a listed row stages one entry per position
+        }
         if (c >= ceil_div(total, chunk)) {
             return;
         }
@@ -549,7 +620,7 @@ mla_decode_kernel(const MlaDecodeParams p)
                 // written with the row's first segment (a == 0): then c0 == c
                 const int4 meta = make_int4(n_slots > 1 ? static_cast<int>(n_slots) : 0, static_cast<int>(c),
                                             first_seg ? 1 : 0, 0);
-                run_segment(seq, row, limit, a, b, n_slots, 2 * c + (first_seg ? 0 : 1), meta);
+                run_segment(seq, row, limit, row_causal(row, seq), a, b, n_slots, 2 * c + (first_seg ? 0 : 1), meta);
                 remaining -= b - a;
                 first_seg = false;
             }
@@ -572,7 +643,9 @@ mla_decode_kernel(const MlaDecodeParams p)
 bool mla_decode_supported(const MlaArgs &a)
 {
     const bool dense = a.block_tables == nullptr;
-    return a.kv_lora_rank == C && a.rope_head_dim == R && a.top_k == 0 && (dense || a.block_size % kStep == 0);
+    // position lists (top_k) go with the paged cache only
+    return a.kv_lora_rank == C && a.rope_head_dim == R && (dense ? a.top_k == 0 : a.block_size % kStep == 0) &&
+           a.top_k <= 2048;
 }
 
 namespace {
@@ -604,8 +677,13 @@ int mla_decode_plan(const MlaArgs &a, MlaPlan *pl)
     tok = tok > 512 ? 512 : (tok < 256 ? 256 : tok);
     pl->chunk_min_steps = static_cast<uint32_t>(tok / kStep);
     pl->n_workgroups = static_cast<uint32_t>(n_cu);
-    const uint64_t max_steps = (max_ctx + kStep - 1) / kStep;
-    const uint64_t chunk_cap = static_cast<uint64_t>(kTblCap - 2) * (dense ? kStep : a.block_size) / kStep;
+    // with position lists no row walks more than top_k positions, and a chunk stages one entry per position
+    const uint64_t max_len = a.top_k != 0 && a.top_k < max_ctx ? a.top_k : max_ctx;
+    const uint64_t max_steps = (max_len + kStep - 1) / kStep;
+    uint64_t chunk_cap = static_cast<uint64_t>(kTblCap - 2) * (dense ? kStep : a.block_size) / kStep;
+    if (a.top_k != 0 && chunk_cap > kTblCap / kStep) {
+        chunk_cap = kTblCap / kStep;
+    }
     const uint64_t by_cap = (static_cast<uint64_t>(a.total_tokens) * max_steps + chunk_cap - 1) / chunk_cap;
     pl->max_chunks = static_cast<uint32_t>(by_cap > pl->n_workgroups ? by_cap : pl->n_workgroups);
     pl->meta_bytes = ((static_cast<size_t>(a.total_tokens) * sizeof(int4) + 255) / 256) * 256;
@@ -658,13 +736,22 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
     p.dense_len = a.dense_len;
     p.chunk_min_steps = pl.chunk_min_steps;
     p.scale_log2e = a.scale * kLog2e;
+    p.topk_indices = a.topk_indices;
+    p.top_k = a.top_k;
+    XL_REQUIRE(a.top_k == 0 || a.topk_indices != nullptr, "top_k > 0 needs topk_indices");
 
-    const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + kTblCap * sizeof(uint32_t);
+    const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + (kTblCap + kTblCap / kStep + 2) * sizeof(uint32_t);
     // the kernel also has a few words of static LDS: ask for exactly the dynamic part
-    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(mla_decode_kernel), lds)) {
+    const bool lists = a.top_k != 0;
+    if (const int rc = ensure_dynamic_lds(lists ? reinterpret_cast<const void *>(mla_decode_kernel<true>)
+                                                : reinterpret_cast<const void *>(mla_decode_kernel<false>), lds)) {
         return rc;
     }
-    mla_decode_kernel<<<dim3(pl.n_workgroups, 1, 1), kNT, lds, stream>>>(p);
+    if (lists) {
+        mla_decode_kernel<true><<<dim3(pl.n_workgroups, 1, 1), kNT, lds, stream>>>(p);
+    } else {
+        mla_decode_kernel<false><<<dim3(pl.n_workgroups, 1, 1), kNT, lds, stream>>>(p);
+    }
     XL_LAUNCH_CHECK();
     // rows that ended up in a single segment were stored directly
     return launch_merge_mla(stream, a.dtype, a.o_absorb, reinterpret_cast<const uint16_t *>(p.part_acc), p.part_ml,

@@ -182,6 +182,39 @@ def test_mla_topk_index_mask(rt, nH, work, top_k):
     check(out.float().cpu(), ref)
 
 
+@pytest.mark.parametrize("top_k", [96, 512])
+def test_mla_topk_lists_with_entries_to_ignore(rt, top_k):
+    """Lists as an indexer that ranks the whole sequence leaves them for prefill rows: ascending, with positions
+    beyond the row's causal range; plus repeats and negative entries. Only the usable entries count, once each
+    (xlite/csrc/kernels/mla_v2.h:697-699; the mask of xlite/tests/kernels/mla.py:293-333 is a set)."""
+    from gvirt_amd._C import mla_attention
+    lens, clens = [7, 1, 3], [700, 1500, 64]
+    c = mla_case(43, lens, clens, 16, bs=64)
+    g = torch.Generator().manual_seed(44)
+    rows = []
+    for l, cl in zip(lens, clens):
+        for r in range(l):
+            total = cl + l                                   # the indexer sees the whole sequence
+            pick = torch.randperm(total, generator=g)[:top_k] if total >= top_k else torch.arange(total)
+            pick = torch.sort(pick).values
+            if pick.numel() < top_k:
+                pick = torch.cat([pick, pick[-1:].expand(top_k - pick.numel())])
+            pick = pick.clone()
+            pick[5] = pick[4]                                # a repeat
+            pick[0] = -1                                     # an unset entry
+            rows.append(pick)
+    topk = torch.stack(rows).int()
+    scale = 192 ** -0.5
+    out = torch.zeros(c["T"], c["nH"], c["C"], dtype=torch.bfloat16, device=DEV)
+    mla_attention(rt, c["qa"].to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), out, c["qsl"].to(DEV),
+                  c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), c["nH"], c["R"], c["C"], c["bs"], c["batch"],
+                  c["maxblk"], scale, topk.to(DEV), top_k)
+    rt.synchronize()
+    ref = O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"],
+                              c["R"], c["C"], c["bs"], c["batch"], c["maxblk"], scale, topk, top_k)
+    check(out.float().cpu(), ref)
+
+
 def test_mla_decode_large_batch_of_short_sequences(rt):
     """More rows than threads in the work-splitting scan (two rows per thread), chunks that span many rows,
     and rows far shorter than a step."""
