@@ -110,9 +110,10 @@ int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, cons
  * scores = (q_absorb . k + qr . pe) * scale, causal as in attention.
  * topk_indices [total_tokens, top_k] int32 (top_k == 0: dense, pointer unused):
  * when top_k > 0 a row whose causal range is longer than top_k attends only to the
- * listed positions (ascending, inside the range); shorter rows see their whole range
- * (xlite/csrc/kernels/mla_v2.h:697-699). The listed rows are gathered into the workspace
- * first, so the workspace size depends on top_k. bf16 only (xlite/csrc/op.cpp:1014).
+ * listed positions (ascending; entries outside the range, negative ones and repeats of
+ * the predecessor are ignored); shorter rows see their whole range
+ * (xlite/csrc/kernels/mla_v2.h:697-699). The workspace size depends on top_k: pass the
+ * call's value to xlite_hip_mla_workspace_bytes. bf16 only (xlite/csrc/op.cpp:1014).
  * workspace: at least xlite_hip_mla_workspace_bytes() for the same shape (required:
  * XLITE_HIP_ENOSPC otherwise; split-KV partials, no initialisation needed).
  * ---------------------------------------------------------------------- */
