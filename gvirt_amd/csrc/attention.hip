@@ -176,6 +176,9 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
     MlaArgs a{q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks,
               0, scale, topk_indices, top_k, dtype, workspace, workspace_bytes};
+    if (kv_lora_rank != 512 || rope_head_dim != 64) {
+        return launch_mla_generic(as_stream(stream), a);  // sizes the matrix-core kernels are not built for
+    }
     if (mla_decode_supported(a)) {
         return launch_mla_decode(as_stream(stream), a);   // with or without position lists
     }
@@ -206,6 +209,9 @@ extern "C" int xlite_hip_mla_v3(void *stream, const void *q_absorb, const void *
     MlaArgs a{q_absorb, qr, k_dense, pe_dense, o_absorb, query_start_loc, lens, cached_lens, nullptr,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, 1, batch, index_topk,
               index_topk, scale, nullptr, 0, dtype, workspace, workspace_bytes};
+    if (kv_lora_rank != 512 || rope_head_dim != 64) {
+        return launch_mla_generic(as_stream(stream), a);
+    }
     if (mla_decode_supported(a)) {
         return launch_mla_decode(as_stream(stream), a);
     }

@@ -130,5 +130,7 @@ uint32_t mfma_pick_splits(uint32_t total_tokens, uint32_t rows_per_token, uint32
                           uint32_t parallel_heads, uint32_t max_ctx, uint32_t tile);
 int launch_mfma_gqa(hipStream_t stream, const AttentionArgs &a);
 int launch_mfma_mla(hipStream_t stream, const MlaArgs &a);
+// mla_generic.hip: any latent / rotary size, no matrix instructions
+int launch_mla_generic(hipStream_t stream, const MlaArgs &a);
 
 }  // namespace xlite

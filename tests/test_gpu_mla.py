@@ -60,6 +60,27 @@ def test_mla_attention_grid(rt, nH, work):
     check(run_mla(rt, c, scale), oracle_mla(c, scale))
 
 
+@pytest.mark.parametrize("nH,C,R", [(1, 16, 64), (3, 96, 32), (2, 40, 8)])
+@pytest.mark.parametrize("work", MLA_WORK)
+def test_mla_attention_other_latent_sizes(rt, nH, C, R, work):
+    """The reference's smallest test model (1 head, kv_lora_rank 16: xlite/tests/kernels/mla.py:54) and other
+    sizes the matrix-core kernels are not built for, through the plain vector kernel; with position lists too."""
+    clens, lens = work
+    c = mla_case(35, lens, clens, nH, bs=16, C=C, R=R)
+    scale = (C // 4 + R) ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
+    if max(cl + l for cl, l in zip(clens, lens)) > 64:
+        from gvirt_amd._C import mla_attention
+        topk = _topk_indices(c, 48, 7)
+        out = torch.zeros(c["T"], nH, C, dtype=torch.bfloat16, device=DEV)
+        mla_attention(rt, c["qa"].to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), out, c["qsl"].to(DEV),
+                      c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), nH, R, C, c["bs"], c["batch"], c["maxblk"],
+                      scale, topk.to(DEV), 48)
+        rt.synchronize()
+        check(out.float().cpu(), O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"],
+                                                     c["tables"], nH, R, C, c["bs"], c["batch"], c["maxblk"], scale, topk, 48))
+
+
 def test_config4_deepseek_r1_decode_sampled(rt):
     """Configuration 4 shape (128 heads, block 64) with 4 of the 32 sequences at full context."""
     ctx = W.c4_context_lengths()[:4]
