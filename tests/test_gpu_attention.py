@@ -249,3 +249,34 @@ def test_config3_qwen25_7b_chunked_prefill_sampled(rt):
         got = run_attention(rt, w)
         ref = oracle_attention(w)
         check(got, ref)
+
+
+@pytest.mark.parametrize("model", [(8, 1, 128, torch.bfloat16), (14, 2, 64, torch.bfloat16), (4, 1, 128, torch.float16)])
+def test_decode_at_the_longest_reference_contexts(rt, model):
+    """The two-sequence decode workloads of xlite/tests/kernels/attention.py:50-57 at their full lengths
+    (60000 and 131071 cached positions), against the oracle."""
+    nH, nKV, d, dtype = model
+    w = generic_case(17, [1, 1], [131071, 60000], nH, nKV, d, 128, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
+@pytest.mark.parametrize("model", [(8, 1, 128, torch.bfloat16), (14, 2, 64, torch.bfloat16)])
+def test_prefill_at_the_longest_reference_length_sampled_rows(rt, model):
+    """The 32769-token prefill of xlite/tests/kernels/attention.py:46 at full length. The oracle takes sampled
+    rows, each as the decode step it is equivalent to (row r of a prefill from an empty cache sees the r keys
+    before it and its own)."""
+    nH, nKV, d, dtype = model
+    n = 32769
+    w = generic_case(18, [n], [0], nH, nKV, d, 128, dtype, rms=True)
+    got = run_attention(rt, w)
+    # the prefill wrote nothing into the cache, which already holds the chunk's keys at positions 0 .. n-1 (the
+    # operator reads keys from the cache only): a decode workload over the same cache sees what row r saw
+    for r in (0, 1, 127, 128, 4099, 20000, n - 1):
+        one = dict(w)
+        one["qkv"] = w["qkv"][r:r + 1].contiguous()
+        one["batch"] = 1
+        one["lens"] = torch.tensor([1], dtype=torch.int32)
+        one["cached_lens"] = torch.tensor([r], dtype=torch.int32)
+        one["query_start_loc"] = torch.tensor([0], dtype=torch.int32)
+        one["output"] = torch.zeros(1, nH * d, dtype=dtype)
+        check(got[r:r + 1], oracle_attention(one))

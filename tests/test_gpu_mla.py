@@ -297,3 +297,10 @@ def test_mla_prefill_128_heads_rows_of_several_sequences(rt):
     c = mla_case(61, [300, 0, 77, 1], [700, 50, 0, 2000], 128, bs=64)
     scale = 192 ** -0.5
     check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
+def test_mla_decode_at_the_longest_reference_context(rt):
+    """xlite/tests/kernels/mla.py:72: two sequences of 131071 cached positions, one new token each."""
+    c = mla_case(36, [1, 1], [131071, 131071], 16)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
