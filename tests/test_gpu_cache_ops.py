@@ -61,9 +61,10 @@ def test_rope_and_cache_mrope_and_empty(rt):
     assert torch.equal(_bits(dev[1]), _bits(kc))
 
 
-@pytest.mark.parametrize("cached,topk", [([127], 512), ([2047, 8191, 45841], 2048), ([2047] * 4, 512), ([16384], 2048)])
+@pytest.mark.parametrize("cached,topk", [([127], 512), ([2047, 8191, 45841], 2048), ([2047] * 4, 512), ([16384], 2048),
+                                         ([131071], 2048), ([32751] * 3, 512), ([4096], 512)])
 def test_gather_sparse_kv_cache_exact(rt, cached, topk):
-    """Workloads of xlite/tests/kernels/gather_sparse_kv_cache.py:37-49 (bounded), exact equality."""
+    """Workloads of xlite/tests/kernels/gather_sparse_kv_cache.py:37-49, exact equality."""
     from gvirt_amd._C import gather_sparse_kv_cache
     g = torch.Generator().manual_seed(len(cached) * 31 + topk)
     bs, C, R = 128, 512, 64

@@ -142,7 +142,7 @@ def test_mla_v2_three_stage(rt, nH, nope, vd):
                c["batch"], c["maxblk"], scale, empty, 0, True)
 
 
-@pytest.mark.parametrize("cached,topk", [([127], 512), ([2047, 8191, 5841], 2048), ([4096], 512)])
+@pytest.mark.parametrize("cached,topk", [([127], 512), ([2047, 8191, 5841], 2048), ([4096], 512), ([131071], 2048), ([32751] * 3, 512)])
 def test_gather_then_mla_v3(rt, cached, topk):
     """Decode + sparse path of xlite/tests/kernels/mla_v3.py (bounded): gather, then dense attention."""
     from gvirt_amd._C import gather_sparse_kv_cache, mla_v3
