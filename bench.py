@@ -92,9 +92,22 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    run_step = step
+    if args.graph:
+        # the step captured once into a HIP graph and replayed: what a launch-bound serving loop would do
+        # (the library only enqueues kernels; its scratch pool was grown by the warm-up)
+        graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                step()
+        torch.cuda.synchronize()
+        run_step = graph.replay
+        for _ in range(3):
+            run_step()
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run_step()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
@@ -156,7 +169,8 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "vs_baseline": None, "dtype": "int8" if int8 else "bf16", "data": "synthetic",
         "config": {"workload": name, "batch": B, "n_heads": s.n_heads, "n_kv_heads": s.n_kv_heads,
                    "head_dim": s.head_dim, "block_size": s.block_size, "ctx_total": int(sum(ctx)),
-                   "ctx_max": int(max(ctx)), "kv_bytes_per_step": int(kv_bytes)},
+                   "ctx_max": int(max(ctx)), "kv_bytes_per_step": int(kv_bytes),
+                   "launch": "graph replay" if args.graph else "eager"},
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
@@ -356,6 +370,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    ap.add_argument("--graph", action="store_true",
+                    help="decode configurations: time replays of the step captured into a HIP graph instead of eager calls")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy kernel: under a counter run its "
                          "FETCH_SIZE / WRITE_SIZE readings give the scale of those counters")
