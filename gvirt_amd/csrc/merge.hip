@@ -169,16 +169,21 @@ merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_a
 }
 
 // The balanced GQA decode kernel's partials: fp32 (O, maximum in the log2 domain, normaliser) in the same
-// per-chunk slots as above, [slot][head][dv]. A wave owns one (row, head); four columns per lane.
-template <typename T>
+// per-chunk slots as above, [slot][head][dv]. A lane owns four columns, so a (row, head) needs dv / 4 lanes
+// and a wave runs 64 / (dv / 4) slots side by side; WPR waves share a (row, head) when there are few of
+// them and many slots each (a long sequence alone in its batch), and add their sums up through LDS.
+constexpr uint64_t kMergeWideBelow = 512;   // (row, head)s up to which four waves share one
+
+template <typename T, int WPR>
 __global__ void __launch_bounds__(256)
 merge_meta_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc, const float *__restrict__ part_ml,
                   const int4 *__restrict__ meta, uint32_t rows, uint32_t n_heads, uint32_t dv)
 {
-    const uint32_t lane = threadIdx.x & 63;
-    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    __shared__ float4 xch[WPR > 1 ? (WPR - 1) * 64 : 1];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * (4 / WPR) + wave / WPR;
     if (rh >= static_cast<uint64_t>(rows) * n_heads) {
-        return;
+        return;   // WPR is 1 (no barrier below) or 4 (the whole workgroup leaves together)
     }
     const uint32_t row = static_cast<uint32_t>(rh / n_heads), head = static_cast<uint32_t>(rh % n_heads);
     const int4 mt = meta[row];
@@ -200,50 +205,73 @@ merge_meta_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc
         mm = fmaxf(mm, __shfl_xor(mm, d));
     }
     const float ms = mm == -INFINITY ? 0.f : mm;
-    for (uint32_t cc = 0; cc < dv / 4; cc += 64) {
-        const uint32_t c = cc + lane;
-        const bool c_ok = c < dv / 4;   // idle lanes still take part in the exchanges
-        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        float lsum = 0.f;
-        for (uint32_t s0 = 0; s0 < n; s0 += 64) {
-            const uint32_t cnt = min(64u, n - s0);
-            float w_lane = 0.f, l_lane = 0.f;
-            if (lane < cnt) {
-                const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
-                w_lane = fast_exp2(ml.x - ms);
-                l_lane = ml.y * w_lane;
+    const uint32_t lanes_per = dv / 4;                 // 16 or 32
+    const uint32_t c = lane % lanes_per;
+    const uint32_t streams = 64 / lanes_per * WPR;     // slots summed side by side
+    const uint32_t stream = (wave % WPR) * (64 / lanes_per) + lane / lanes_per;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float lsum = 0.f;
+    for (uint32_t s0 = 0; s0 < n; s0 += 64) {
+        const uint32_t cnt = min(64u, n - s0);
+        float w_lane = 0.f, l_lane = 0.f;
+        if (lane < cnt) {
+            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
+            w_lane = fast_exp2(ml.x - ms);
+            l_lane = ml.y * w_lane;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            l_lane += __shfl_xor(l_lane, d);
+        }
+        lsum += l_lane;
+        for (uint32_t j = 0; j < cnt; j += 4 * streams) {   // uniform trip count: every lane takes part in the exchanges
+            float4 x[4];
+            float w[4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4; u++) {
+                const uint32_t idx = j + u * streams + stream;
+                const uint32_t safe = min(idx, cnt - 1);
+                x[u] = *reinterpret_cast<const float4 *>(part_acc + slot_of(s0 + safe) * dv + c * 4);
+                w[u] = __shfl(w_lane, static_cast<int>(safe));
+                w[u] = idx < cnt ? w[u] : 0.f;
             }
 #pragma unroll
-            for (int d = 32; d >= 1; d >>= 1) {
-                l_lane += __shfl_xor(l_lane, d);
-            }
-            lsum += l_lane;
-            for (uint32_t j = 0; j < cnt; j += 4) {
-                float4 x[4];
-                float w[4];
-#pragma unroll
-                for (uint32_t u = 0; u < 4; u++) {
-                    const uint32_t idx = min(j + u, cnt - 1);
-                    x[u] = c_ok ? *reinterpret_cast<const float4 *>(part_acc + slot_of(s0 + idx) * dv + c * 4)
-                                : make_float4(0.f, 0.f, 0.f, 0.f);
-                    w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
-                }
-#pragma unroll
-                for (uint32_t u = 0; u < 4; u++) {
-                    acc.x += x[u].x * w[u];
-                    acc.y += x[u].y * w[u];
-                    acc.z += x[u].z * w[u];
-                    acc.w += x[u].w * w[u];
-                }
+            for (uint32_t u = 0; u < 4; u++) {
+                acc.x += x[u].x * w[u];
+                acc.y += x[u].y * w[u];
+                acc.z += x[u].z * w[u];
+                acc.w += x[u].w * w[u];
             }
         }
-        if (c_ok) {
-            const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-            uint2 o;
-            o.x = T::pack(acc.x * inv, acc.y * inv);
-            o.y = T::pack(acc.z * inv, acc.w * inv);
-            *reinterpret_cast<uint2 *>(out + rh * dv + c * 4) = o;
+    }
+    for (uint32_t d = 32; d >= lanes_per; d >>= 1) {
+        acc.x += __shfl_xor(acc.x, static_cast<int>(d));
+        acc.y += __shfl_xor(acc.y, static_cast<int>(d));
+        acc.z += __shfl_xor(acc.z, static_cast<int>(d));
+        acc.w += __shfl_xor(acc.w, static_cast<int>(d));
+    }
+    if constexpr (WPR > 1) {
+        if (wave != 0) {
+            xch[(wave - 1) * 64 + lane] = acc;
         }
+        __syncthreads();
+        if (wave != 0) {
+            return;
+        }
+        for (uint32_t w = 0; w + 1 < WPR; w++) {
+            const float4 o = xch[w * 64 + lane];
+            acc.x += o.x;
+            acc.y += o.y;
+            acc.z += o.z;
+            acc.w += o.w;
+        }
+    }
+    if (lane < lanes_per) {
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+        uint2 o;
+        o.x = T::pack(acc.x * inv, acc.y * inv);
+        o.y = T::pack(acc.z * inv, acc.w * inv);
+        *reinterpret_cast<uint2 *>(out + rh * dv + c * 4) = o;
     }
 }
 
@@ -311,13 +339,27 @@ int launch_merge_meta(hipStream_t stream, int dtype, void *out, const float *acc
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
+    if (dv != 64 && dv != 128) {
+        return fail(XLITE_HIP_EINVAL, __func__, "value width " + std::to_string(dv) + " is neither 64 nor 128");
+    }
     const uint64_t total_rh = static_cast<uint64_t>(rows) * n_heads;
-    const dim3 grid(static_cast<uint32_t>((total_rh + 3) / 4), 1, 1);
     const int4 *m4 = reinterpret_cast<const int4 *>(meta);
-    if (dtype == XLITE_HIP_BF16) {
-        merge_meta_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
+    uint16_t *o = static_cast<uint16_t *>(out);
+    const bool bf = dtype == XLITE_HIP_BF16;
+    if (total_rh <= kMergeWideBelow) {   // few (row, head)s: a workgroup each
+        const dim3 grid(static_cast<uint32_t>(total_rh), 1, 1);
+        if (bf) {
+            merge_meta_kernel<BF16, 4><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        } else {
+            merge_meta_kernel<FP16, 4><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        }
     } else {
-        merge_meta_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
+        const dim3 grid(static_cast<uint32_t>((total_rh + 3) / 4), 1, 1);
+        if (bf) {
+            merge_meta_kernel<BF16, 1><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        } else {
+            merge_meta_kernel<FP16, 1><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        }
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

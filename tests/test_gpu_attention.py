@@ -138,6 +138,17 @@ def test_decode_ragged_batches_balanced_split(rt, model, batch, lo, hi, long_one
     check(run_attention(rt, w), oracle_attention(w))
 
 
+@pytest.mark.parametrize("model", [(32, 8, 128, 128, torch.bfloat16), (14, 2, 64, 128, torch.bfloat16),
+                                   (28, 4, 128, 16, torch.float16), (16, 1, 64, 64, torch.float16)])
+@pytest.mark.parametrize("clens", [[40000], [33000, 150, 12000], [6000] * 5])
+def test_decode_few_sequences_many_partials(rt, model, clens):
+    """Few (row, head)s whose rows are cut into up to a chunk per compute unit: the merge sums the partial
+    slots in parallel streams (side by side in a wave's lanes and in the four waves of a workgroup)."""
+    nH, nKV, d, bs, dtype = model
+    w = generic_case(23, [1] * len(clens), clens, nH, nKV, d, bs, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 def test_decode_int8_kv(rt):
     ctx = [129, 4100, 640, 17, 2048, 9000]
     w = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=True)
