@@ -87,20 +87,25 @@ merge_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc,
     }
 }
 
+constexpr uint64_t kMergeWideBelow = 512;   // (row, head)s up to which four waves share one
+
 // The merge of the MLA decode kernel's partials: O is stored normalised (O_s / l_s) in 16 bits,
 // out = sum_s (w_s l_s) Ohat_s / sum_s (w_s l_s). A row's segments sit in per-chunk slots: meta[row] =
 // (segments n, first chunk c0, first-in-chunk flag f); segment 0 is slot 2 c0 + (1 - f), segment s slot
 // 2 (c0 + s). A wave owns one (row, head): lane s computes the weight of segment s, then the segments' rows
 // (eight columns per lane) are read four at a time so that several loads are in flight per lane.
-template <typename T>
+// With few (row, head)s WPR = 4 waves share one, each summing every fourth segment, and add up through LDS.
+template <typename T, int WPR>
 __global__ void __launch_bounds__(256)
 merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_acc, const float *__restrict__ part_ml,
                  const int4 *__restrict__ meta, uint32_t rows, uint32_t n_heads, uint32_t dv)
 {
-    const uint32_t lane = threadIdx.x & 63;
-    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    __shared__ float xch[WPR > 1 ? (WPR - 1) * 9 * 64 : 1];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t stream = wave % WPR;
+    const uint64_t rh = static_cast<uint64_t>(blockIdx.x) * (4 / WPR) + wave / WPR;
     if (rh >= static_cast<uint64_t>(rows) * n_heads) {
-        return;
+        return;   // WPR is 1 (no barrier below) or 4 (the whole workgroup leaves together)
     }
     const uint32_t row = static_cast<uint32_t>(rh / n_heads), head = static_cast<uint32_t>(rh % n_heads);
     const int4 mt = meta[row];
@@ -134,15 +139,17 @@ merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_a
                 const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
                 w_lane = fast_exp2(ml.x - ms) * ml.y;
             }
-            for (uint32_t j = 0; j < cnt; j += 4) {
+            for (uint32_t j = 0; j < cnt; j += 4 * WPR) {
                 uint4 x[4];
                 float w[4];
 #pragma unroll
                 for (uint32_t u = 0; u < 4; u++) {
-                    const uint32_t idx = min(j + u, cnt - 1);
+                    const uint32_t want = j + u * WPR + stream;
+                    const uint32_t idx = min(want, cnt - 1);
                     x[u] = c_ok ? *reinterpret_cast<const uint4 *>(part_acc + slot_of(s0 + idx) * dv + c * 8)
                                 : make_uint4(0, 0, 0, 0);
-                    w[u] = j + u < cnt ? __shfl(w_lane, static_cast<int>(j + u)) : 0.f;
+                    w[u] = __shfl(w_lane, static_cast<int>(idx));
+                    w[u] = want < cnt ? w[u] : 0.f;
                 }
 #pragma unroll
                 for (uint32_t u = 0; u < 4; u++) {
@@ -154,6 +161,27 @@ merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_a
                         acc[2 * k + 1] += T::hi(xs[k]) * w[u];
                     }
                 }
+            }
+        }
+        if constexpr (WPR > 1) {
+            // one column pass at most: the waves of a (row, head) meet at the barrier the same number of times
+            if (wave != 0) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    xch[((wave - 1) * 9 + k) * 64 + lane] = acc[k];
+                }
+                xch[((wave - 1) * 9 + 8) * 64 + lane] = wsum;
+            }
+            __syncthreads();
+            if (wave != 0) {
+                return;
+            }
+            for (uint32_t w = 0; w + 1 < WPR; w++) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    acc[k] += xch[(w * 9 + k) * 64 + lane];
+                }
+                wsum += xch[(w * 9 + 8) * 64 + lane];
             }
         }
         const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
@@ -172,8 +200,6 @@ merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_a
 // per-chunk slots as above, [slot][head][dv]. A lane owns four columns, so a (row, head) needs dv / 4 lanes
 // and a wave runs 64 / (dv / 4) slots side by side; WPR waves share a (row, head) when there are few of
 // them and many slots each (a long sequence alone in its batch), and add their sums up through LDS.
-constexpr uint64_t kMergeWideBelow = 512;   // (row, head)s up to which four waves share one
-
 template <typename T, int WPR>
 __global__ void __launch_bounds__(256)
 merge_meta_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc, const float *__restrict__ part_ml,
@@ -322,12 +348,23 @@ int launch_merge_mla(hipStream_t stream, int dtype, void *out, const uint16_t *a
         return XLITE_HIP_OK;
     }
     const uint64_t total_rh = static_cast<uint64_t>(rows) * n_heads;
-    const dim3 grid(static_cast<uint32_t>((total_rh + 3) / 4), 1, 1);
     const int4 *m4 = reinterpret_cast<const int4 *>(meta);
-    if (dtype == XLITE_HIP_BF16) {
-        merge_mla_kernel<BF16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
+    uint16_t *o = static_cast<uint16_t *>(out);
+    const bool bf = dtype == XLITE_HIP_BF16;
+    if (total_rh <= kMergeWideBelow && dv <= 512) {   // few (row, head)s: a workgroup each
+        const dim3 grid(static_cast<uint32_t>(total_rh), 1, 1);
+        if (bf) {
+            merge_mla_kernel<BF16, 4><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        } else {
+            merge_mla_kernel<FP16, 4><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        }
     } else {
-        merge_mla_kernel<FP16><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(out), acc, ml, m4, rows, n_heads, dv);
+        const dim3 grid(static_cast<uint32_t>((total_rh + 3) / 4), 1, 1);
+        if (bf) {
+            merge_mla_kernel<BF16, 1><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        } else {
+            merge_mla_kernel<FP16, 1><<<grid, 256, 0, stream>>>(o, acc, ml, m4, rows, n_heads, dv);
+        }
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;

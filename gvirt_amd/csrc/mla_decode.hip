@@ -671,10 +671,10 @@ int mla_decode_plan(const MlaArgs &a, MlaPlan *pl)
         XL_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
         cu_dev = dev;
     }
-    // half of what one workgroup per compute unit would get if every row were as long as allowed, between 256
+    // half of what one workgroup per compute unit would get if every row were as long as allowed, between 128
     // and 512 positions
     uint64_t tok = max_ctx * a.total_tokens / static_cast<uint64_t>(n_cu) / 2;
-    tok = tok > 512 ? 512 : (tok < 256 ? 256 : tok);
+    tok = tok > 512 ? 512 : (tok < 128 ? 128 : tok);
     pl->chunk_min_steps = static_cast<uint32_t>(tok / kStep);
     pl->n_workgroups = static_cast<uint32_t>(n_cu);
     // with position lists no row walks more than top_k positions, and a chunk stages one entry per position

@@ -256,6 +256,15 @@ def test_mla_decode_one_long_row_among_short_ones(rt):
     check(run_mla(rt, c, scale), oracle_mla(c, scale))
 
 
+@pytest.mark.parametrize("nH,clens", [(128, [20000]), (16, [50000, 77, 9000]), (128, [3000] * 4), (8, [2500] * 40)])
+def test_mla_decode_few_rows_many_partials(rt, nH, clens):
+    """Few (row, head)s cut into a chunk per compute unit: four waves of the merge share a (row, head); the
+    last case is just above that path's limit."""
+    c = mla_case(35, [1] * len(clens), clens, nH)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
 def test_dsa_decode_pipeline_indexer_to_masked_mla(rt):
     """DeepSeek sparse attention, decode step: indexer_topk picks the positions, mla_attention attends to
     them (xlite/csrc/model.cpp:384-427). The lists go from one operator to the other untouched; the result is
