@@ -33,19 +33,28 @@ def _req(cond: bool, msg: str) -> None:
 
 
 def _dev(name: str, t: torch.Tensor, dtype=None) -> None:
+    # the checks first, the messages only when one fails: formatting a device or dtype costs more than the checks
+    if isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous() and (dtype is None or t.dtype == dtype):
+        return
     _req(isinstance(t, torch.Tensor), "%s: expected a tensor" % name)
     _req(t.is_cuda, "%s: expected a GPU tensor, got %s" % (name, t.device))
     _req(t.is_contiguous(), "%s: tensor must be contiguous" % name)
-    if dtype is not None:
-        _req(t.dtype == dtype, "%s: dtype %s unsupported! (expected %s)" % (name, t.dtype, dtype))
+    raise RuntimeError("%s: dtype %s unsupported! (expected %s)" % (name, t.dtype, dtype))
 
 
 def _act_dtype(name: str, *tensors: torch.Tensor) -> int:
     dt = tensors[0].dtype
-    _req(dt in _DT, "%s: dtype %s unsupported!" % (name, dt))
+    code = _DT.get(dt)
+    if code is None:
+        raise RuntimeError("%s: dtype %s unsupported!" % (name, dt))
     for t in tensors:
-        _req(t.dtype == dt, "%s: mixed dtypes %s / %s unsupported!" % (name, dt, t.dtype))
-    return _DT[dt]
+        if t.dtype != dt:
+            raise RuntimeError("%s: mixed dtypes %s / %s unsupported!" % (name, dt, t.dtype))
+    return code
+
+
+# torch's current stream of a device as a raw handle, without building a Stream object
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 class Runtime:
@@ -113,6 +122,8 @@ class Runtime:
         return self._pool
 
     def stream(self) -> ctypes.c_void_p:
+        if _raw_stream is not None:
+            return ctypes.c_void_p(_raw_stream(self.devid))
         return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
 
     def finish(self) -> None:
@@ -214,8 +225,8 @@ def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
         _req(k_scale.numel() * head_dim == k_cache.numel() and v_scale.numel() * head_dim == v_cache.numel(),
              "attention: one scale per (block, slot, kv head) expected")
     else:
-        _req(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
-             "attention: qkv %s kCache %s vCache %s unsupported!" % (qkv.dtype, k_cache.dtype, v_cache.dtype))
+        if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+            raise RuntimeError("attention: qkv %s kCache %s vCache %s unsupported!" % (qkv.dtype, k_cache.dtype, v_cache.dtype))
     T = qkv.shape[0]
     _req(n_kv_heads > 0 and n_heads % n_kv_heads == 0, "attention: n_heads must be a multiple of n_kv_heads")
     _req(qkv.numel() == T * (n_heads + 2 * n_kv_heads) * head_dim, "attention: qkv shape mismatch")
@@ -270,7 +281,8 @@ def mla_attention(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_cache
     for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens),
                  ("block_tables", block_tables)):
         _dev(n, t, torch.int32)
-    _req(q_absorb.dtype == torch.bfloat16, "mla: qAbsorb dtype %s unsupported!" % q_absorb.dtype)
+    if q_absorb.dtype != torch.bfloat16:
+        raise RuntimeError("mla: qAbsorb dtype %s unsupported!" % q_absorb.dtype)
     dt = _act_dtype("mla", q_absorb, qr, k_cache, pe_cache, o_absorb)
     if top_k > 2048:
         raise RuntimeError("mla: topK should be less than or equal to 2048")
@@ -348,7 +360,8 @@ def mla_v3(rt: Runtime, q_absorb: torch.Tensor, qr: torch.Tensor, k_dense_cache:
         _dev(n, t)
     for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens)):
         _dev(n, t, torch.int32)
-    _req(q_absorb.dtype == torch.bfloat16, "mla_v3: qAbsorb dtype %s unsupported!" % q_absorb.dtype)
+    if q_absorb.dtype != torch.bfloat16:
+        raise RuntimeError("mla_v3: qAbsorb dtype %s unsupported!" % q_absorb.dtype)
     dt = _act_dtype("mla_v3", q_absorb, qr, k_dense_cache, pe_dense_cache, o_absorb)
     T = q_absorb.shape[0]
     _req(k_dense_cache.numel() == batch * index_topk * kv_lora_rank, "mla_v3: k_dense shape mismatch")
@@ -412,7 +425,8 @@ def indexer_scores(rt: Runtime, q: torch.Tensor, k_cache: torch.Tensor, weight: 
     dt = _indexer_check("indexer_scores", q, k_cache, weight, query_start_loc, lens, cached_lens, block_tables,
                         n_heads, head_dim, batch, max_num_block)
     _dev("scores", scores)
-    _req(scores.dtype == q.dtype, "indexer_scores: scores dtype %s unsupported!" % scores.dtype)
+    if scores.dtype != q.dtype:
+        raise RuntimeError("indexer_scores: scores dtype %s unsupported!" % scores.dtype)
     T = q.shape[0]
     _req(scores.numel() == T * max_num_block * block_size, "indexer_scores: scores shape mismatch")
     _lib.check(rt._lib.xlite_hip_indexer_scores(

@@ -133,7 +133,7 @@ __device__ __forceinline__ uint32_t swizzle(uint32_t row)
 // ---------------------------------------------------------------------------------------------------
 constexpr uint32_t kSplitTblCap = 1024;         // block-table entries staged per segment
 constexpr uint32_t kSplitSeqCap = 4096;         // sequences whose prefix sums fit in LDS (with 2^28 steps in all)
-constexpr uint32_t kSplitMinChunk = 8;          // steps: no chunk below 128 positions
+constexpr uint32_t kSplitMinChunk = 4;          // steps: no chunk below 64 positions
 constexpr uint32_t kSplitMaxWorkgroups = 512;   // grid bound the partial slots are sized for (one workgroup per compute unit)
 constexpr uint32_t kSplitLdsWords = kSplitTblCap + kWaves;   // + batch + 1
 
