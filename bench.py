@@ -45,6 +45,21 @@ def _time_region(torch, fn, iters):
     return a.elapsed_time(b) / iters
 
 
+def _launch_dist(torch, fn, launches=100):
+    """Median, 10th and 90th percentile (ms) of `launches` back-to-back calls of `fn`, each between its own
+    pair of HIP events on the stream the kernels are launched on."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for i in range(launches):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    t = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(launches))
+    pick = lambda q: round(t[min(launches - 1, int(q * launches))], 4)
+    return {"median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9), "launches": launches}
+
+
 def _cpu_info():
     model = "unknown"
     try:
@@ -174,6 +189,7 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
+        "attention_ms_dist": _launch_dist(torch, attn),
         "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_mfma_kernel (+ merge_meta_kernel)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name.split()[0]),
@@ -313,7 +329,7 @@ def bench_mla(args, torch, rt):
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "c4 deepseek-r1 MLA absorbed decode", "batch": 32, "n_heads": 128, "ctx_total": int(sum(ctx)),
                        "kv_bytes_per_step": int(w["kv_bytes"]), "flops_per_step": int(w["flops"])},
-            "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1),
+            "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1), "attention_ms_dist": _launch_dist(torch, step),
             "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_mla_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c4"),
                          "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
