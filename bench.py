@@ -25,7 +25,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
-MEASURED_TRAFFIC_BYTES = {"c2": 1080231715, "c4": 325287281}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080231715, "c3": 302377378, "c4": 325287281, "c5": 1623716142}
 
 
 def _events(torch):
@@ -267,7 +267,7 @@ def bench_prefill(args, torch, rt):
             "tokens_per_s": round(tokens / (ms * 1e-3), 1),
             "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                         "traffic": None, "algorithmic_flops_per_step": int(flops)},
+                         "traffic": MEASURED_TRAFFIC_BYTES.get("c3"), "algorithmic_flops_per_step": int(flops)},
             "cpu_baseline": cpu}
 
 
