@@ -323,6 +323,9 @@ mla_decode_kernel(const MlaDecodeParams p)
                 const uint32_t soff = (step % kStages) * STAGE_BYTES;
                 const uint32_t lane_pos = t + gi4;
                 float mx = -INFINITY;
+                // the softmax runs at a raised wave priority: its vector instructions go ahead of the products of
+                // the SIMD's other wave (1-2 % on the step; raising it around the products instead gains nothing)
+                __builtin_amdgcn_s_setprio(2);
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++) {
 #pragma unroll
@@ -396,6 +399,7 @@ mla_decode_kernel(const MlaDecodeParams p)
                 // 32 tiles of 16 latent columns, one k-step of 32 positions in the order (16 mt + 4 gi + k),
                 // which is the order the lane's own probabilities already have
                 const uint4 pb = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+                __builtin_amdgcn_s_setprio(0);
                 typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
                 uint32_t xv[8];
 #pragma unroll
