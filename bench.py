@@ -25,7 +25,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
-MEASURED_TRAFFIC_BYTES = {"c2": 1080231715, "c3": 302377378, "c4": 325287281, "c5": 1623716142}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080233210, "c3": 302337768, "c4": 325291619, "c5": 1623718207}
 
 
 def _events(torch):
