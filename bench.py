@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c3|c4|c5|idx|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config default|c2|c1|c3|c4|c5|idx|all]
 
 Default (what the driver runs): configuration 2 of BASELINE.json — Llama-3-8B-shape GQA
 flash-decode, batch 64, every sequence at context 4096, bf16 paged KV cache with block size 128,
@@ -11,8 +11,13 @@ line; `value` is KV bytes read per second over the whole step. `roofline` prices
 kernel (the decode attention kernel) against the 8 TB/s HBM peak; `cpu_baseline` times the CPU
 oracle on a bounded sample of the same workload on the host cores.
 
-Other configurations (`--config`) print the same kind of line for their own workload; `all`
-prints one line per configuration (the first line is still configuration 2).
+With no `--config` the same line also carries `other_configs`: configurations 1, 3, 4 and 5 measured in
+the same run, each with its own value, roofline and CPU baseline. `--config c1|c2|c3|c4|c5|idx` prints the
+line of that workload alone; `all` prints one line per configuration (the first is configuration 2).
+
+Cache residency: configurations 2, 3 and 5 stream far more than the 256 MB of last-level cache per step.
+Configuration 4 (233 MB of latent cache) rotates over four distinct cache sets (932 MB) so that no step finds
+its cache resident; configuration 1 (0.8 MB) is timed step by step with a 1 GiB fill between the steps.
 """
 import argparse
 import json
@@ -26,6 +31,17 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
 MEASURED_TRAFFIC_BYTES = {"c2": 1080233210, "c3": 302337768, "c4": 325291619, "c5": 1623718207}
+# where each constant comes from: the committed counter summary whose "HBM traffic per launch" line holds it
+TRAFFIC_SOURCE = {"c2": "profiles/decode_dma_kernel_c2_llama3_8b_b64_ctx4096.md",
+                  "c3": "profiles/prefill_kernel_c3_qwen25_7b_chunked.md",
+                  "c4": "profiles/mla_decode_kernel_c4_deepseek_r1_b32.md",
+                  "c5": "profiles/decode_mfma_kernel_int8_c5_llama3_8b_b128_ragged.md"}
+
+
+def _traffic(key):
+    return {"traffic": MEASURED_TRAFFIC_BYTES.get(key),
+            "traffic_source": (TRAFFIC_SOURCE[key] + " (rocprofv3 --pmc runs of an earlier invocation of this command, "
+                               "not measured by this run)") if key in MEASURED_TRAFFIC_BYTES else None}
 
 
 def _events(torch):
@@ -79,7 +95,20 @@ def _cpu_threads(torch):
     return n
 
 
-def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_rope=True):
+def _flushed_steps(torch, fn, steps, flush):
+    """Milliseconds of `steps` calls of `fn`, each between its own pair of HIP events on the launching stream,
+    with `flush()` (untimed) before every one."""
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        flush()
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in ev]
+
+
+def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_rope=True, cold=False):
     from gvirt_amd import workloads as W
     from gvirt_amd import _C
     dev = "cuda:0"
@@ -120,15 +149,28 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         for _ in range(3):
             run_step()
         torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run_step()
-    torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    residency = "streams %.0f MB per step, far beyond the 256 MB last-level cache" % (w["kv_bytes"] / 1e6)
+    if cold:
+        # a working set that would sit in the last-level cache: every timed step follows a 1 GiB fill
+        junk = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        flush = lambda: junk.fill_(1.0)
+        ms_step = sum(_flushed_steps(torch, run_step, args.steps, flush)) / args.steps
+        t_attn = _flushed_steps(torch, attn, max(args.steps, 20), flush)
+        ms_kernel = sum(t_attn) / len(t_attn)
+        t_rope = _flushed_steps(torch, rope, max(args.steps, 20), flush) if r is not None else [0.0]
+        ms_rope = sum(t_rope) / len(t_rope)
+        residency = "cold: a 1 GiB fill runs (untimed) before every timed step; each step between its own events"
+        del junk
+    else:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run_step()
+        torch.cuda.synchronize()
+        ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # dominant kernel alone: back-to-back launches of the attention op between two events
-    ms_kernel = _time_region(torch, attn, max(args.steps, 20))
-    ms_rope = _time_region(torch, rope, max(args.steps, 20)) if r is not None else 0.0
+        # dominant kernel alone: back-to-back launches of the attention op between two events
+        ms_kernel = _time_region(torch, attn, max(args.steps, 20))
+        ms_rope = _time_region(torch, rope, max(args.steps, 20)) if r is not None else 0.0
 
     kv_bytes = w["kv_bytes"]
     qo_bytes = 2 * B * s.n_heads * s.head_dim * 2 + sum((c + s.block_size - 1) // s.block_size for c in ctx) * 4
@@ -185,15 +227,14 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "config": {"workload": name, "batch": B, "n_heads": s.n_heads, "n_kv_heads": s.n_kv_heads,
                    "head_dim": s.head_dim, "block_size": s.block_size, "ctx_total": int(sum(ctx)),
                    "ctx_max": int(max(ctx)), "kv_bytes_per_step": int(kv_bytes),
-                   "launch": "graph replay" if args.graph else "eager"},
+                   "launch": "graph replay" if args.graph else "eager", "cache_residency": residency},
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
         "attention_ms_dist": _launch_dist(torch, attn),
         "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_mfma_kernel (+ merge_meta_kernel)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name.split()[0]),
-                     "algorithmic_bytes_per_launch": int(alg_bytes)},
+                     **_traffic(name.split()[0]), "algorithmic_bytes_per_launch": int(alg_bytes)},
         "cpu_baseline": cpu,
     }
 
@@ -267,7 +308,7 @@ def bench_prefill(args, torch, rt):
             "tokens_per_s": round(tokens / (ms * 1e-3), 1),
             "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES.get("c3"), "algorithmic_flops_per_step": int(flops)},
+                         **_traffic("c3"), "algorithmic_flops_per_step": int(flops)},
             "cpu_baseline": cpu}
 
 
@@ -276,25 +317,72 @@ def bench_mla(args, torch, rt):
     from gvirt_amd import _C
     s = W.MlaShape()
     ctx = W.c4_context_lengths()
-    w = W.mla_decode(s, ctx, W.SEED_BASE + 4, device="cuda:0")
+    # four distinct cache sets (same lengths, different contents, tables and queries), used in turn: 4 x 233 MB
+    # cannot stay in the 256 MB last-level cache between the steps that use one set
+    n_sets = 4
+    sets = [W.mla_decode(s, ctx, W.SEED_BASE + 4 + 1000 * i, device="cuda:0") for i in range(n_sets)]
+    w = sets[0]
     rt.blocking = False
+    turn = [0]
+
+    def run(x):
+        _C.mla_attention(rt, x["q_absorb"], x["qr"], x["k_cache"], x["pe_cache"], x["o_absorb"], x["query_start_loc"],
+                         x["lens"], x["cached_lens"], x["block_tables"], s.n_heads, s.rope_head_dim, s.kv_lora_rank,
+                         s.block_size, x["batch"], x["max_num_blocks"], s.scale)
 
     def step():
-        _C.mla_attention(rt, w["q_absorb"], w["qr"], w["k_cache"], w["pe_cache"], w["o_absorb"], w["query_start_loc"],
-                         w["lens"], w["cached_lens"], w["block_tables"], s.n_heads, s.rope_head_dim, s.kv_lora_rank,
-                         s.block_size, w["batch"], w["max_num_blocks"], s.scale)
+        run(sets[turn[0] % n_sets])
+        turn[0] += 1
 
-    for _ in range(args.warmup):
+    for _ in range(max(args.warmup, n_sets)):
         step()
-    ms = _time_region(torch, step, args.steps)
+    steps = ((max(args.steps, n_sets) + n_sets - 1) // n_sets) * n_sets   # every set equally often
+    ms = _time_region(torch, step, steps)
+    ms_resident = _time_region(torch, lambda: run(w), steps)   # one set over and over, for comparison
     gbs = w["kv_bytes"] / (ms * 1e-3) / 1e9
     tf = w["flops"] / (ms * 1e-3) / 1e12
+    dist = _launch_dist(torch, step)
+
+    # the two einsums of the mla_v2 operator around the attention (W_UK absorb, W_UV), reported separately
+    g = torch.Generator(device="cuda:0").manual_seed(W.SEED_BASE + 44)
+    B, H, C, N, V = w["batch"], s.n_heads, s.kv_lora_rank, s.nope_head_dim, s.v_head_dim
+    q_nope = torch.randn(B, H, N + s.rope_head_dim, generator=g, device="cuda:0").bfloat16()
+    wuk = [(torch.randn(H, N, C, generator=g, device="cuda:0") * N ** -0.5).bfloat16() for _ in range(n_sets * 4)]
+    wuv = [(torch.randn(H, C, V, generator=g, device="cuda:0") * C ** -0.5).bfloat16() for _ in range(n_sets * 4)]
+    q_abs = torch.empty(B, H * C, dtype=torch.bfloat16, device="cuda:0")
+    o_v = torch.empty(B, H * V, dtype=torch.bfloat16, device="cuda:0")
+    et = [0]
+
+    def absorb():   # 16 weight sets of 16.8 MB in turn: 268 MB, not resident between uses
+        _C._einsum(rt, "bench", q_nope, wuk[et[0] % len(wuk)], q_abs, B, H, N, C, False, False, t_stride=N + s.rope_head_dim)
+        et[0] += 1
+
+    def unabsorb():
+        _C._einsum(rt, "bench", w["o_absorb"], wuv[et[0] % len(wuv)], o_v, B, H, C, V, False, False)
+        et[0] += 1
+
+    for f in (absorb, unabsorb):
+        for _ in range(3):
+            f()
+    ms_abs = _time_region(torch, absorb, 32)
+    ms_unabs = _time_region(torch, unabsorb, 32)
+    wbytes = H * N * C * 2
+    _C._einsum(rt, "bench", q_nope, wuk[0], q_abs, B, H, N, C, False, False, t_stride=N + s.rope_head_dim)
+    torch.cuda.synchronize()
+    ein_err = float((q_abs.view(B, H, C).float() - torch.einsum("mht,htd->mhd", q_nope[:, :, :N].float(), wuk[0].float())).abs().max())
+    einsum = {"absorb_ms": round(ms_abs, 4), "unabsorb_ms": round(ms_unabs, 4), "weight_bytes_each": wbytes,
+              "absorb_GBs": round((wbytes + q_nope.numel() * 2 + q_abs.numel() * 2) / (ms_abs * 1e-3) / 1e9, 1),
+              "unabsorb_GBs": round((wbytes + q_abs.numel() * 2 + o_v.numel() * 2) / (ms_unabs * 1e-3) / 1e9, 1),
+              "frac_of_hbm_peak": round((wbytes + q_nope.numel() * 2 + q_abs.numel() * 2) / (ms_abs * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+              "max_abs_err_vs_torch_fp32": ein_err,
+              "note": "einsum_kernel, 16 weight sets used in turn; bound by the 16.8 MB weight read"}
     cpu = None
     if not args.no_cpu:
         # the oracle (the checker, not the thing measured) on two of the sequences: parity, then its rate
         sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
         from oracle import xlite_oracle as O
         ncpu = _cpu_threads(torch)
+        run(w)
         torch.cuda.synchronize()
         sample = [0, len(ctx) // 2]
         c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in w.items()}
@@ -325,13 +413,17 @@ def bench_mla(args, torch, rt):
                "max_abs_err_vs_gpu": float(err.max())}
     floor_ms = max(w["kv_bytes"] / (HBM_PEAK_GBS * 1e9), w["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12)) * 1e3
     return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
-            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+            "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, n_sets), "ms_per_step": round(ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "c4 deepseek-r1 MLA absorbed decode", "batch": 32, "n_heads": 128, "ctx_total": int(sum(ctx)),
-                       "kv_bytes_per_step": int(w["kv_bytes"]), "flops_per_step": int(w["flops"])},
-            "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1), "attention_ms_dist": _launch_dist(torch, step),
+                       "kv_bytes_per_step": int(w["kv_bytes"]), "flops_per_step": int(w["flops"]),
+                       "cache_residency": "%d distinct cache sets of %.0f MB used in turn (%.0f MB in all, beyond the 256 MB "
+                                          "last-level cache); one set over and over takes %.4f ms per step" %
+                                          (n_sets, w["kv_bytes"] / 1e6, n_sets * w["kv_bytes"] / 1e6, ms_resident)},
+            "tflops": round(tf, 2), "tokens_per_s": round(32 / (ms * 1e-3), 1), "attention_ms_dist": dist,
+            "ms_per_step_one_resident_set": round(ms_resident, 4), "einsums": einsum,
             "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_mla_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c4"),
+                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), **_traffic("c4"),
                          "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
             "cpu_baseline": cpu}
 
@@ -384,7 +476,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="c2")
+    ap.add_argument("--config", default="default",
+                    help="default: configuration 2 with the other configurations attached; c1..c5, idx: that one alone; "
+                         "all: one line each")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
     ap.add_argument("--graph", action="store_true",
                     help="decode configurations: time replays of the step captured into a HIP graph instead of eager calls")
@@ -411,26 +505,44 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    def run_config(c):
+        if c == "c2":
+            return bench_gqa_decode(args, torch, rt, "c2 llama-3-8b GQA flash-decode + reshape_and_cache", W.LLAMA3_8B,
+                                    [4096] * 64, W.SEED_BASE + 2)
+        if c == "c1":
+            return bench_gqa_decode(args, torch, rt, "c1 qwen2-0.5b GQA decode", W.QWEN2_05B, W.c1_context_lengths(),
+                                    W.SEED_BASE + 1, cold=True)
+        if c == "c5":
+            return bench_gqa_decode(args, torch, rt, "c5 llama-3-8b int8-KV decode", W.LLAMA3_8B, W.c5_context_lengths(),
+                                    W.SEED_BASE + 5, int8=True)
+        if c == "c3":
+            return bench_prefill(args, torch, rt)
+        if c == "c4":
+            return bench_mla(args, torch, rt)
+        if c == "idx":
+            return bench_indexer(args, torch, rt)
+        raise SystemExit("unknown config " + c)
+
+    if args.config == "default":
+        # the headline line (configuration 2) carrying the other configurations measured in the same run
+        out = run_config("c2")
+        others = {}
+        for c in ("c1", "c3", "c4", "c5"):
+            try:
+                o = run_config(c)
+                for k in ("metric", "n_gpus", "higher_is_better", "scaling", "vs_baseline", "data"):
+                    o.pop(k, None)
+                others[c] = o
+            except (Exception, SystemExit) as e:   # the headline line is printed whatever happens to the others
+                others[c] = {"error": "%s: %s" % (type(e).__name__, e)}
+            torch.cuda.empty_cache()
+        out["other_configs"] = others
+        print(json.dumps(out), flush=True)
+        return
     todo = ["c2", "c1", "c5", "c3", "c4"] if args.config == "all" else [args.config]
     for c in todo:
-        if c == "c2":
-            out = bench_gqa_decode(args, torch, rt, "c2 llama-3-8b GQA flash-decode + reshape_and_cache", W.LLAMA3_8B,
-                                   [4096] * 64, W.SEED_BASE + 2)
-        elif c == "c1":
-            out = bench_gqa_decode(args, torch, rt, "c1 qwen2-0.5b GQA decode", W.QWEN2_05B, W.c1_context_lengths(),
-                                   W.SEED_BASE + 1)
-        elif c == "c5":
-            out = bench_gqa_decode(args, torch, rt, "c5 llama-3-8b int8-KV decode", W.LLAMA3_8B, W.c5_context_lengths(),
-                                   W.SEED_BASE + 5, int8=True)
-        elif c == "c3":
-            out = bench_prefill(args, torch, rt)
-        elif c == "c4":
-            out = bench_mla(args, torch, rt)
-        elif c == "idx":
-            out = bench_indexer(args, torch, rt)
-        else:
-            raise SystemExit("unknown config " + c)
-        print(json.dumps(out), flush=True)
+        print(json.dumps(run_config(c)), flush=True)
+        torch.cuda.empty_cache()
 
 
 if __name__ == "__main__":

@@ -91,6 +91,7 @@ class Runtime:
         self.aic_num = self.num_cu
         self.aiv_num = self.num_cu
         self._pool: Optional[torch.Tensor] = None
+        self._retired: List[torch.Tensor] = []
         self.init_tensor_pool(size)
 
     # -- reference API ---------------------------------------------------------------------
@@ -111,10 +112,18 @@ class Runtime:
 
     # -- scratch -------------------------------------------------------------------------------
     def _grow(self, nbytes: int) -> None:
+        """One scratch pool per Runtime, shared by every call on it: calls that use one Runtime from two
+        streams at once race on it (the reference's Runtime is not re-entrant either,
+        xlite/csrc/runtime.cpp:42). A pool that was handed out is never freed while the Runtime lives:
+        kernels still queued and captured graphs keep its address."""
         nbytes = max(nbytes, 1 << 20)
         if self._pool is None or self._pool.numel() < nbytes:
             if self._pool is not None:
-                torch.cuda.synchronize(self.device)
+                if torch.cuda.is_current_stream_capturing():
+                    raise RuntimeError("Runtime: the scratch pool must grow to %d bytes, which cannot happen while a "
+                                       "graph is being captured; run the shape once before the capture or give "
+                                       "Runtime a larger size" % nbytes)
+                self._retired.append(self._pool)
             self._pool = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
 
     def workspace(self, nbytes: int) -> torch.Tensor:

@@ -5,9 +5,12 @@ using namespace xlite;
 
 namespace {
 
+// As many query rows as sequences: a decode step in all but contrived batches (the lengths live in
+// device memory, so the host cannot look). The decode kernels work row by row and do not rely on it: a
+// batch such as lens = [2, 0] is served correctly, only without sharing the cache reads of a
+// sequence's rows. Reference: decode iff every length is 1 (xlite/csrc/runtime.cpp:466-470).
 bool is_decode_batch(uint32_t total_tokens, uint32_t batch)
 {
-    // every sequence contributes at least one row, so equality means one row each
     return total_tokens == batch;
 }
 
@@ -60,10 +63,6 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
                "n_heads must be a positive multiple of n_kv_heads");
     XL_REQUIRE(block_size > 0 && max_num_block > 0, "block_size and max_num_block must be positive");
     XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || (k_scale && v_scale), "int8 KV cache needs k_scale and v_scale");
-    XL_REQUIRE(total_tokens >= batch, "fewer query tokens than sequences");
-    if (batch == 0 || total_tokens == 0) {
-        return XLITE_HIP_OK;
-    }
     AttentionArgs a{qkv, k_cache, v_cache, output, query_start_loc, lens, cached_lens, block_tables,
                     total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
                     dtype, kv_dtype, k_scale, v_scale, workspace, workspace_bytes};
@@ -172,7 +171,6 @@ extern "C" int xlite_hip_mla_attention(void *stream, const void *q_absorb, const
                    cached_lens && block_tables,
                "null tensor");
     XL_REQUIRE(n_heads > 0 && block_size > 0 && max_num_blocks > 0, "zero head count or block geometry");
-    XL_REQUIRE(total_tokens >= batch, "fewer query tokens than sequences");
     MlaArgs a{q_absorb, qr, k_cache, pe_cache, o_absorb, query_start_loc, lens, cached_lens, block_tables,
               total_tokens, n_heads, rope_head_dim, kv_lora_rank, block_size, batch, max_num_blocks,
               0, scale, topk_indices, top_k, dtype, workspace, workspace_bytes};

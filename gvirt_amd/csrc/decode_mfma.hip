@@ -20,7 +20,9 @@
 // kernel merges the partials of every query row (merge.hip).
 //
 // Replaces the split-KV path of the reference (xlite/csrc/kernels/flash_attention.h:323-628) for
-// batches in which every sequence contributes one query row.
+// batches with as many query rows as sequences. The unit of work is the query row: in the usual decode
+// step every sequence has one, but sequences without rows and sequences with several (row r sees
+// cached + r + 1 positions) are served alike.
 #include "attention_common.h"
 
 namespace xlite {
@@ -83,6 +85,7 @@ struct DecodeMfmaParams {
     uint32_t max_num_block;
     uint32_t n_sub;        // sub ranges of a segment handled by different waves (kv heads < 8)
     uint32_t batch;
+    uint32_t total_rows;   // query rows of the batch (one per sequence in a plain decode step)
 };
 
 // 8 cache elements (uint4 = 16-bit, uint2 = int8) -> 8 x 16-bit in a uint4
@@ -121,21 +124,21 @@ __device__ __forceinline__ uint32_t swizzle(uint32_t row)
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Work split of the decode kernels: every sequence owns ceil(limit / 16) steps, limit its visible range;
-// the sequences' steps laid end to end are cut into equal chunks, one per workgroup (the lengths live in
+// Work split of the decode kernels: every query row owns ceil(limit / 16) steps, limit its visible range;
+// the rows' steps laid end to end are cut into equal chunks, one per workgroup (the lengths live in
 // device memory, so every workgroup computes the prefix sums itself), so that ragged batches keep every
-// compute unit equally busy. A chunk that crosses a sequence boundary runs as several segments. Only a
-// chunk's first and last segment can be parts of sequences that continue in other chunks: chunk c owns the
-// partial slots 2c (its first segment) and 2c + 1 (its last, when that is another one); a sequence cut into
+// compute unit equally busy. A chunk that crosses a row boundary runs as several segments. Only a
+// chunk's first and last segment can be parts of rows that continue in other chunks: chunk c owns the
+// partial slots 2c (its first segment) and 2c + 1 (its last, when that is another one); a row cut into
 // n segments that starts in chunk c0 finds them at 2 c0 (+ 1 unless it is that chunk's first segment),
-// 2 (c0 + 1), ... and its meta entry (n, c0, first flag) tells the merge kernel so. Sequences inside one
+// 2 (c0 + 1), ... and its meta entry (n, c0, first flag) tells the merge kernel so. Rows inside one
 // chunk are final.
 // ---------------------------------------------------------------------------------------------------
 constexpr uint32_t kSplitTblCap = 1024;         // block-table entries staged per segment
-constexpr uint32_t kSplitSeqCap = 4096;         // sequences whose prefix sums fit in LDS (with 2^28 steps in all)
+constexpr uint32_t kSplitSeqCap = 4096;         // query rows whose prefix sums fit in LDS (with 2^28 steps in all)
 constexpr uint32_t kSplitMinChunk = 4;          // steps: no chunk below 64 positions
 constexpr uint32_t kSplitMaxWorkgroups = 512;   // grid bound the partial slots are sized for (one workgroup per compute unit)
-constexpr uint32_t kSplitLdsWords = kSplitTblCap + kWaves;   // + batch + 1
+constexpr uint32_t kSplitLdsWords = kSplitTblCap + kWaves;   // + rows + 1
 
 // what is the same in every lane, said so: scalar address arithmetic follows
 __device__ __forceinline__ uint32_t uni(uint32_t x)
@@ -145,37 +148,55 @@ __device__ __forceinline__ uint32_t uni(uint32_t x)
 
 struct DecodeSplit {
     const DecodeMfmaParams &p;
-    uint32_t *wave_tot, *pref;   // LDS: kWaves words, batch + 1 words
-    uint32_t lane, wave, B;
+    uint32_t *wave_tot, *pref;   // LDS: kWaves words, rows + 1 words
+    uint32_t lane, wave, R;      // R: query rows of the batch, the units of the split
     bool in_lanes;
-    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_tok = 0, total = 0, chunk = 0, n_chunks = 0;
+    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_seq = 0, total = 0, chunk = 0, n_chunks = 0;
 
     // `lanes_ok`: a kernel short of registers keeps the sums in LDS whatever the batch
     __device__ __forceinline__ DecodeSplit(const DecodeMfmaParams &params, uint32_t *lds, uint32_t lane_, uint32_t wave_,
                                            bool lanes_ok = true)
-        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_), B(params.batch),
-          in_lanes(lanes_ok && params.batch <= 64)
+        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_), R(params.total_rows),
+          in_lanes(lanes_ok && params.total_rows <= 64)
     {
     }
-    __device__ __forceinline__ uint32_t steps_of(uint32_t i, uint32_t *limit) const
+    // The sequence that owns query row t. A batch of one row per sequence answers at once; otherwise (some
+    // sequences without rows, others with several) the last sequence that starts at or before t: a
+    // sequence without rows shares its start with its successor, so the last one is the owner.
+    __device__ __forceinline__ uint32_t seq_of_row(uint32_t t) const
     {
-        const int32_t ql = p.lens[i];
-        *limit = ql > 0 ? static_cast<uint32_t>(p.cached_lens[i] + 1) : 0u;   // the visible range of the sequence's row
-        if (ql <= 0 && blockIdx.x == 0) {
-            reinterpret_cast<int4 *>(p.part_meta)[p.query_start_loc[i]] = make_int4(0, 0, 0, 0);   // nothing to merge
+        if (t < p.batch && p.query_start_loc[t] == static_cast<int32_t>(t) && p.lens[t] == 1) {
+            return t;
         }
+        uint32_t lo = 0, hi = p.batch;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (p.query_start_loc[mid] <= static_cast<int32_t>(t)) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        return lo;
+    }
+    // steps of row t; *limit = its visible range: row r of its sequence sees cached + r + 1 positions
+    __device__ __forceinline__ uint32_t steps_of(uint32_t t, uint32_t *limit, uint32_t *seq) const
+    {
+        const uint32_t s = seq_of_row(t);
+        const int32_t lim = p.cached_lens[s] + (static_cast<int32_t>(t) - p.query_start_loc[s]) + 1;
+        *limit = static_cast<uint32_t>(lim > 1 ? lim : 1);
+        *seq = s;
         return ceil_div(*limit, static_cast<uint32_t>(kStep));
     }
-    // Exclusive prefix sums of the step counts. Up to 64 sequences: every wave keeps them in its lanes
-    // (lane = sequence), nothing goes through LDS. More: thread t owns `ipt` consecutive sequences and the
-    // sums land in LDS, each entry packed with its sequence's (limit - 1) % 16. Contains barriers in the
+    // Exclusive prefix sums of the step counts. Up to 64 rows: every wave keeps them in its lanes
+    // (lane = row), nothing goes through LDS. More: thread t owns `ipt` consecutive rows and the
+    // sums land in LDS, each entry packed with its row's (limit - 1) % 16. Contains barriers in the
     // second case: every thread of the workgroup calls it.
     __device__ __forceinline__ void scan()
     {
         if (in_lanes) {
-            if (lane < B) {
-                ln_tok = static_cast<uint32_t>(p.query_start_loc[lane]);
-                ln_steps = steps_of(lane, &ln_limit);
+            if (lane < R) {
+                ln_steps = steps_of(lane, &ln_limit, &ln_seq);
             }
             uint32_t incl = ln_steps;
 #pragma unroll
@@ -186,11 +207,11 @@ struct DecodeSplit {
             ln_pref = incl - ln_steps;
             total = uni(__shfl(incl, 63));
         } else {
-            const uint32_t ipt = ceil_div(B, static_cast<uint32_t>(kWaves * 64));
-            const uint32_t i0 = min(B, threadIdx.x * ipt), i1 = min(B, i0 + ipt);
-            uint32_t mine = 0, limit;
+            const uint32_t ipt = ceil_div(R, static_cast<uint32_t>(kWaves * 64));
+            const uint32_t i0 = min(R, threadIdx.x * ipt), i1 = min(R, i0 + ipt);
+            uint32_t mine = 0, limit, seq;
             for (uint32_t i = i0; i < i1; i++) {
-                mine += steps_of(i, &limit);
+                mine += steps_of(i, &limit, &seq);
             }
             uint32_t incl = mine;
 #pragma unroll
@@ -208,15 +229,15 @@ struct DecodeSplit {
             }
             uint32_t run = before + incl - mine;
             for (uint32_t i = i0; i < i1; i++) {
-                const uint32_t n = steps_of(i, &limit);
+                const uint32_t n = steps_of(i, &limit, &seq);
                 pref[i] = (run << 4) | ((limit - 1) & 15u);
                 run += n;
             }
             if (threadIdx.x == kWaves * 64 - 1) {
-                pref[B] = (before + incl) << 4;
+                pref[R] = (before + incl) << 4;
             }
             __syncthreads();
-            total = uni(pref[B]) >> 4;
+            total = uni(pref[R]) >> 4;
         }
         if (total != 0) {
             chunk = max(ceil_div(total, gridDim.x), kSplitMinChunk);
@@ -224,8 +245,8 @@ struct DecodeSplit {
             n_chunks = ceil_div(total, chunk);
         }
     }
-    // first step, step count and visible range of sequence i
-    __device__ __forceinline__ void seq_info(uint32_t i, uint32_t *first, uint32_t *n, uint32_t *limit) const
+    // first step, step count and visible range of row i (every row has at least one step)
+    __device__ __forceinline__ void row_info(uint32_t i, uint32_t *first, uint32_t *n, uint32_t *limit) const
     {
         if (in_lanes) {
             *first = uni(__shfl(ln_pref, static_cast<int>(i)));
@@ -235,17 +256,17 @@ struct DecodeSplit {
             const uint32_t a = uni(pref[i]), b = uni(pref[i + 1]);
             *first = a >> 4;
             *n = (b >> 4) - *first;
-            *limit = *n == 0 ? 0u : (*n - 1) * kStep + (a & 15u) + 1;
+            *limit = (*n - 1) * kStep + (a & 15u) + 1;
         }
     }
-    // the sequence that holds step `start`: the last one whose prefix is <= start
-    __device__ __forceinline__ uint32_t seq_of(uint32_t start) const
+    // the row that holds step `start`: the last one whose prefix is <= start
+    __device__ __forceinline__ uint32_t row_of_step(uint32_t start) const
     {
         if (in_lanes) {
-            const uint64_t mask = __ballot(lane < B && ln_pref <= start);
+            const uint64_t mask = __ballot(lane < R && ln_pref <= start);
             return static_cast<uint32_t>(__builtin_popcountll(mask)) - 1;
         }
-        uint32_t lo = 0, hi = B;
+        uint32_t lo = 0, hi = R;
         while (hi - lo > 1) {
             const uint32_t mid = (lo + hi) >> 1;
             if ((uni(pref[mid]) >> 4) <= start) {
@@ -256,33 +277,29 @@ struct DecodeSplit {
         }
         return lo;
     }
-    __device__ __forceinline__ uint32_t tok_of(uint32_t seq) const
+    __device__ __forceinline__ uint32_t seq_of(uint32_t row) const
     {
-        return in_lanes ? uni(__shfl(ln_tok, static_cast<int>(seq))) : static_cast<uint32_t>(p.query_start_loc[seq]);
+        return in_lanes ? uni(__shfl(ln_seq, static_cast<int>(row))) : uni(seq_of_row(uni(row)));
     }
-    // segment(seq, tok, t0, t1, whole, partial slot, first piece of its sequence, meta of the sequence)
+    // segment(seq, row, t0, t1, whole, partial slot, first piece of its row, meta of the row)
     template <typename F>
     __device__ __forceinline__ void for_each_segment(F &&segment) const
     {
         for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
             const uint32_t start = c * chunk, end = min(total, start + chunk);
-            uint32_t seq = seq_of(start), pos = start;
+            uint32_t row = row_of_step(start), pos = start;
             while (pos < end) {
                 uint32_t first, n, limit;
-                seq_info(seq, &first, &n, &limit);
-                if (n == 0) {
-                    seq++;
-                    continue;
-                }
+                row_info(row, &first, &n, &limit);
                 const uint32_t a = pos - first, b = min(n, a + (end - pos));
                 const bool whole = a == 0 && b == n;
                 const bool first_seg = pos == start;
                 const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
                 const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
-                segment(uni(seq), tok_of(seq), uni(a * kStep), uni(min(limit, b * kStep)), whole,
+                segment(seq_of(row), uni(row), uni(a * kStep), uni(min(limit, b * kStep)), whole,
                         uni(2 * c + (first_seg ? 0u : 1u)), a == 0, meta);
                 pos += b - a;
-                seq++;
+                row++;
             }
         }
     }
@@ -951,7 +968,7 @@ template <typename T>
 int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
-                       (kSplitLdsWords + p.batch + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + p.total_rows + 1) * sizeof(uint32_t);
     auto kernel = decode_dma_kernel<T>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
@@ -966,7 +983,7 @@ template <typename T, int D, bool KV8, bool MULTI_SUB>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
-                       (kSplitLdsWords + p.batch + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + p.total_rows + 1) * sizeof(uint32_t);
     auto kernel = decode_mfma_kernel<T, D, KV8, MULTI_SUB>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
@@ -992,7 +1009,7 @@ bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_
                            uint32_t total_tokens)
 {
     const uint32_t group = n_heads / n_kv_heads;
-    // one row per sequence; the work split keeps the batch's prefix sums in LDS
+    // the work split keeps the prefix sums of the batch's rows in LDS
     (void)n_kv_heads;
     return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16 && total_tokens <= kSplitSeqCap;
 }
@@ -1048,8 +1065,9 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     p.block_size = a.block_size;
     p.max_num_block = a.max_num_block;
     p.batch = a.batch;
+    p.total_rows = a.total_tokens;
     DecodeSplitPlan pl{};
-    decode_split_plan(a.batch, a.n_heads, a.head_dim, a.block_size, a.max_num_block, &pl);
+    decode_split_plan(a.total_tokens, a.n_heads, a.head_dim, a.block_size, a.max_num_block, &pl);
     const size_t need = pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
     if (a.workspace == nullptr || a.workspace_bytes < need) {
         return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small: need " + std::to_string(need) +

@@ -34,6 +34,7 @@ constexpr int kThreads = kWaves * 64;
 constexpr int kMTile = kWaves * 32;
 constexpr int BN = 64;                    // positions per KV tile
 constexpr int kStages = 4;
+constexpr size_t kLdsLimit = 160 * 1024;   // LDS of a compute unit: the stages plus the staged block-table row must fit
 constexpr int NT = BN / 32;               // 32-position sub tiles
 constexpr uint32_t kMinSplitTiles = 8;          // a KV split walks at least 512 positions
 
@@ -520,7 +521,11 @@ bool prefill_mfma_supported(const AttentionArgs &a)
     // the division by the block size is a multiply-high, exact while position * block_size < 2^32
     // the positions of one copy instruction (1 KiB: four rows of head_dim 128, eight of head_dim 64) share a block
     const uint32_t per_copy = a.head_dim == 128 ? 4 : 8;
+    // the sequence's block-table row is staged in LDS behind the KV stages
+    const size_t lds = static_cast<size_t>(kStages) * 2 * BN * a.head_dim * 2 +
+                       (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     return (a.head_dim == 128 || a.head_dim == 64) && a.kv_dtype == XLITE_HIP_KV_SAME && a.block_size % per_copy == 0 &&
+           lds <= kLdsLimit &&
            static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32) &&
            a.n_heads % a.n_kv_heads == 0;
 }
@@ -594,7 +599,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     const size_t lds = static_cast<size_t>(kStages) * 2 * BN * a.head_dim * 2 +
                        (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     const bool bf = a.dtype == XLITE_HIP_BF16;
-    XL_REQUIRE(lds <= 160 * 1024, "block table too long for the prefill kernel");
+    XL_REQUIRE(lds <= kLdsLimit, "block table too long for the prefill kernel");
     const void *kernel = a.head_dim == 128
                              ? (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 128>)
                                    : reinterpret_cast<const void *>(prefill_kernel<FP16, 128>))

@@ -149,6 +149,39 @@ def test_decode_few_sequences_many_partials(rt, model, clens):
     check(run_attention(rt, w), oracle_attention(w))
 
 
+# sequences without rows and sequences with several, with as many rows as sequences (the batch shape the
+# decode kernels are chosen by) and otherwise
+ZERO_LEN_WORK = [([100, 50], [2, 0]), ([10, 700, 33], [0, 3, 0]), ([5, 9, 300], [1, 0, 1]), ([100, 50], [1, 0]),
+                 ([0, 0, 0], [0, 3, 0]), ([40, 2000, 7, 129], [0, 0, 4, 0]), ([300, 20], [0, 1])]
+
+
+@pytest.mark.parametrize("model", [(32, 8, 128, 128, torch.bfloat16), (14, 2, 64, 128, torch.bfloat16),
+                                   (8, 1, 128, 16, torch.float16), (64, 2, 128, 128, torch.bfloat16),
+                                   (8, 2, 128, 20, torch.bfloat16)])
+@pytest.mark.parametrize("work", ZERO_LEN_WORK)
+def test_zero_length_sequences(rt, model, work):
+    """Decode iff every length is 1 (xlite/csrc/runtime.cpp:466-470); a batch with as many rows as sequences
+    need not be one. Rows of absent sequences do not exist; row r of a sequence sees cached + r + 1 keys."""
+    nH, nKV, d, bs, dtype = model
+    clens, lens = work
+    w = generic_case(31, lens, clens, nH, nKV, d, bs, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
+@pytest.mark.parametrize("batch", [100, 700])
+def test_zero_length_sequences_many_rows(rt, batch):
+    """The same with more rows than a wave has lanes (prefix sums of the split through LDS): lengths of 0, 1 and
+    2 that add up to the number of sequences."""
+    rng = np.random.default_rng(batch)
+    lens = [1] * batch
+    for i in rng.choice(batch // 2, size=batch // 5, replace=False):
+        lens[2 * i], lens[2 * i + 1] = 2, 0
+    clens = [int(x) for x in rng.integers(1, 900, size=batch)]
+    w = generic_case(32, lens, clens, 32, 8, 128, 128, torch.bfloat16, rms=True)
+    assert sum(lens) == batch
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 def test_decode_int8_kv(rt):
     ctx = [129, 4100, 640, 17, 2048, 9000]
     w = W.gqa_decode(W.LLAMA3_8B, ctx, 77, int8_kv=True)
@@ -291,3 +324,14 @@ def test_prefill_at_the_longest_reference_length_sampled_rows(rt, model):
         one["query_start_loc"] = torch.tensor([0], dtype=torch.int32)
         one["output"] = torch.zeros(1, nH * d, dtype=dtype)
         check(got[r:r + 1], oracle_attention(one))
+
+
+@pytest.mark.parametrize("model,lens", [((8, 1, 128, 16, torch.bfloat16), [3]), ((64, 2, 128, 16, torch.bfloat16), [1]),
+                                        ((14, 2, 64, 8, torch.float16), [2])])
+def test_block_tables_too_long_for_the_streaming_prefill_kernel(rt, model, lens):
+    """More block-table entries per sequence than the streaming prefill kernel can stage next to its KV stages
+    (a 131k-token context at block size 16): the call is served by the kernels without that bound."""
+    nH, nKV, d, bs, dtype = model
+    w = generic_case(19, lens, [131100], nH, nKV, d, bs, dtype, rms=True)
+    assert w["max_num_block"] > 8191
+    check(run_attention(rt, w), oracle_attention(w))
