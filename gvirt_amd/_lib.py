@@ -17,6 +17,8 @@ SIGNATURES = {
     "xlite_hip_rope_and_cache": (_i32, [_vp] * 7 + [_u32] * 6 + [_i32, _u64, _u64, _i32]),
     "xlite_hip_attention_workspace_bytes": (_sz, [_u32] * 7),
     "xlite_hip_attention": (_i32, [_vp] * 9 + [_u32] * 7 + [_i32, _i32, _vp, _vp, _vp, _sz]),
+    "xlite_hip_attention_noalloc_scratch_bytes": (_sz, []),
+    "xlite_hip_attention_noalloc": (_i32, [_vp] * 9 + [_u32] * 7 + [_i32, _i32, _vp, _vp]),
     "xlite_hip_mla_workspace_bytes": (_sz, [_u32] * 8),
     "xlite_hip_mla_attention": (_i32, [_vp] * 10 + [_u32] * 7 + [_f32, _vp, _u32, _i32, _vp, _sz]),
     "xlite_hip_mla_v3": (_i32, [_vp] * 9 + [_u32] * 6 + [_f32, _i32, _vp, _sz]),

@@ -342,6 +342,27 @@ int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *k_cache, in
                                   uint32_t rot_dim, uint32_t block_size, int is_neox,
                                   uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype);
 
+/* ------------------------------------------------------------------------
+ * attention_noalloc - xlite_hip_attention for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid it). It has no
+ * counterpart in the reference, whose operators draw scratch from the Runtime's tensor pool.
+ * Same arguments and results as xlite_hip_attention without the workspace: the split-KV
+ * partial results go to a buffer of XLITE_HIP_NOALLOC_SCRATCH_BYTES that is part of the
+ * library's device image (one copy per GPU, held until the process ends). The call
+ * allocates and frees nothing. A shape whose xlite_hip_attention_workspace_bytes() exceeds
+ * the buffer is refused with XLITE_HIP_ENOSPC. Every call on a GPU shares that GPU's
+ * buffer: calls that overlap on one GPU (two streams, two threads) race on it.
+ * ---------------------------------------------------------------------- */
+#define XLITE_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+size_t xlite_hip_attention_noalloc_scratch_bytes(void);
+int xlite_hip_attention_noalloc(void *stream, const void *qkv, const void *k_cache, const void *v_cache,
+                                void *output, const int32_t *query_start_loc, const int32_t *lens,
+                                const int32_t *cached_lens, const int32_t *block_tables,
+                                uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                                uint32_t head_dim, uint32_t block_size, uint32_t batch,
+                                uint32_t max_num_block, int dtype, int kv_dtype, const float *k_scale,
+                                const float *v_scale);
+
 #ifdef __cplusplus
 }
 #endif
