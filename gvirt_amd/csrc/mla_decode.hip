@@ -144,6 +144,25 @@ mla_decode_kernel(const MlaDecodeParams p)
         const bool single = n_slots == 1;
         const bool listed = LISTS && causal > p.top_k;
         const uint32_t blk0 = dense || listed ? 0 : t0 / p.block_size;
+        // ---- [q_absorb | qr] of the lane's head: 16 bytes of every 64-byte k-step. Heads past the end repeat
+        // the last one; their results are never stored. The first pass's loads are issued here, ahead of the
+        // block-table lookups, so that both travel together.
+        uint4 qreg[KS_C + KS_R];
+        auto load_q = [&](uint32_t h0) {
+            const uint32_t head = h0 + wave * 16 + col;
+            const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + min(head, p.n_heads - 1);
+            const uint4 *qa = reinterpret_cast<const uint4 *>(p.q_absorb + rh * C) + gi;
+            const uint4 *qq = reinterpret_cast<const uint4 *>(p.qr + rh * R) + gi;
+#pragma unroll
+            for (int ks = 0; ks < KS_C; ks++) {
+                qreg[ks] = qa[4 * ks];
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS_R; ks++) {
+                qreg[KS_C + ks] = qq[4 * ks];
+            }
+        };
+        load_q(0);
         if (listed) {
             // cache row of every list entry of the segment (tbl_lds[i] for entry t0 + i) and, per step, the mask
             // of its usable entries: inside the causal range, not a repeat of its predecessor. The others point
@@ -182,27 +201,8 @@ mla_decode_kernel(const MlaDecodeParams p)
             const uint32_t head = hw + col;
             const bool h_ok = head < p.n_heads;
 
-            // ---- [q_absorb | qr] of the lane's head: 16 bytes of every 64-byte k-step. Heads past the end
-            // repeat the last one; their results are never stored.
-            uint4 qreg[KS_C + KS_R];
-            {
-                const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + min(head, p.n_heads - 1);
-                const uint4 *qa = reinterpret_cast<const uint4 *>(p.q_absorb + rh * C) + gi;
-                const uint4 *qq = reinterpret_cast<const uint4 *>(p.qr + rh * R) + gi;
-#pragma unroll
-                for (int ks = 0; ks < KS_C; ks++) {
-                    qreg[ks] = qa[4 * ks];
-                }
-#pragma unroll
-                for (int ks = 0; ks < KS_R; ks++) {
-                    qreg[KS_C + ks] = qq[4 * ks];
-                }
-                // the loads must have landed before the loop: a wait for them inside it would also wait for
-                // the cache copies in flight
-#pragma unroll
-                for (int ks = 0; ks < KS_C + KS_R; ks++) {
-                    asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
-                }
+            if (h0 != 0) {
+                load_q(h0);
             }
             f32x4_t O[DT];
 #pragma unroll
@@ -440,6 +440,14 @@ mla_decode_kernel(const MlaDecodeParams p)
             for (int i = 0; i < kDepth; i++) {
                 issue(min(static_cast<uint32_t>(i), last));
             }
+            // The query loads were issued before these copies and complete before them (memory operations finish
+            // in order); their latency overlaps the copies'. They must have landed before the loop: a wait for
+            // them inside it would also wait for the cache copies in flight. The wait the compiler places here
+            // counts the copies too, so it errs on the late side.
+#pragma unroll
+            for (int ks = 0; ks < KS_C + KS_R; ks++) {
+                asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+            }
             f32x4_t S[2];
             for (uint32_t it = 0; it < n_steps; it++) {
                 {
@@ -498,18 +506,28 @@ mla_decode_kernel(const MlaDecodeParams p)
         __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
     };
 
-    // ---- the work list. Every query row owns ceil(limit / 32) steps; the rows' steps, laid end to end, are
-    // cut into chunks of equal length, one chunk per workgroup (more when a chunk would not fit the block
-    // table staging), so that ragged batches keep every compute unit equally busy. A chunk that crosses a
-    // row boundary is processed as several segments. Only a chunk's first and last segment can be parts of
-    // rows that continue in other chunks: chunk c owns the partial slots 2c (its first segment) and 2c + 1
-    // (its last, when that is another one), and a row cut into n segments starting in chunk c0 finds them at
-    // 2 c0 (+ 1 unless it is that chunk's first segment), 2 (c0 + 1), 2 (c0 + 2), ...
+    // ---- the work list. Every query row owns ceil(limit / 32) steps.
+    // Few rows (at most 64: a decode batch with several workgroups per row): every row is cut into chunks of its
+    // own, so that no workgroup pays the set-up of a segment (query load, pipeline fill, partial store) twice.
+    // With G workgroups the chunk bound is the smallest L for which sum ceil(n_t / L) <= G; row t then gets
+    // ceil(n_t / L) chunks of equal length. Everything lives in the lanes of a wave (lane = row), every wave
+    // computing the same.
+    // Many rows: the rows' steps, laid end to end, are cut into chunks of equal length, one chunk per workgroup
+    // (more when a chunk would not fit the block table staging); a chunk that crosses a row boundary is
+    // processed as several segments.
+    // Either way only a chunk's first and last segment can be parts of rows that continue in other chunks:
+    // chunk c owns the partial slots 2c (its first segment) and 2c + 1 (its last, when that is another one), and
+    // a row cut into n segments starting in chunk c0 finds them at 2 c0 (+ 1 unless it is that chunk's first
+    // segment), 2 (c0 + 1), 2 (c0 + 2), ...
     __shared__ uint32_t scan_ws[kWaves];
     __shared__ uint32_t found[4];
     const uint32_t B = p.batch, T = p.total_rows;
-    // the sequence that owns query row t (query_start_loc is a prefix sum), or B
+    // the sequence that owns query row t (query_start_loc is a prefix sum), or B. A batch of one row per
+    // sequence answers with one round of loads.
     auto seq_of = [&](uint32_t t) {
+        if (t < B && p.query_start_loc[t] == static_cast<int32_t>(t) && p.lens[t] == 1) {
+            return t;
+        }
         uint32_t lo = 0, hi = B;
         while (lo < hi) {
             const uint32_t mid = (lo + hi) / 2;
@@ -544,6 +562,79 @@ mla_decode_kernel(const MlaDecodeParams p)
         const uint32_t causal = row_causal(t, seq);
         return LISTS && causal > p.top_k ? p.top_k : causal;
     };
+    uint32_t chunk_cap = (kTblCap - 2) * p.block_size / kStep;
+    if (LISTS) {
+        chunk_cap = min(chunk_cap, static_cast<uint32_t>(kTblCap / kStep));   // a listed row stages one entry per position
+    }
+
+    if (T <= 64) {
+        uint32_t my_seq = B, my_causal = 0, my_limit = 0, my_n = 0;
+        if (lane < T) {
+            my_seq = seq_of(lane);
+            my_causal = row_causal(lane, my_seq);
+            my_limit = LISTS && my_causal > p.top_k ? p.top_k : my_causal;
+            my_n = ceil_div(my_limit, static_cast<uint32_t>(kStep));
+            if (my_n == 0 && blockIdx.x == 0 && wave == 0) {
+                reinterpret_cast<int4 *>(p.part_meta)[lane] = make_int4(0, 0, 0, 0);   // a row without keys: nothing to merge
+            }
+        }
+        auto wave_sum = [&](uint32_t v) {
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                v += __shfl_xor(v, d);
+            }
+            return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+        };
+        const uint32_t total = wave_sum(my_n);
+        if (total == 0) {
+            return;
+        }
+        // the smallest chunk bound that needs no more chunks than there are workgroups
+        uint32_t bound = max(ceil_div(total, gridDim.x), p.chunk_min_steps);
+        uint32_t my_k = 0, n_chunks = 0;
+        bool fits = false;
+        for (uint32_t tries = 0; tries < 24 && bound <= chunk_cap; tries++, bound++) {
+            my_k = ceil_div(my_n, bound);
+            n_chunks = wave_sum(my_k);
+            if (n_chunks <= gridDim.x) {
+                fits = true;
+                break;
+            }
+        }
+        if (fits) {
+            const uint32_t c = blockIdx.x;
+            if (c >= n_chunks) {
+                return;
+            }
+            uint32_t incl = my_k;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(incl, d);
+                incl += lane >= static_cast<uint32_t>(d) ? up : 0u;
+            }
+            const uint32_t my_base = incl - my_k;   // first chunk of the lane's row
+            const uint32_t row = static_cast<uint32_t>(__builtin_popcountll(__ballot(my_base <= c && lane < T))) - 1;
+            // rows without steps share their base with the next row: the last row whose base is <= c owns the
+            // chunk only if it has chunks, and a row with steps after such rows has the larger lane index
+            const uint32_t r_seq = __builtin_amdgcn_readfirstlane(__shfl(my_seq, static_cast<int>(row)));
+            const uint32_t r_causal = __builtin_amdgcn_readfirstlane(__shfl(my_causal, static_cast<int>(row)));
+            const uint32_t r_limit = __builtin_amdgcn_readfirstlane(__shfl(my_limit, static_cast<int>(row)));
+            const uint32_t r_n = __builtin_amdgcn_readfirstlane(__shfl(my_n, static_cast<int>(row)));
+            const uint32_t r_k = __builtin_amdgcn_readfirstlane(__shfl(my_k, static_cast<int>(row)));
+            const uint32_t r_base = __builtin_amdgcn_readfirstlane(__shfl(my_base, static_cast<int>(row)));
+            const uint32_t len = ceil_div(r_n, r_k);          // equal chunks inside the row, none above the bound
+            const uint32_t n_slots = ceil_div(r_n, len);      // the chunks that are not empty
+            const uint32_t j = c - r_base;
+            if (j >= n_slots) {
+                return;
+            }
+            const int4 meta = make_int4(n_slots > 1 ? static_cast<int>(n_slots) : 0, static_cast<int>(r_base), 1, 0);
+            run_segment(r_seq, row, r_limit, r_causal, j * len, min(r_n, (j + 1) * len), n_slots, 2 * c, meta);
+            return;
+        }
+        // no bound within reach (rows far longer than the staging allows): the general split below
+    }
+
     for (uint32_t c = blockIdx.x;; c += gridDim.x) {
         // block-wide prefix sums of the rows' step counts (redone for every chunk: nothing of it stays in
         // registers while a segment runs)
@@ -583,10 +674,7 @@ mla_decode_kernel(const MlaDecodeParams p)
         }
         total = __builtin_amdgcn_readfirstlane(total);
         uint32_t chunk = max(ceil_div(total, gridDim.x), p.chunk_min_steps);
-        chunk = min(chunk, (kTblCap - 2) * p.block_size / kStep);
-        if (LISTS) {
-            chunk = min(chunk, static_cast<uint32_t>(kTblCap / kStep));   // a listed row stages one entry per position
-        }
+        chunk = min(chunk, chunk_cap);
         if (c >= ceil_div(total, chunk)) {
             return;
         }
