@@ -8,7 +8,8 @@ Tensors are borrowed for the call and results are written in place, as in the re
   * contiguity, device and dtype are checked and raise RuntimeError (the reference assumes them);
   * kernels run on torch's current HIP stream; the call blocks until they finish unless
     `Runtime.blocking` is set to False (the reference always synchronises, _C.cpp:1182);
-  * `attention` accepts keyword-only `k_scale` / `v_scale` for an int8 KV cache.
+  * `attention` and `rope_and_cache` accept keyword-only `k_scale` / `v_scale` for a quantised KV cache
+    (int8 or float8_e4m3fn, one fp32 scale per token and kv head).
 PyTorch is used only to own device memory and streams.
 """
 from __future__ import annotations
@@ -21,6 +22,8 @@ import torch
 from . import _lib
 
 _DT = {torch.float16: 0, torch.bfloat16: 1}
+# element types of a quantised KV cache (one byte per element, fp32 scale per token and kv head)
+_KV_DT = {torch.int8: 1, torch.float8_e4m3fn: 2}
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -173,15 +176,18 @@ def rope_and_cache(rt: Runtime, inout: torch.Tensor, k_cache: torch.Tensor, v_ca
                    v_scale: Optional[torch.Tensor] = None) -> None:
     """RoPE in place on the fused q|k|v rows and the write of K and V into the paged caches
     (xlite/_C.pyi:1251-1290). Extension (keyword-only): with `k_scale` and `v_scale`
-    [num_blocks, block_size, n_kv_heads] fp32 the caches are int8 and the rows are quantised as they are
-    written (scale = absmax / 127 per token and kv head)."""
+    [num_blocks, block_size, n_kv_heads] fp32 the caches are int8 or float8_e4m3fn and the rows are quantised as
+    they are written (scale = absmax / 127, or absmax / 448, per token and kv head)."""
     if not is_neox:
         raise RuntimeError("rope_and_cache: unsupported rope type gptj")
     int8 = k_scale is not None or v_scale is not None
     for n, t in (("inout", inout), ("cosin", cosin)):
         _dev(n, t)
     for n, t in (("k_cache", k_cache), ("v_cache", v_cache)):
-        _dev(n, t, torch.int8 if int8 else None)
+        _dev(n, t)
+    if int8:
+        _req(k_cache.dtype in _KV_DT and v_cache.dtype == k_cache.dtype,
+             "rope_and_cache: scales given but the caches are neither int8 nor float8_e4m3fn")
     _dev("position", position, torch.int64)
     _dev("slot_mapping", slot_mapping, torch.int32)
     dt = _act_dtype("rope_and_cache", inout, cosin) if int8 else _act_dtype("rope_and_cache", inout, k_cache, v_cache, cosin)
@@ -198,10 +204,10 @@ def rope_and_cache(rt: Runtime, inout: torch.Tensor, k_cache: torch.Tensor, v_ca
         for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
             _dev(n, t, torch.float32)
             _req(t.numel() * head_dim == k_cache.numel(), "rope_and_cache: %s shape mismatch" % n)
-        _lib.check(rt._lib.xlite_hip_rope_and_cache_int8(
+        _lib.check(rt._lib.xlite_hip_rope_and_cache_quant(
             rt.stream(), _ptr(inout), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(position),
             _ptr(cosin), _ptr(slot_mapping), T, n_heads, n_kv_heads, head_dim, rot_dim, block_size, 1, mrope_mask_h,
-            mrope_mask_w, dt))
+            mrope_mask_w, dt, _KV_DT[k_cache.dtype]))
     else:
         _lib.check(rt._lib.xlite_hip_rope_and_cache(
             rt.stream(), _ptr(inout), _ptr(k_cache), _ptr(v_cache), _ptr(position), _ptr(cosin), _ptr(slot_mapping),
@@ -229,8 +235,8 @@ def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
         _req(k_scale is not None and v_scale is not None, "attention: k_scale and v_scale go together")
         _dev("k_scale", k_scale, torch.float32)
         _dev("v_scale", v_scale, torch.float32)
-        _req(k_cache.dtype == torch.int8 and v_cache.dtype == torch.int8,
-             "attention: scales given but the caches are not int8")
+        _req(k_cache.dtype in _KV_DT and v_cache.dtype == k_cache.dtype,
+             "attention: scales given but the caches are neither int8 nor float8_e4m3fn")
         _req(k_scale.numel() * head_dim == k_cache.numel() and v_scale.numel() * head_dim == v_cache.numel(),
              "attention: one scale per (block, slot, kv head) expected")
     else:
@@ -242,12 +248,14 @@ def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     _req(output.numel() == T * n_heads * head_dim, "attention: output shape mismatch")
     _req(min(query_start_loc.numel(), lens.numel(), cached_lens.numel()) >= batch, "attention: metadata shorter than batch")
     _req(block_tables.numel() >= batch * max_num_block, "attention: block_tables shorter than batch * max_num_block")
-    need = rt._lib.xlite_hip_attention_workspace_bytes(T, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block)
+    kv = _KV_DT[k_cache.dtype] if int8 else 0
+    need = rt._lib.xlite_hip_attention_workspace_bytes_kv(T, n_heads, n_kv_heads, head_dim, block_size, batch,
+                                                          max_num_block, kv)
     ws = rt.workspace(need)
     _lib.check(rt._lib.xlite_hip_attention(
         rt.stream(), _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(output), _ptr(query_start_loc), _ptr(lens),
         _ptr(cached_lens), _ptr(block_tables), T, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
-        dt, 1 if int8 else 0, _ptr(k_scale), _ptr(v_scale), _ptr(ws), ws.numel()))
+        dt, kv, _ptr(k_scale), _ptr(v_scale), _ptr(ws), ws.numel()))
     rt.finish()
 
 
@@ -596,15 +604,20 @@ def get_tile_size_of_cached_kv(cached_lens: List[int], query_lens: List[int], he
     return rc
 
 
-def quantize_kv_int8(rt: Runtime, x: torch.Tensor):
-    """x [..., head_dim] (fp16/bf16) -> (int8 tensor of the same shape, fp32 scales [...]).
-    Not part of the reference API (its caches are never quantised)."""
+def quantize_kv(rt: Runtime, x: torch.Tensor, kv_dtype: torch.dtype = torch.int8):
+    """x [..., head_dim] (fp16/bf16) -> (tensor of `kv_dtype` - int8 or float8_e4m3fn - of the same shape, fp32
+    scales [...]). Not part of the reference API (its caches are never quantised)."""
     _dev("x", x)
-    dt = _act_dtype("quantize_kv_int8", x)
+    dt = _act_dtype("quantize_kv", x)
+    _req(kv_dtype in _KV_DT, "quantize_kv: kv_dtype must be int8 or float8_e4m3fn")
     d = x.shape[-1]
     rows = x.numel() // d
-    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    q = torch.empty(x.shape, dtype=kv_dtype, device=x.device)
     s = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
-    _lib.check(rt._lib.xlite_hip_quantize_kv_int8(rt.stream(), _ptr(x), _ptr(q), _ptr(s), rows, d, dt))
+    _lib.check(rt._lib.xlite_hip_quantize_kv(rt.stream(), _ptr(x), _ptr(q), _ptr(s), rows, d, dt, _KV_DT[kv_dtype]))
     rt.finish()
     return q, s
+
+
+def quantize_kv_int8(rt: Runtime, x: torch.Tensor):
+    return quantize_kv(rt, x, torch.int8)

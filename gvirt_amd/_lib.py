@@ -16,6 +16,7 @@ SIGNATURES = {
     "xlite_hip_device_info": (_i32, [_i32, _vp, _vp, _vp, _sz]),
     "xlite_hip_rope_and_cache": (_i32, [_vp] * 7 + [_u32] * 6 + [_i32, _u64, _u64, _i32]),
     "xlite_hip_attention_workspace_bytes": (_sz, [_u32] * 7),
+    "xlite_hip_attention_workspace_bytes_kv": (_sz, [_u32] * 7 + [_i32]),
     "xlite_hip_attention": (_i32, [_vp] * 9 + [_u32] * 7 + [_i32, _i32, _vp, _vp, _vp, _sz]),
     "xlite_hip_attention_noalloc_scratch_bytes": (_sz, []),
     "xlite_hip_attention_noalloc": (_i32, [_vp] * 9 + [_u32] * 7 + [_i32, _i32, _vp, _vp]),
@@ -28,7 +29,9 @@ SIGNATURES = {
     "xlite_hip_einsum_mht_mhd": (_i32, [_vp] * 4 + [_u32] * 5 + [_i32, _i32]),
     "xlite_hip_get_tile_size_of_cached_kv": (_i32, [_vp, _vp] + [_u32] * 5),
     "xlite_hip_prepare_attn": (_i32, [_vp, _vp, _u32, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp]),
+    "xlite_hip_quantize_kv": (_i32, [_vp] * 4 + [_u64, _u32, _i32, _i32]),
     "xlite_hip_quantize_kv_int8": (_i32, [_vp] * 4 + [_u64, _u32, _i32]),
+    "xlite_hip_rope_and_cache_quant": (_i32, [_vp] * 9 + [_u32] * 6 + [_i32, _u64, _u64, _i32, _i32]),
     "xlite_hip_rope_and_cache_int8": (_i32, [_vp] * 9 + [_u32] * 6 + [_i32, _u64, _u64, _i32]),
     "xlite_hip_qk_rms_norm": (_i32, [_vp] * 7 + [_u32] * 7 + [_f32, _i32]),
     "xlite_hip_indexer_scores": (_i32, [_vp] * 9 + [_u32] * 6 + [_i32]),

@@ -16,14 +16,12 @@ bool is_decode_batch(uint32_t total_tokens, uint32_t batch)
 
 }  // namespace
 
-extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
-                                                      uint32_t n_kv_heads, uint32_t head_dim,
-                                                      uint32_t block_size, uint32_t batch,
-                                                      uint32_t max_num_block)
+namespace {
+
+// scratch of a batch over 16-bit caches
+size_t workspace_bytes_16(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                          uint32_t block_size, uint32_t batch, uint32_t max_num_block)
 {
-    if (total_tokens == 0 || batch == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || head_dim < 8) {
-        return 0;
-    }
     const uint32_t max_ctx = max_num_block * block_size;
     if (is_decode_batch(total_tokens, batch)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
@@ -42,6 +40,45 @@ extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uin
                     prefill_mfma_workspace_bytes(total_tokens, n_heads, n_kv_heads, head_dim, batch, max_ctx));
 }
 
+// A quantised cache is read directly by the streaming decode kernel (and, int8 only, by the vector decode
+// kernel); every other batch goes through a 16-bit copy of its blocks.
+bool quantised_direct(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
+                      uint32_t batch, int kv_dtype)
+{
+    if (!is_decode_batch(total_tokens, batch)) {
+        return false;
+    }
+    return decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens) ||
+           (kv_dtype == XLITE_HIP_KV_INT8 && decode_supported(head_dim));
+}
+
+}  // namespace
+
+extern "C" size_t xlite_hip_attention_workspace_bytes_kv(uint32_t total_tokens, uint32_t n_heads,
+                                                         uint32_t n_kv_heads, uint32_t head_dim,
+                                                         uint32_t block_size, uint32_t batch,
+                                                         uint32_t max_num_block, int kv_dtype)
+{
+    if (total_tokens == 0 || batch == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || head_dim < 8) {
+        return 0;
+    }
+    size_t need = workspace_bytes_16(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block);
+    if (kv_dtype != XLITE_HIP_KV_SAME &&
+        !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
+        need += kv_dequant_bytes(n_kv_heads, head_dim, block_size, batch, max_num_block);
+    }
+    return need;
+}
+
+extern "C" size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
+                                                      uint32_t n_kv_heads, uint32_t head_dim,
+                                                      uint32_t block_size, uint32_t batch,
+                                                      uint32_t max_num_block)
+{
+    return xlite_hip_attention_workspace_bytes_kv(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch,
+                                                  max_num_block, XLITE_HIP_KV_SAME);
+}
+
 extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache,
                                    const void *v_cache, void *output,
                                    const int32_t *query_start_loc, const int32_t *lens,
@@ -53,7 +90,8 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
                                    size_t workspace_bytes)
 {
     XL_REQUIRE(dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16, "qkv/kCache/vCache/output dtype unsupported!");
-    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || kv_dtype == XLITE_HIP_KV_INT8, "kv cache dtype unsupported!");
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || kv_dtype == XLITE_HIP_KV_INT8 || kv_dtype == XLITE_HIP_KV_FP8,
+               "kv cache dtype unsupported!");
     if (batch == 0 || total_tokens == 0) {
         return XLITE_HIP_OK;
     }
@@ -62,11 +100,18 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
     XL_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "n_heads must be a positive multiple of n_kv_heads");
     XL_REQUIRE(block_size > 0 && max_num_block > 0, "block_size and max_num_block must be positive");
-    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || (k_scale && v_scale), "int8 KV cache needs k_scale and v_scale");
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME || (k_scale && v_scale), "a quantised KV cache needs k_scale and v_scale");
     AttentionArgs a{qkv, k_cache, v_cache, output, query_start_loc, lens, cached_lens, block_tables,
                     total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
                     dtype, kv_dtype, k_scale, v_scale, workspace, workspace_bytes};
     hipStream_t s = as_stream(stream);
+    if (kv_dtype != XLITE_HIP_KV_SAME &&
+        !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
+        XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");
+        if (const int rc = launch_kv_dequant(s, &a)) {   // from here on: 16-bit caches in the workspace
+            return rc;
+        }
+    }
     if (is_decode_batch(total_tokens, batch)) {
         XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
@@ -74,7 +119,7 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         }
         // more than 16 query heads per kv head, or a block size that is not a multiple of 16: the prefill
         // kernel takes the rows of a sequence as one (ragged) M tile and splits the KV range
-        if (kv_dtype == XLITE_HIP_KV_SAME && prefill_mfma_supported(a)) {
+        if (a.kv_dtype == XLITE_HIP_KV_SAME && prefill_mfma_supported(a)) {
             return launch_prefill_mfma(s, a);
         }
         // head_dim 64 or block sizes that are not a multiple of 4 at such shapes, int8 caches with wide groups
@@ -84,8 +129,8 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         // shrink the split count to what the caller's workspace can hold
         const uint32_t max_ctx = max_num_block * block_size;
         while (ceil_div(max_ctx, tile) > 1 &&
-               (workspace == nullptr ||
-                decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile)) > workspace_bytes)) {
+               (a.workspace == nullptr ||
+                decode_workspace_bytes(total_tokens, n_heads, head_dim, ceil_div(max_ctx, tile)) > a.workspace_bytes)) {
             tile *= 2;
         }
         int rc = launch_decode(s, a, tile);
@@ -95,7 +140,6 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         XL_LAUNCH_CHECK();
         return XLITE_HIP_OK;
     }
-    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_SAME, "the int8 KV cache is supported for decode batches only");
     XL_REQUIRE(mfma_gqa_supported(head_dim), "head_dim must be 64 or 128");
     if (prefill_mfma_supported(a)) {
         return launch_prefill_mfma(s, a);

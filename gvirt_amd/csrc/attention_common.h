@@ -119,6 +119,10 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a);
 size_t prefill_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                     uint32_t batch, uint32_t max_ctx);
 
+// kv_dequant.hip: the 16-bit copy of a quantised cache's visible blocks, at the front of the workspace
+size_t kv_dequant_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size, uint32_t batch, uint32_t max_num_block);
+int launch_kv_dequant(hipStream_t stream, AttentionArgs *a);
+
 // mla_topk.hip
 size_t mla_topk_scratch_bytes(uint32_t total_tokens, uint32_t kv_lora_rank, uint32_t rope_head_dim, uint32_t top_k);
 int launch_mla_topk(hipStream_t stream, const MlaArgs &a);

@@ -50,8 +50,8 @@ extern "C" int xlite_hip_attention_noalloc(void *stream, const void *qkv, const 
     if (batch == 0 || total_tokens == 0) {
         return XLITE_HIP_OK;
     }
-    const size_t need = xlite_hip_attention_workspace_bytes(total_tokens, n_heads, n_kv_heads, head_dim, block_size,
-                                                            batch, max_num_block);
+    const size_t need = xlite_hip_attention_workspace_bytes_kv(total_tokens, n_heads, n_kv_heads, head_dim, block_size,
+                                                               batch, max_num_block, kv_dtype);
     if (need > XLITE_HIP_NOALLOC_SCRATCH_BYTES) {
         return fail(XLITE_HIP_ENOSPC, __func__,
                     "this shape needs " + std::to_string(need) + " bytes of scratch, the built-in buffer holds " +

@@ -11,6 +11,54 @@ union Vec16 {
     uint32_t w[4];
 };
 
+// One chunk pair of a q or k head: elements e0 .. e0+7 of the rotary span's first half (`a`) with their partners
+// in the second half (`b`), rotated in place; q is then scaled. Rounding follows calc_cossin_cast
+// (xlite/csrc/kernels/rope_and_cache.h:93-129): each product is rounded to the storage type, the difference /
+// sum is formed in fp32 and rounded again; the q scale is applied in fp32 and rounded once more (:576-586).
+template <typename T>
+__device__ __forceinline__ void rotate_chunk_pair(Vec16 &a, Vec16 &b, uint32_t e0, uint32_t half, uint32_t t,
+                                                  uint32_t num_tokens, uint32_t rot_dim, const int64_t *position,
+                                                  const uint16_t *cosin, uint64_t mask_h, uint64_t mask_w, bool is_q,
+                                                  float q_scale)
+{
+    Vec16 c, s;
+    if ((mask_h | mask_w) == 0) {
+        const uint16_t *cs = cosin + static_cast<uint64_t>(position[t]) * rot_dim;
+        c.v = *reinterpret_cast<const uint4 *>(cs + e0);
+        s.v = *reinterpret_cast<const uint4 *>(cs + half + e0);
+    } else {
+        // lane j of the rotary half takes its angle from the height / width position
+        // when bit j of the matching mask is set, else from the temporal position
+        const uint16_t *cs_t = cosin + static_cast<uint64_t>(position[t]) * rot_dim;
+        const uint16_t *cs_h = cosin + static_cast<uint64_t>(position[num_tokens + t]) * rot_dim;
+        const uint16_t *cs_w = cosin + static_cast<uint64_t>(position[2ull * num_tokens + t]) * rot_dim;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t lane = e0 + j;
+            const uint16_t *src = ((mask_h >> lane) & 1) ? cs_h : ((mask_w >> lane) & 1) ? cs_w : cs_t;
+            c.h[j] = src[lane];
+            s.h[j] = src[half + lane];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float x1 = T::to_f32(a.h[j]), x2 = T::to_f32(b.h[j]);
+        const float cc = T::to_f32(c.h[j]), ss = T::to_f32(s.h[j]);
+        const float p1 = T::to_f32(T::from_f32(x1 * cc));
+        const float p2 = T::to_f32(T::from_f32(x2 * ss));
+        const float p3 = T::to_f32(T::from_f32(x2 * cc));
+        const float p4 = T::to_f32(T::from_f32(x1 * ss));
+        uint16_t o1 = T::from_f32(p1 - p2);
+        uint16_t o2 = T::from_f32(p3 + p4);
+        if (is_q) {
+            o1 = T::from_f32(T::to_f32(o1) * q_scale);
+            o2 = T::from_f32(T::to_f32(o2) * q_scale);
+        }
+        a.h[j] = o1;
+        b.h[j] = o2;
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // rope_and_cache (xlite/csrc/kernels/rope_and_cache.h:206-610)
 // One item = one (token, head slot, chunk pair): a thread rotates 8 elements of the first
@@ -36,7 +84,6 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
     const uint32_t items_per_token = slots * items_per_head;
     const uint64_t total = static_cast<uint64_t>(num_tokens) * items_per_token;
     const uint32_t half = rot_dim / 2;
-    const bool mrope = (mask_h | mask_w) != 0;
 
     for (uint64_t idx = blockIdx.x * static_cast<uint64_t>(blockDim.x) + threadIdx.x; idx < total;
          idx += static_cast<uint64_t>(gridDim.x) * blockDim.x) {
@@ -64,46 +111,7 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
             a.v = *reinterpret_cast<const uint4 *>(row + e0);
             b.v = *reinterpret_cast<const uint4 *>(row + e0 + half);
             if (is_q || is_k) {
-                Vec16 c, s;
-                if (!mrope) {
-                    const uint16_t *cs = cosin + static_cast<uint64_t>(position[t]) * rot_dim;
-                    c.v = *reinterpret_cast<const uint4 *>(cs + e0);
-                    s.v = *reinterpret_cast<const uint4 *>(cs + half + e0);
-                } else {
-                    // lane j of the rotary half takes its angle from the height / width position
-                    // when bit j of the matching mask is set, else from the temporal position
-                    const uint16_t *cs_t = cosin + static_cast<uint64_t>(position[t]) * rot_dim;
-                    const uint16_t *cs_h =
-                        cosin + static_cast<uint64_t>(position[num_tokens + t]) * rot_dim;
-                    const uint16_t *cs_w =
-                        cosin + static_cast<uint64_t>(position[2ull * num_tokens + t]) * rot_dim;
-#pragma unroll
-                    for (int j = 0; j < 8; j++) {
-                        const uint32_t lane = e0 + j;
-                        const uint16_t *src = ((mask_h >> lane) & 1) ? cs_h
-                                              : ((mask_w >> lane) & 1) ? cs_w
-                                                                       : cs_t;
-                        c.h[j] = src[lane];
-                        s.h[j] = src[half + lane];
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const float x1 = T::to_f32(a.h[j]), x2 = T::to_f32(b.h[j]);
-                    const float cc = T::to_f32(c.h[j]), ss = T::to_f32(s.h[j]);
-                    const float p1 = T::to_f32(T::from_f32(x1 * cc));
-                    const float p2 = T::to_f32(T::from_f32(x2 * ss));
-                    const float p3 = T::to_f32(T::from_f32(x2 * cc));
-                    const float p4 = T::to_f32(T::from_f32(x1 * ss));
-                    uint16_t o1 = T::from_f32(p1 - p2);
-                    uint16_t o2 = T::from_f32(p3 + p4);
-                    if (is_q) {
-                        o1 = T::from_f32(T::to_f32(o1) * q_scale);
-                        o2 = T::from_f32(T::to_f32(o2) * q_scale);
-                    }
-                    a.h[j] = o1;
-                    b.h[j] = o2;
-                }
+                rotate_chunk_pair<T>(a, b, e0, half, t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
                 *reinterpret_cast<uint4 *>(row + e0) = a.v;
                 *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
             }
@@ -342,50 +350,119 @@ qk_rms_norm_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, 
     }
 }
 
-// one row by the 16 lanes of a group
+// ---------------------------------------------------------------------------------------
+// Quantised KV caches (no counterpart in the reference): one fp32 scale per (token, kv head) row,
+//   int8:      scale = absmax / 127, q = clamp(rint(x / scale), -127, 127)
+//   fp8 e4m3:  scale = absmax / 448, q = e4m3(x / scale) (round to nearest even; 448 is the format's maximum)
+// and x^ = q * scale. A row of zeros has scale 0 and is divided by 1 instead.
+// ---------------------------------------------------------------------------------------
+template <int KV>
+struct QuantFmt;
+template <>
+struct QuantFmt<XLITE_HIP_KV_INT8> {
+    static constexpr float kMax = 127.0f;
+    // eight quotients -> eight bytes
+    static __device__ __forceinline__ uint2 pack8(const float (&y)[8])
+    {
+        uint32_t w[2] = {0, 0};
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float q = fminf(fmaxf(rintf(y[j]), -127.f), 127.f);
+            w[j / 4] |= (static_cast<uint32_t>(static_cast<int32_t>(q)) & 0xffu) << (8 * (j % 4));
+        }
+        return make_uint2(w[0], w[1]);
+    }
+};
+template <>
+struct QuantFmt<XLITE_HIP_KV_FP8> {
+    static constexpr float kMax = 448.0f;
+    static __device__ __forceinline__ uint2 pack8(const float (&y)[8])
+    {
+        int w0 = 0, w1 = 0;
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], w0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], w1, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+        return make_uint2(static_cast<uint32_t>(w0), static_cast<uint32_t>(w1));
+    }
+};
+
 template <typename T>
-__device__ __forceinline__ void quantize_row(const uint16_t *x, int8_t *dst, float *scale_out, uint32_t head_dim,
+__device__ __forceinline__ float chunk_absmax(const Vec16 &a)
+{
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        m = fmaxf(m, fabsf(T::to_f32(a.h[j])));
+    }
+    return m;
+}
+
+template <typename T, int KV>
+__device__ __forceinline__ uint2 quantize_chunk(const Vec16 &a, float safe)
+{
+    float y[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        y[j] = T::to_f32(a.h[j]) / safe;
+    }
+    return QuantFmt<KV>::pack8(y);
+}
+
+// max over the 16 lanes of a group
+__device__ __forceinline__ float group16_max(float m)
+{
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) {
+        m = fmaxf(m, __shfl_xor(m, o));
+    }
+    return m;
+}
+
+// one row (head_dim a multiple of 8) by the 16 lanes of a group, a 16-byte chunk per lane and turn
+template <typename T, int KV>
+__device__ __forceinline__ void quantize_row(const uint16_t *x, unsigned char *dst, float *scale_out, uint32_t head_dim,
                                              uint32_t lane)
 {
     float amax = 0.f;
-    for (uint32_t i = lane; i < head_dim; i += 16) {
-        amax = fmaxf(amax, fabsf(T::to_f32(x[i])));
+    for (uint32_t c = lane; c < head_dim / 8; c += 16) {
+        Vec16 a;
+        a.v = *reinterpret_cast<const uint4 *>(x + c * 8);
+        amax = fmaxf(amax, chunk_absmax<T>(a));
     }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) {
-        amax = fmaxf(amax, __shfl_xor(amax, o));
-    }
-    const float scale = amax / 127.0f;
+    amax = group16_max(amax);
+    const float scale = amax / QuantFmt<KV>::kMax;
     const float safe = scale > 0.f ? scale : 1.0f;
-    for (uint32_t i = lane; i < head_dim; i += 16) {
-        float q = rintf(T::to_f32(x[i]) / safe);
-        q = fminf(fmaxf(q, -127.f), 127.f);
-        dst[i] = static_cast<int8_t>(q);
+    for (uint32_t c = lane; c < head_dim / 8; c += 16) {
+        Vec16 a;
+        a.v = *reinterpret_cast<const uint4 *>(x + c * 8);
+        *reinterpret_cast<uint2 *>(dst + c * 8) = quantize_chunk<T, KV>(a, safe);
     }
     if (lane == 0) {
         *scale_out = scale;
     }
 }
 
-template <typename T>
+template <typename T, int KV>
 __global__ void __launch_bounds__(256)
-quantize_kv_kernel(const uint16_t *__restrict__ src, int8_t *__restrict__ dst,
+quantize_kv_kernel(const uint16_t *__restrict__ src, unsigned char *__restrict__ dst,
                    float *__restrict__ scales, uint64_t rows, uint32_t head_dim)
 {
     const uint32_t group = threadIdx.x / 16, lane = threadIdx.x % 16;
     const uint32_t groups = blockDim.x / 16;
     for (uint64_t r = blockIdx.x * static_cast<uint64_t>(groups) + group; r < rows;
          r += static_cast<uint64_t>(gridDim.x) * groups) {
-        quantize_row<T>(src + r * head_dim, dst + r * head_dim, scales + r, head_dim, lane);
+        quantize_row<T, KV>(src + r * head_dim, dst + r * head_dim, scales + r, head_dim, lane);
     }
 }
 
-// The K (already rotated) and V rows of the fused activation rows, quantised into the int8 caches at the
-// tokens' slots: row r = (token, K | V, kv head).
-template <typename T>
+// The K (already rotated) and V rows of the fused activation rows, quantised into the caches at the
+// tokens' slots: row r = (token, K | V, kv head). The second launch of the two-launch form, for head shapes the
+// fused kernel below does not take.
+template <typename T, int KV>
 __global__ void __launch_bounds__(256)
-quantize_to_cache_kernel(const uint16_t *__restrict__ inout, int8_t *__restrict__ k_cache,
-                         int8_t *__restrict__ v_cache, float *__restrict__ k_scale, float *__restrict__ v_scale,
+quantize_to_cache_kernel(const uint16_t *__restrict__ inout, unsigned char *__restrict__ k_cache,
+                         unsigned char *__restrict__ v_cache, float *__restrict__ k_scale, float *__restrict__ v_scale,
                          const int32_t *__restrict__ slot_mapping, uint32_t num_tokens, uint32_t n_heads,
                          uint32_t n_kv_heads, uint32_t head_dim)
 {
@@ -401,7 +478,80 @@ quantize_to_cache_kernel(const uint16_t *__restrict__ inout, int8_t *__restrict_
         const uint32_t kvh = is_v ? rem - n_kv_heads : rem;
         const uint16_t *x = inout + (static_cast<uint64_t>(t) * slots + n_heads + rem) * head_dim;
         const uint64_t row = static_cast<uint64_t>(static_cast<uint32_t>(slot_mapping[t])) * n_kv_heads + kvh;
-        quantize_row<T>(x, (is_v ? v_cache : k_cache) + row * head_dim, (is_v ? v_scale : k_scale) + row, head_dim, lane);
+        quantize_row<T, KV>(x, (is_v ? v_cache : k_cache) + row * head_dim, (is_v ? v_scale : k_scale) + row, head_dim, lane);
+    }
+}
+
+// rope_and_cache with the quantisation fused into the write (one launch): a group of 16 lanes owns one
+// (token, head slot), a lane one item of it - a chunk pair of the rotary span or a chunk beyond it - so heads
+// of at most 16 items (head_dim 128 with any rotary span, head_dim 256 fully rotated). q heads are rotated and
+// scaled in place; k heads are rotated in place, v heads left as they are, and both go to the cache as the
+// quantisation of the 16-bit row: the group's lanes agree on the row's absmax by four exchanges.
+template <typename T, int KV>
+__global__ void __launch_bounds__(256)
+rope_quant_cache_kernel(uint16_t *__restrict__ inout, unsigned char *__restrict__ k_cache,
+                        unsigned char *__restrict__ v_cache, float *__restrict__ k_scale, float *__restrict__ v_scale,
+                        const int64_t *__restrict__ position, const uint16_t *__restrict__ cosin,
+                        const int32_t *__restrict__ slot_mapping, uint32_t num_tokens, uint32_t n_heads,
+                        uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim, float q_scale, uint64_t mask_h,
+                        uint64_t mask_w)
+{
+    const uint32_t rot_pairs = rot_dim / 16;
+    const uint32_t items_per_head = head_dim / 8 - rot_pairs;   // <= 16
+    const uint32_t slots = n_heads + 2 * n_kv_heads;
+    const uint32_t half = rot_dim / 2;
+    const uint32_t group = threadIdx.x / 16, lane = threadIdx.x % 16;
+    const uint32_t groups = blockDim.x / 16;
+    const uint64_t total = static_cast<uint64_t>(num_tokens) * slots;
+    // every lane of a group runs the same number of turns: the exchanges below need all sixteen
+    for (uint64_t g = blockIdx.x * static_cast<uint64_t>(groups) + group; g < total;
+         g += static_cast<uint64_t>(gridDim.x) * groups) {
+        const uint32_t t = static_cast<uint32_t>(g / slots);
+        const uint32_t hs = static_cast<uint32_t>(g % slots);
+        uint16_t *row = inout + (static_cast<uint64_t>(t) * slots + hs) * head_dim;
+        const bool is_q = hs < n_heads;
+        const bool is_k = !is_q && hs < n_heads + n_kv_heads;
+        const bool active = lane < items_per_head;
+        const bool rot = active && lane < rot_pairs;
+        const uint32_t e0 = rot ? lane * 8 : (lane + rot_pairs) * 8;
+        Vec16 a, b;
+        a.v = make_uint4(0, 0, 0, 0);
+        b.v = make_uint4(0, 0, 0, 0);
+        if (active) {
+            a.v = *reinterpret_cast<const uint4 *>(row + e0);
+            if (rot) {
+                b.v = *reinterpret_cast<const uint4 *>(row + e0 + half);
+            }
+            if (rot && (is_q || is_k)) {
+                rotate_chunk_pair<T>(a, b, e0, half, t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
+                *reinterpret_cast<uint4 *>(row + e0) = a.v;
+                *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
+            } else if (is_q) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    a.h[j] = T::from_f32(T::to_f32(a.h[j]) * q_scale);
+                }
+                *reinterpret_cast<uint4 *>(row + e0) = a.v;
+            }
+        }
+        if (is_q) {
+            continue;   // uniform inside the group
+        }
+        const float amax = group16_max(fmaxf(chunk_absmax<T>(a), chunk_absmax<T>(b)));
+        const float scale = amax / QuantFmt<KV>::kMax;
+        const float safe = scale > 0.f ? scale : 1.0f;
+        const uint32_t kvh = is_k ? hs - n_heads : hs - n_heads - n_kv_heads;
+        const uint64_t crow = static_cast<uint64_t>(static_cast<uint32_t>(slot_mapping[t])) * n_kv_heads + kvh;
+        unsigned char *dst = (is_k ? k_cache : v_cache) + crow * head_dim;
+        if (active) {
+            *reinterpret_cast<uint2 *>(dst + e0) = quantize_chunk<T, KV>(a, safe);
+            if (rot) {
+                *reinterpret_cast<uint2 *>(dst + e0 + half) = quantize_chunk<T, KV>(b, safe);
+            }
+        }
+        if (lane == 0) {
+            (is_k ? k_scale : v_scale)[crow] = scale;
+        }
     }
 }
 
@@ -416,18 +566,18 @@ static uint32_t grid_for(uint64_t work_threads, uint32_t block)
 
 using namespace xlite;
 
-// Argument checks and launch of the rope kernel; with `with_cache` false the 16-bit caches are not written.
-static int rope_launch(void *stream, void *inout, void *k_cache, void *v_cache, const int64_t *position,
-                       const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads,
-                       uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, int is_neox,
-                       uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, bool with_cache)
+// Argument checks shared by the rope launchers; *q_scale receives the factor applied to q.
+static int rope_check(const void *inout, const int64_t *position, const void *cosin, const int32_t *slot_mapping,
+                      uint32_t num_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim,
+                      uint32_t block_size, int is_neox, uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype,
+                      float *q_scale)
 {
     XL_REQUIRE(is_neox, "unsupported rope type gptj");
     XL_REQUIRE(dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16, "dtype unsupported!");
     if (num_tokens == 0) {
         return XLITE_HIP_OK;
     }
-    XL_REQUIRE(inout && position && cosin && slot_mapping && (!with_cache || (k_cache && v_cache)), "null tensor");
+    XL_REQUIRE(inout && position && cosin && slot_mapping, "null tensor");
     XL_REQUIRE(n_heads > 0 && n_kv_heads > 0 && block_size > 0, "zero head count or block size");
     XL_REQUIRE(head_dim % 8 == 0 && head_dim > 0, "head_dim must be a multiple of 8");
     XL_REQUIRE(rot_dim % 16 == 0 && rot_dim > 0 && rot_dim <= head_dim,
@@ -440,6 +590,25 @@ static int rope_launch(void *stream, void *inout, void *k_cache, void *v_cache, 
         // the fp16 kernel of the reference multiplies by the scale rounded to fp16
         scale = static_cast<float>(static_cast<_Float16>(scale));
     }
+    *q_scale = scale;
+    return XLITE_HIP_OK;
+}
+
+// Launch of the rope kernel; with `with_cache` false the 16-bit caches are not written.
+static int rope_launch(void *stream, void *inout, void *k_cache, void *v_cache, const int64_t *position,
+                       const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads,
+                       uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, int is_neox,
+                       uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, bool with_cache)
+{
+    float scale = 0.f;
+    if (const int rc = rope_check(inout, position, cosin, slot_mapping, num_tokens, n_heads, n_kv_heads, head_dim, rot_dim,
+                                  block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype, &scale)) {
+        return rc;
+    }
+    if (num_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
+    XL_REQUIRE(!with_cache || (k_cache && v_cache), "null tensor");
     const uint64_t items = static_cast<uint64_t>(num_tokens) * (n_heads + 2 * n_kv_heads) *
                            (head_dim / 8 - rot_dim / 16);
     const uint32_t grid = grid_for(items, 256);
@@ -471,6 +640,69 @@ extern "C" int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache
                        head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype, true);
 }
 
+extern "C" int xlite_hip_rope_and_cache_quant(void *stream, void *inout, void *k_cache, void *v_cache,
+                                              float *k_scale, float *v_scale, const int64_t *position,
+                                              const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens,
+                                              uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                              uint32_t rot_dim, uint32_t block_size, int is_neox,
+                                              uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, int kv_dtype)
+{
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_INT8 || kv_dtype == XLITE_HIP_KV_FP8, "kv cache dtype unsupported!");
+    unsigned char *kc = static_cast<unsigned char *>(k_cache), *vc = static_cast<unsigned char *>(v_cache);
+    const bool fused = head_dim % 8 == 0 && rot_dim % 16 == 0 && rot_dim <= head_dim && head_dim / 8 - rot_dim / 16 <= 16;
+    if (!fused) {
+        // wide heads: the rotation first, then a quantising write of the rotated K rows and the V rows
+        const int rc = rope_launch(stream, inout, nullptr, nullptr, position, cosin, slot_mapping, num_tokens, n_heads,
+                                   n_kv_heads, head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype,
+                                   false);
+        if (rc != XLITE_HIP_OK || num_tokens == 0) {
+            return rc;
+        }
+        XL_REQUIRE(k_cache && v_cache && k_scale && v_scale, "null tensor");
+        const uint32_t grid = grid_for(static_cast<uint64_t>(num_tokens) * 2 * n_kv_heads * 16, 256);
+        auto launch = [&](auto tag, auto kv) {
+            using T = decltype(tag);
+            quantize_to_cache_kernel<T, decltype(kv)::value><<<grid, 256, 0, as_stream(stream)>>>(
+                static_cast<const uint16_t *>(inout), kc, vc, k_scale, v_scale, slot_mapping, num_tokens, n_heads, n_kv_heads,
+                head_dim);
+        };
+        using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
+        using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;
+        if (dtype == XLITE_HIP_BF16) {
+            kv_dtype == XLITE_HIP_KV_INT8 ? launch(BF16{}, I8{}) : launch(BF16{}, F8{});
+        } else {
+            kv_dtype == XLITE_HIP_KV_INT8 ? launch(FP16{}, I8{}) : launch(FP16{}, F8{});
+        }
+        XL_LAUNCH_CHECK();
+        return XLITE_HIP_OK;
+    }
+    float scale = 0.f;
+    if (const int rc = rope_check(inout, position, cosin, slot_mapping, num_tokens, n_heads, n_kv_heads, head_dim, rot_dim,
+                                  block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype, &scale)) {
+        return rc;
+    }
+    if (num_tokens == 0) {
+        return XLITE_HIP_OK;
+    }
+    XL_REQUIRE(k_cache && v_cache && k_scale && v_scale, "null tensor");
+    const uint32_t grid = grid_for(static_cast<uint64_t>(num_tokens) * (n_heads + 2 * n_kv_heads) * 16, 256);
+    auto launch = [&](auto tag, auto kv) {
+        using T = decltype(tag);
+        rope_quant_cache_kernel<T, decltype(kv)::value><<<grid, 256, 0, as_stream(stream)>>>(
+            static_cast<uint16_t *>(inout), kc, vc, k_scale, v_scale, position, static_cast<const uint16_t *>(cosin),
+            slot_mapping, num_tokens, n_heads, n_kv_heads, head_dim, rot_dim, scale, mrope_mask_h, mrope_mask_w);
+    };
+    using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
+    using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;
+    if (dtype == XLITE_HIP_BF16) {
+        kv_dtype == XLITE_HIP_KV_INT8 ? launch(BF16{}, I8{}) : launch(BF16{}, F8{});
+    } else {
+        kv_dtype == XLITE_HIP_KV_INT8 ? launch(FP16{}, I8{}) : launch(FP16{}, F8{});
+    }
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
 extern "C" int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *k_cache, int8_t *v_cache,
                                              float *k_scale, float *v_scale, const int64_t *position,
                                              const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens,
@@ -478,25 +710,9 @@ extern "C" int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *
                                              uint32_t rot_dim, uint32_t block_size, int is_neox,
                                              uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype)
 {
-    const int rc = rope_launch(stream, inout, nullptr, nullptr, position, cosin, slot_mapping, num_tokens, n_heads,
-                               n_kv_heads, head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype,
-                               false);
-    if (rc != XLITE_HIP_OK || num_tokens == 0) {
-        return rc;
-    }
-    XL_REQUIRE(k_cache && v_cache && k_scale && v_scale, "null tensor");
-    const uint32_t grid = grid_for(static_cast<uint64_t>(num_tokens) * 2 * n_kv_heads * 16, 256);
-    if (dtype == XLITE_HIP_BF16) {
-        quantize_to_cache_kernel<BF16><<<grid, 256, 0, as_stream(stream)>>>(
-            static_cast<const uint16_t *>(inout), k_cache, v_cache, k_scale, v_scale, slot_mapping, num_tokens, n_heads,
-            n_kv_heads, head_dim);
-    } else {
-        quantize_to_cache_kernel<FP16><<<grid, 256, 0, as_stream(stream)>>>(
-            static_cast<const uint16_t *>(inout), k_cache, v_cache, k_scale, v_scale, slot_mapping, num_tokens, n_heads,
-            n_kv_heads, head_dim);
-    }
-    XL_LAUNCH_CHECK();
-    return XLITE_HIP_OK;
+    return xlite_hip_rope_and_cache_quant(stream, inout, k_cache, v_cache, k_scale, v_scale, position, cosin, slot_mapping,
+                                          num_tokens, n_heads, n_kv_heads, head_dim, rot_dim, block_size, is_neox,
+                                          mrope_mask_h, mrope_mask_w, dtype, XLITE_HIP_KV_INT8);
 }
 
 extern "C" int xlite_hip_qk_rms_norm(void *stream, const void *in, void *out, const void *q_norm,
@@ -643,26 +859,35 @@ extern "C" int xlite_hip_mla_prepare(void *stream, void *attn_qkvc, const void *
     return XLITE_HIP_OK;
 }
 
-extern "C" int xlite_hip_quantize_kv_int8(void *stream, const void *src, int8_t *dst, float *scales,
-                                          uint64_t rows, uint32_t head_dim, int dtype)
+extern "C" int xlite_hip_quantize_kv(void *stream, const void *src, void *dst, float *scales, uint64_t rows,
+                                     uint32_t head_dim, int dtype, int kv_dtype)
 {
     XL_REQUIRE(dtype == XLITE_HIP_BF16 || dtype == XLITE_HIP_FP16, "dtype unsupported!");
+    XL_REQUIRE(kv_dtype == XLITE_HIP_KV_INT8 || kv_dtype == XLITE_HIP_KV_FP8, "kv cache dtype unsupported!");
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
     XL_REQUIRE(src && dst && scales, "null tensor");
-    XL_REQUIRE(head_dim > 0, "head_dim must be positive");
-    if (rows == 0) {
-        return XLITE_HIP_OK;
-    }
+    XL_REQUIRE(head_dim > 0 && head_dim % 8 == 0, "head_dim must be a positive multiple of 8");
     const uint32_t grid = grid_for(rows * 16, 256);
+    auto launch = [&](auto tag, auto kv) {
+        using T = decltype(tag);
+        quantize_kv_kernel<T, decltype(kv)::value><<<grid, 256, 0, as_stream(stream)>>>(
+            static_cast<const uint16_t *>(src), static_cast<unsigned char *>(dst), scales, rows, head_dim);
+    };
+    using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
+    using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;
     if (dtype == XLITE_HIP_BF16) {
-        quantize_kv_kernel<BF16><<<grid, 256, 0, as_stream(stream)>>>(
-            static_cast<const uint16_t *>(src), dst, scales, rows, head_dim);
+        kv_dtype == XLITE_HIP_KV_INT8 ? launch(BF16{}, I8{}) : launch(BF16{}, F8{});
     } else {
-        quantize_kv_kernel<FP16><<<grid, 256, 0, as_stream(stream)>>>(
-            static_cast<const uint16_t *>(src), dst, scales, rows, head_dim);
+        kv_dtype == XLITE_HIP_KV_INT8 ? launch(FP16{}, I8{}) : launch(FP16{}, F8{});
     }
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
+}
+
+extern "C" int xlite_hip_quantize_kv_int8(void *stream, const void *src, int8_t *dst, float *scales,
+                                          uint64_t rows, uint32_t head_dim, int dtype)
+{
+    return xlite_hip_quantize_kv(stream, src, dst, scales, rows, head_dim, dtype, XLITE_HIP_KV_INT8);
 }

@@ -111,6 +111,24 @@ __device__ __forceinline__ uint4 widen(const uint2 &raw)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// fp8 (OCP e4m3) -> fp16 scaled by 2^-8, exactly, in three vector instructions per two values: the byte's
+// exponent and mantissa fields, shifted to the top of fp16's, read as that format give the value times 2^-8
+// (biases 7 and 15), for normal and subnormal bytes alike; the sign bit moves to bit 15. The factor 2^8 is
+// applied to the scores and to the output. (NaN bytes, which a quantiser never writes, would read as finite.)
+struct Fp8Tag {};
+template <typename T>
+__device__ __forceinline__ uint4 widen(const uint2 &raw, Fp8Tag)
+{
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        // bytes (2 (j % 2), 2 (j % 2) + 1) of word j / 2 to the high bytes of the two halves
+        const uint32_t x = __builtin_amdgcn_perm(0u, (&raw.x)[j / 2], (j % 2) ? 0x030c020cu : 0x010c000cu);
+        w[j] = ((x >> 1) & 0x3f803f80u) | (x & 0x80008000u);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // XOR pattern applied to the 16-byte chunk index of LDS row `row`. One pattern serves both read
 // shapes: 16 lanes reading the same chunk of 16 consecutive rows (K as MFMA A operand) land in 16
 // different chunk slots, and 8 consecutive rows read as 32-byte pieces (transposing V read) land
@@ -305,10 +323,12 @@ struct DecodeSplit {
     }
 };
 
-template <typename T, int D, bool KV8, bool MULTI_SUB>
+template <typename T, int D, int KVF, bool MULTI_SUB>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_mfma_kernel(const DecodeMfmaParams p)
 {
+    constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;                  // a cache of bytes with per-position scales
+    constexpr float kKvMul = KVF == XLITE_HIP_KV_FP8 ? 256.f : 1.f;  // fp8 bytes are widened to value * 2^-8
     constexpr int CH = D / 8;            // 16-byte chunks per LDS row
     constexpr int ROWB = D * 2;          // LDS bytes per row
     constexpr int KS = D / 32;           // k-steps of the QK product
@@ -534,8 +554,13 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 constexpr int SL = decltype(slot_tag)::value;
 #pragma unroll
                 for (int i = 0; i < NV; i++) {
-                    *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i]) = widen<T>(kreg[SL][i]);
-                    *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i] + TILE_BYTES) = widen<T>(vreg[SL][i]);
+                    if constexpr (KVF == XLITE_HIP_KV_FP8) {
+                        *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i]) = widen<T>(kreg[SL][i], Fp8Tag{});
+                        *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i] + TILE_BYTES) = widen<T>(vreg[SL][i], Fp8Tag{});
+                    } else {
+                        *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i]) = widen<T>(kreg[SL][i]);
+                        *reinterpret_cast<uint4 *>(smem + SL * STAGE_BYTES + w_off[i] + TILE_BYTES) = widen<T>(vreg[SL][i]);
+                    }
                 }
                 if constexpr (KV8) {
                     if (s_active) {
@@ -574,7 +599,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 float mx = -INFINITY;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    float v = S[e] * kLog2e;
+                    float v = S[e] * (kLog2e * kKvMul);
                     if constexpr (KV8) {
                         v *= reinterpret_cast<const float *>(&kscale)[e];
                     }
@@ -686,8 +711,9 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             }
             if (kv_ok && col < g_valid && my_sub == 0) {
                 // O^T lane layout: column = head `col`, rows 16 mt + 4 jq + e
+                // (fp8 cache: O carries the factor 2^-8 of the widened values; it leaves through the normaliser)
                 if (single) {
-                    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+                    const float inv = l_tot > 0.f ? kKvMul / l_tot : 0.f;
                     uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
@@ -704,7 +730,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
                     }
                     if (jq == 0) {
-                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot * (1.0f / kKvMul));
                     }
                 }
             }
@@ -979,12 +1005,13 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
     return XLITE_HIP_OK;
 }
 
-template <typename T, int D, bool KV8, bool MULTI_SUB>
+template <typename T, int D, int KVF, bool MULTI_SUB>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
+    constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
                        (kSplitLdsWords + p.total_rows + 1) * sizeof(uint32_t);
-    auto kernel = decode_mfma_kernel<T, D, KV8, MULTI_SUB>;
+    auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
             return rc;
@@ -996,11 +1023,24 @@ int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
     return XLITE_HIP_OK;
 }
 
-template <typename T, int D, bool KV8>
+template <typename T, int D, int KVF>
 int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
-    return p.n_sub > 1 ? launch_inst<T, D, KV8, true>(stream, p, grid_x)
-                       : launch_inst<T, D, KV8, false>(stream, p, grid_x);
+    return p.n_sub > 1 ? launch_inst<T, D, KVF, true>(stream, p, grid_x)
+                       : launch_inst<T, D, KVF, false>(stream, p, grid_x);
+}
+
+template <typename T, int D>
+int launch_fmt(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x, int kv_dtype)
+{
+    switch (kv_dtype) {
+    case XLITE_HIP_KV_INT8:
+        return launch_one<T, D, XLITE_HIP_KV_INT8>(stream, p, grid_x);
+    case XLITE_HIP_KV_FP8:
+        return launch_one<T, D, XLITE_HIP_KV_FP8>(stream, p, grid_x);
+    default:
+        return launch_one<T, D, XLITE_HIP_KV_SAME>(stream, p, grid_x);
+    }
 }
 
 }  // namespace
@@ -1045,7 +1085,6 @@ size_t decode_mfma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t he
 
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
 {
-    const bool kv8 = a.kv_dtype == XLITE_HIP_KV_INT8;
     const bool bf = a.dtype == XLITE_HIP_BF16;
     DecodeMfmaParams p{};
     p.q = static_cast<const uint16_t *>(a.qkv);
@@ -1091,15 +1130,9 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
         rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
     } else if (a.head_dim == 128) {
-        if (bf) {
-            rc = kv8 ? launch_one<BF16, 128, true>(stream, p, grid_x) : launch_one<BF16, 128, false>(stream, p, grid_x);
-        } else {
-            rc = kv8 ? launch_one<FP16, 128, true>(stream, p, grid_x) : launch_one<FP16, 128, false>(stream, p, grid_x);
-        }
-    } else if (bf) {
-        rc = kv8 ? launch_one<BF16, 64, true>(stream, p, grid_x) : launch_one<BF16, 64, false>(stream, p, grid_x);
+        rc = bf ? launch_fmt<BF16, 128>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 128>(stream, p, grid_x, a.kv_dtype);
     } else {
-        rc = kv8 ? launch_one<FP16, 64, true>(stream, p, grid_x) : launch_one<FP16, 64, false>(stream, p, grid_x);
+        rc = bf ? launch_fmt<BF16, 64>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 64>(stream, p, grid_x, a.kv_dtype);
     }
     if (rc != XLITE_HIP_OK) {
         return rc;

@@ -78,8 +78,19 @@ def _randn(shape, gen, device, dtype, scale: float = 1.0, chunk: int = 1 << 26) 
     return out
 
 
+def quantize_cache(x: torch.Tensor, kv_dtype: torch.dtype):
+    """Per (position, kv head) symmetric quantisation of a cache tensor [..., head_dim] to int8 (scale =
+    absmax / 127) or float8_e4m3fn (scale = absmax / 448); returns the bytes and the fp32 scales."""
+    xf = x.float()
+    scale = xf.abs().amax(dim=-1) / (127.0 if kv_dtype == torch.int8 else 448.0)
+    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+    y = xf / safe.unsqueeze(-1)
+    q = torch.clamp(torch.round(y), -127, 127).to(torch.int8) if kv_dtype == torch.int8 else y.to(kv_dtype)
+    return q, scale.contiguous()
+
+
 def gqa_decode(shape: GqaShape, ctx: List[int], seed: int, device="cpu", int8_kv: bool = False,
-               spare_blocks: int = 2) -> Dict:
+               spare_blocks: int = 2, kv_dtype: Optional[torch.dtype] = None) -> Dict:
     """One decode step: every sequence has ctx[i] - 1 cached tokens and one new token whose K/V is
     already in the cache (the operator reads only the caches)."""
     gen = torch.Generator(device=device).manual_seed(seed)
@@ -98,14 +109,12 @@ def gqa_decode(shape: GqaShape, ctx: List[int], seed: int, device="cpu", int8_kv
              cached_lens=torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=device),
              block_tables=t["tables"].flatten().contiguous(), max_num_block=t["max_num_block"],
              k_scale=None, v_scale=None)
+    if int8_kv and kv_dtype is None:
+        kv_dtype = torch.int8
+    int8_kv = kv_dtype is not None
     if int8_kv:
         for name in ("k", "v"):
-            x = w[name + "_cache"].float()
-            amax = x.abs().amax(dim=-1)
-            scale = amax / 127.0
-            safe = torch.where(scale > 0, scale, torch.ones_like(scale))
-            w[name + "_cache"] = torch.clamp(torch.round(x / safe.unsqueeze(-1)), -127, 127).to(torch.int8)
-            w[name + "_scale"] = scale.contiguous()
+            w[name + "_cache"], w[name + "_scale"] = quantize_cache(w[name + "_cache"], kv_dtype)
     kv_elt = 1 if int8_kv else 2
     total_ctx = sum(ctx)
     w["kv_bytes"] = total_ctx * KV * D * 2 * kv_elt + (total_ctx * KV * 2 * 4 if int8_kv else 0)

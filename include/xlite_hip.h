@@ -32,9 +32,10 @@ extern "C" {
 /* element types (same order as xlite/csrc/base.h XDtype FP16/BF16) */
 #define XLITE_HIP_FP16 0
 #define XLITE_HIP_BF16 1
-/* KV cache element types: the activation dtype, or int8 with fp32 scales */
+/* KV cache element types: the activation dtype, or int8 / fp8 (OCP e4m3) with fp32 scales */
 #define XLITE_HIP_KV_SAME 0
 #define XLITE_HIP_KV_INT8 1
+#define XLITE_HIP_KV_FP8 2
 
 /* Message of the last failed call on this thread ("" if none). */
 const char *xlite_hip_last_error(void);
@@ -68,9 +69,14 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  *
  * qkv         [total_tokens, (n_heads + 2*n_kv_heads) * head_dim]; only q is read,
  *             already rotated and scaled by rope_and_cache
- * k_cache/v_cache  paged caches as above; when kv_dtype == XLITE_HIP_KV_INT8 they
- *             hold int8 and k_scale/v_scale [num_blocks, block_size, n_kv_heads]
- *             fp32 hold the per-token-per-head scales (x = q8 * scale)
+ * k_cache/v_cache  paged caches as above; when kv_dtype is XLITE_HIP_KV_INT8 or
+ *             XLITE_HIP_KV_FP8 they hold one byte per element and k_scale/v_scale
+ *             [num_blocks, block_size, n_kv_heads] fp32 hold the per-token-per-head scales
+ *             (x = q * scale). Decode batches of the streaming kernel's shapes (at most 16
+ *             query heads per kv head, block size a multiple of 16) read the bytes directly;
+ *             every other batch over a quantised cache (prefill, chunked prefill, mixed
+ *             batches, other decode shapes) first copies the blocks it can see into a 16-bit
+ *             cache in the workspace, which xlite_hip_attention_workspace_bytes_kv() sizes.
  * output      [total_tokens, n_heads * head_dim]
  * query_start_loc, lens, cached_lens  [batch] int32
  * block_tables [batch * max_num_block] int32
@@ -78,8 +84,9 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  * No softmax scale is applied here (q arrives pre-scaled).
  *
  * workspace   device scratch of at least xlite_hip_attention_workspace_bytes()
- *             (split-KV partial results; contents need no initialisation and
- *             are not preserved). Decode batches need all of it
+ *             (or ..._bytes_kv() for a quantised cache; split-KV partial results;
+ *             contents need no initialisation and are not preserved). Decode batches
+ *             and batches over a quantised cache need all of it
  *             (XLITE_HIP_ENOSPC otherwise); a prefill batch given less, or
  *             NULL, still works but does not split the KV axis.
  * ---------------------------------------------------------------------- */
@@ -88,6 +95,11 @@ size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_hea
                                            uint32_t n_kv_heads, uint32_t head_dim,
                                            uint32_t block_size, uint32_t batch,
                                            uint32_t max_num_block);
+/* the same for a given cache element type (the call above is kv_dtype = XLITE_HIP_KV_SAME) */
+size_t xlite_hip_attention_workspace_bytes_kv(uint32_t total_tokens, uint32_t n_heads,
+                                              uint32_t n_kv_heads, uint32_t head_dim,
+                                              uint32_t block_size, uint32_t batch,
+                                              uint32_t max_num_block, int kv_dtype);
 
 int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, const void *v_cache,
                         void *output, const int32_t *query_start_loc, const int32_t *lens,
@@ -321,20 +333,35 @@ int xlite_hip_indexer_topk(void *stream, const void *q, const void *k_cache, con
                            uint32_t top_k, int dtype, void *workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------------------------------
- * int8 KV-cache helper (no counterpart in the reference, whose caches are always
- * the activation dtype): quantise rows of `src` [rows, head_dim] into `dst` int8
- * with one fp32 scale per row, scale = absmax/127, q = clamp(rint(x/scale), -127, 127).
+ * Quantised KV caches (no counterpart in the reference, whose caches are always the
+ * activation dtype). One fp32 scale per (token, kv head) row of head_dim elements:
+ *   XLITE_HIP_KV_INT8: scale = absmax / 127, q = clamp(rint(x / scale), -127, 127)
+ *   XLITE_HIP_KV_FP8:  scale = absmax / 448, q = e4m3(x / scale), OCP e4m3, round to nearest even
+ * and x = q * scale. A row of zeros gets scale 0.
+ * quantize_kv: rows of `src` [rows, head_dim] (16-bit) into `dst` (one byte per element) and
+ * `scales` [rows]. quantize_kv_int8 is the same with kv_dtype = XLITE_HIP_KV_INT8.
  * ---------------------------------------------------------------------- */
+int xlite_hip_quantize_kv(void *stream, const void *src, void *dst, float *scales, uint64_t rows,
+                          uint32_t head_dim, int dtype, int kv_dtype);
 int xlite_hip_quantize_kv_int8(void *stream, const void *src, int8_t *dst, float *scales,
                                uint64_t rows, uint32_t head_dim, int dtype);
 
 /* ------------------------------------------------------------------------
- * rope_and_cache with quantise-on-write for the int8 KV cache (no counterpart in the
- * reference): the same rotation and q scaling as xlite_hip_rope_and_cache, in place; the
- * rotated K rows and the V rows are then quantised as above into
- * k_cache / v_cache [num_blocks, block_size, n_kv_heads, head_dim] int8 with
- * k_scale / v_scale [num_blocks, block_size, n_kv_heads] fp32 at the tokens' slots.
+ * rope_and_cache with quantise-on-write (no counterpart in the reference; the write it extends
+ * is xlite/csrc/kernels/rope_and_cache.h:486-501, :563-564): the same rotation and q scaling as
+ * xlite_hip_rope_and_cache, in place; the rotated K rows and the V rows go to
+ * k_cache / v_cache [num_blocks, block_size, n_kv_heads, head_dim] (one byte per element) as the
+ * quantisation above of the 16-bit rows, with k_scale / v_scale [num_blocks, block_size,
+ * n_kv_heads] fp32, at the tokens' slots. One kernel launch for heads of at most 16 items
+ * (head_dim / 8 - rot_dim / 16 <= 16); wider heads take a second, quantising launch.
+ * rope_and_cache_int8 is the same with kv_dtype = XLITE_HIP_KV_INT8.
  * ---------------------------------------------------------------------- */
+int xlite_hip_rope_and_cache_quant(void *stream, void *inout, void *k_cache, void *v_cache,
+                                   float *k_scale, float *v_scale, const int64_t *position,
+                                   const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens,
+                                   uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                                   uint32_t rot_dim, uint32_t block_size, int is_neox,
+                                   uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, int kv_dtype);
 int xlite_hip_rope_and_cache_int8(void *stream, void *inout, int8_t *k_cache, int8_t *v_cache,
                                   float *k_scale, float *v_scale, const int64_t *position,
                                   const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens,

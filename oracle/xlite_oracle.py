@@ -41,6 +41,8 @@ piece of the reference (paths under /root/reference/):
   quantize_kv_int8 / dequantize_kv_int8   not in the reference (its caches are never
                        quantised); definition from the benchmark contract:
                        scale = absmax/127 per (token, kv head), symmetric.
+  quantize_kv_fp8 / dequantize_kv_fp8     not in the reference either; the same layout with OCP e4m3 bytes,
+                       scale = absmax/448 (the format's largest value), round to nearest even.
 
 Pinning status (what independent evidence each function is checked against in
 tests/test_oracle_pins.py):
@@ -676,4 +678,19 @@ def quantize_kv_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 def dequantize_kv_int8(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    return q.float() * scale.unsqueeze(-1)
+
+
+def quantize_kv_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [..., head_dim] -> (float8_e4m3fn same shape, fp32 scale [...]); scale = absmax/448 (the largest e4m3
+    value), the quotient rounded to nearest even by torch's conversion (the OCP e4m3 format, no infinities)."""
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1)
+    scale = amax / 448.0
+    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+    q = (xf / safe.unsqueeze(-1)).to(torch.float8_e4m3fn)
+    return q, scale
+
+
+def dequantize_kv_fp8(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     return q.float() * scale.unsqueeze(-1)

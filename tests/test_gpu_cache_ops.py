@@ -137,21 +137,36 @@ def test_mla_prepare(rt, dtype):
     assert int(dk2.abs().sum()) == 0
 
 
-def test_quantize_kv_int8_matches_definition(rt):
-    from gvirt_amd._C import quantize_kv_int8
-    g = torch.Generator().manual_seed(9)
-    x = torch.randn(3, 128, 8, 128, generator=g).bfloat16()
-    x[0, 0, 0] = 0
-    q, s = quantize_kv_int8(rt, x.to(DEV))
-    qr, sr = O.quantize_kv_int8(x)
-    assert torch.equal(q.cpu(), qr) and torch.equal(s.cpu(), sr)
+QUANT = {torch.int8: O.quantize_kv_int8, torch.float8_e4m3fn: O.quantize_kv_fp8}
 
 
+def _same(a, b):
+    return torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+@pytest.mark.parametrize("kv_dtype", [torch.int8, torch.float8_e4m3fn])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("nH,nKV,d,rot", [(32, 8, 128, 128), (14, 2, 64, 64), (8, 4, 128, 64)])
-def test_rope_and_cache_int8_quantise_on_write(rt, dtype, nH, nKV, d, rot):
-    """The rows land in the int8 cache as the oracle's quantisation of the oracle's rotated rows: bit-exact
-    (values and scales); slots of other tokens keep their contents."""
+def test_quantize_kv_matches_definition(rt, kv_dtype, dtype):
+    from gvirt_amd._C import quantize_kv, quantize_kv_int8
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(3, 128, 8, 128, generator=g) * torch.rand(3, 128, 8, 1, generator=g) * 4).to(dtype)
+    x[0, 0, 0] = 0
+    x[1, 5, 2] *= 1e-4      # a tiny row: its quotients still span the format's whole range
+    q, s = quantize_kv(rt, x.to(DEV), kv_dtype)
+    qr, sr = QUANT[kv_dtype](x)
+    assert q.dtype == kv_dtype and _same(q.cpu(), qr) and torch.equal(s.cpu(), sr)
+    if kv_dtype == torch.int8:
+        q2, s2 = quantize_kv_int8(rt, x.to(DEV))
+        assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
+@pytest.mark.parametrize("kv_dtype", [torch.int8, torch.float8_e4m3fn])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nH,nKV,d,rot", [(32, 8, 128, 128), (14, 2, 64, 64), (8, 4, 128, 64), (4, 2, 256, 256), (4, 1, 256, 64)])
+def test_rope_and_cache_quantise_on_write(rt, kv_dtype, dtype, nH, nKV, d, rot):
+    """The rows land in the quantised cache as the oracle's quantisation of the oracle's rotated rows: bit-exact
+    (values and scales); slots of other tokens keep their contents. One launch for heads of at most 16 items
+    (all but the last shape), two for wider ones."""
     from gvirt_amd._C import rope_and_cache
     g = torch.Generator().manual_seed(300 + nH + d + rot)
     T, bs, NB = 37, 16, 5
@@ -160,8 +175,8 @@ def test_rope_and_cache_int8_quantise_on_write(rt, dtype, nH, nKV, d, rot):
     cosin = _cosin(rot, 512, dtype)
     pos = torch.randint(0, 512, (T,), generator=g)
     slots = torch.randperm(NB * bs, generator=g)[:T].int()
-    kq = torch.full((NB, bs, nKV, d), 9, dtype=torch.int8, device=DEV)
-    vq = torch.full((NB, bs, nKV, d), -9, dtype=torch.int8, device=DEV)
+    fill = lambda v: torch.full((NB, bs, nKV, d), v, dtype=torch.int8).view(kv_dtype).to(DEV)
+    kq, vq = fill(9), fill(-9)
     ks = torch.full((NB, bs, nKV), 5.0, device=DEV)
     vs = torch.full((NB, bs, nKV), -5.0, device=DEV)
     dev_inout = inout.to(DEV)
@@ -172,14 +187,15 @@ def test_rope_and_cache_int8_quantise_on_write(rt, dtype, nH, nKV, d, rot):
     vc = torch.zeros(NB, bs, nKV, d).to(dtype)
     O.rope_and_cache_ref(inout, kc, vc, pos, cosin, slots, nH, nKV, d, rot, bs)
     assert torch.equal(_bits(dev_inout), _bits(inout))
-    kq_ref, ks_ref = O.quantize_kv_int8(kc)
-    vq_ref, vs_ref = O.quantize_kv_int8(vc)
+    kq_ref, ks_ref = QUANT[kv_dtype](kc)
+    vq_ref, vs_ref = QUANT[kv_dtype](vc)
     written = torch.zeros(NB * bs, dtype=torch.bool)
     written[slots.long()] = True
     w = written.view(NB, bs)
-    assert torch.equal(kq.cpu()[w], kq_ref[w]) and torch.equal(vq.cpu()[w], vq_ref[w])
+    b = lambda t: t.cpu().view(torch.int8)
+    assert torch.equal(b(kq)[w], b(kq_ref)[w]) and torch.equal(b(vq)[w], b(vq_ref)[w])
     assert torch.equal(ks.cpu()[w], ks_ref[w]) and torch.equal(vs.cpu()[w], vs_ref[w])
-    assert bool((kq.cpu()[~w] == 9).all()) and bool((vq.cpu()[~w] == -9).all())
+    assert bool((b(kq)[~w] == 9).all()) and bool((b(vq)[~w] == -9).all())
     assert bool((ks.cpu()[~w] == 5.0).all()) and bool((vs.cpu()[~w] == -5.0).all())
 
 

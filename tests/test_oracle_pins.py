@@ -285,6 +285,49 @@ def test_int8_roundtrip_bound():
     assert int(z.abs().max()) == 0 and float(sz.max()) == 0.0
 
 
+def _e4m3_value(byte: int) -> float:
+    """A byte of the OCP e4m3 format by its definition: sign, 4 exponent bits (bias 7), 3 mantissa bits; exponent
+    0 is subnormal (no implicit one, 2^-6); 0x7f / 0xff are NaN and there are no infinities."""
+    s, e, m = byte >> 7, (byte >> 3) & 15, byte & 7
+    if e == 15 and m == 7:
+        return float("nan")
+    mag = (m / 8.0) * 2.0 ** -6 if e == 0 else (1.0 + m / 8.0) * 2.0 ** (e - 7)
+    return -mag if s else mag
+
+
+def test_fp8_quantiser_against_the_format_definition():
+    """The fp8 cache format is pinned by brute force over the format's 256 bytes: torch decodes every byte to the
+    value the definition gives, and the quantiser picks, for every element, the representable value nearest to
+    x / scale (ties to the even mantissa), with scale = absmax / 448; the round trip error is at most half a step
+    of the format at that magnitude."""
+    table = torch.tensor([_e4m3_value(b) for b in range(256)], dtype=torch.float64)
+    dec = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).double()
+    finite = ~torch.isnan(table)
+    assert torch.equal(dec[finite], table[finite]) and bool(torch.isnan(dec[~finite]).all())
+    assert float(table[finite].max()) == 448.0
+    g = torch.Generator().manual_seed(16)
+    x = (torch.randn(5, 4, 64, generator=g) * torch.tensor([1e-3, 1.0, 37.0, 1e3]).view(1, 4, 1)).bfloat16()
+    q, s = O.quantize_kv_fp8(x)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.float32
+    assert torch.equal(s, x.float().abs().amax(-1) / 448.0)
+    y = (x.float() / s.unsqueeze(-1)).double()                      # the quotients, exactly representable in fp64
+    pos = table[:127]                                                # non-negative finite values, ascending
+    codes = q.view(torch.uint8).long()
+    for yy, cc in zip(y.flatten().tolist(), codes.flatten().tolist()):
+        d = (pos - abs(yy)).abs()
+        best = float(d.min())
+        cands = [i for i in range(127) if float(d[i]) == best]
+        want = cands[0] if len(cands) == 1 else [i for i in cands if i % 2 == 0][0]   # tie: even mantissa
+        assert (cc & 127) == want and ((cc >> 7) == (1 if yy < 0 else 0) or want == 0), (yy, cc, want)
+    assert int((codes & 127).max()) == 126                           # every row reaches the format's maximum, 448
+    back = O.dequantize_kv_fp8(q, s)
+    step = torch.where(y.abs() >= 2.0 ** -6, 2.0 ** (torch.floor(torch.log2(y.abs().clamp_min(2.0 ** -6))) - 3), torch.tensor(2.0 ** -9, dtype=torch.float64))
+    # (the quotient and the product back are fp32 operations: a few 2^-24 of |x| on top of the format's half step)
+    assert bool(((back.double() - x.double()).abs() <= 0.5 * step * s.unsqueeze(-1).double() + 4e-7 * x.double().abs() + 1e-30).all())
+    z, sz = O.quantize_kv_fp8(torch.zeros(2, 8))
+    assert int(z.view(torch.uint8).max()) == 0 and float(sz.max()) == 0.0
+
+
 def test_fp16_conversions_in_c_match_torch():
     g = torch.Generator().manual_seed(15)
     vals = torch.cat([torch.randn(2000, generator=g) * 10 ** torch.randint(-9, 6, (2000,), generator=g).float(),
