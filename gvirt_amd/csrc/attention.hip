@@ -40,6 +40,18 @@ size_t workspace_bytes_16(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv
                     prefill_mfma_workspace_bytes(total_tokens, n_heads, n_kv_heads, head_dim, batch, max_ctx));
 }
 
+// A batch that is mostly decode rows with prefills among them (what a continuous-batching scheduler issues: the
+// reference's decode flag is per batch, xlite/csrc/runtime.cpp:466-470) is served by two kernels: the
+// sequences with one query row by the streaming decode kernel, the others by the streaming prefill kernel.
+// Decided from the shape alone (the lengths live in device memory): at least 16 sequences and fewer than 4
+// rows per sequence on average.
+bool mixed_split(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
+                 uint32_t batch)
+{
+    return !is_decode_batch(total_tokens, batch) && batch >= 16 && total_tokens > batch && total_tokens < 4 * batch &&
+           decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, batch);
+}
+
 // A quantised cache is read directly by the streaming decode kernel (and, int8 only, by the vector decode
 // kernel); every other batch goes through a 16-bit copy of its blocks.
 bool quantised_direct(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
@@ -63,6 +75,9 @@ extern "C" size_t xlite_hip_attention_workspace_bytes_kv(uint32_t total_tokens, 
         return 0;
     }
     size_t need = workspace_bytes_16(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block);
+    if (mixed_split(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch)) {
+        need += decode_mfma_workspace_bytes(total_tokens, n_heads, head_dim, block_size, max_num_block);
+    }
     if (kv_dtype != XLITE_HIP_KV_SAME &&
         !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
         need += kv_dequant_bytes(n_kv_heads, head_dim, block_size, batch, max_num_block);
@@ -105,6 +120,22 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
                     total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
                     dtype, kv_dtype, k_scale, v_scale, workspace, workspace_bytes};
     hipStream_t s = as_stream(stream);
+    AttentionArgs as16 = a;   // the shape as the 16-bit kernels will see it
+    as16.kv_dtype = XLITE_HIP_KV_SAME;
+    if (mixed_split(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch) && prefill_mfma_supported(as16)) {
+        // the decode rows first, straight from the cache (quantised or not); its scratch is the front of the workspace
+        const size_t dec = decode_mfma_workspace_bytes(total_tokens, n_heads, head_dim, block_size, max_num_block);
+        AttentionArgs d = a;
+        d.rows_mode = kOnlySingle;
+        if (workspace != nullptr && workspace_bytes >= dec) {
+            if (const int rc = launch_decode_mfma(s, d)) {
+                return rc;
+            }
+            a.rows_mode = kSkipSingle;
+            a.workspace = static_cast<char *>(workspace) + dec;
+            a.workspace_bytes = workspace_bytes - dec;
+        }   // (too little scratch: one kernel serves every row, as for any prefill batch)
+    }
     if (kv_dtype != XLITE_HIP_KV_SAME &&
         !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
         XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");

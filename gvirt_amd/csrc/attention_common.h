@@ -20,7 +20,11 @@ struct AttentionArgs {
     const float *v_scale;
     void *workspace;
     size_t workspace_bytes;
+    // a batch served by two kernels: kOnlySingle = only the sequences with exactly one query row (the decode
+    // kernels), kSkipSingle = all the others (the prefill kernel, the dequantising copy)
+    int rows_mode;
 };
+enum { kAllRows = 0, kOnlySingle = 1, kSkipSingle = 2 };
 
 struct MlaArgs {
     const void *q_absorb;

@@ -86,6 +86,7 @@ struct DecodeMfmaParams {
     uint32_t n_sub;        // sub ranges of a segment handled by different waves (kv heads < 8)
     uint32_t batch;
     uint32_t total_rows;   // query rows of the batch (one per sequence in a plain decode step)
+    uint32_t only_single;  // 1: the units of the split are the sequences, and only those with one query row take part
 };
 
 // 8 cache elements (uint4 = 16-bit, uint2 = int8) -> 8 x 16-bit in a uint4
@@ -166,16 +167,17 @@ __device__ __forceinline__ uint32_t uni(uint32_t x)
 
 struct DecodeSplit {
     const DecodeMfmaParams &p;
-    uint32_t *wave_tot, *pref;   // LDS: kWaves words, rows + 1 words
-    uint32_t lane, wave, R;      // R: query rows of the batch, the units of the split
+    uint32_t *wave_tot, *pref;   // LDS: kWaves words, units + 1 words
+    uint32_t lane, wave, R;      // R: units of the split - the batch's query rows, or its sequences (only_single)
     bool in_lanes;
-    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_seq = 0, total = 0, chunk = 0, n_chunks = 0;
+    uint32_t ln_pref = 0, ln_steps = 0, ln_limit = 0, ln_seq = 0, ln_tok = 0, total = 0, chunk = 0, n_chunks = 0;
 
     // `lanes_ok`: a kernel short of registers keeps the sums in LDS whatever the batch
     __device__ __forceinline__ DecodeSplit(const DecodeMfmaParams &params, uint32_t *lds, uint32_t lane_, uint32_t wave_,
                                            bool lanes_ok = true)
-        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_), R(params.total_rows),
-          in_lanes(lanes_ok && params.total_rows <= 64)
+        : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_),
+          R(params.only_single ? params.batch : params.total_rows),
+          in_lanes(lanes_ok && (params.only_single ? params.batch : params.total_rows) <= 64)
     {
     }
     // The sequence that owns query row t. A batch of one row per sequence answers at once; otherwise (some
@@ -197,13 +199,34 @@ struct DecodeSplit {
         }
         return lo;
     }
-    // steps of row t; *limit = its visible range: row r of its sequence sees cached + r + 1 positions
-    __device__ __forceinline__ uint32_t steps_of(uint32_t t, uint32_t *limit, uint32_t *seq) const
+    // Steps of unit u; *limit = its visible range (row r of a sequence sees cached + r + 1 positions), *seq and
+    // *tok its sequence and query row. With only_single the unit is sequence u, which takes part when it has
+    // exactly one row; the rows of the others are marked "nothing to merge" (`mark`, first workgroup only): another
+    // kernel writes them.
+    __device__ __forceinline__ uint32_t steps_of(uint32_t u, uint32_t *limit, uint32_t *seq, uint32_t *tok, bool mark) const
     {
-        const uint32_t s = seq_of_row(t);
-        const int32_t lim = p.cached_lens[s] + (static_cast<int32_t>(t) - p.query_start_loc[s]) + 1;
+        if (p.only_single) {
+            const int32_t ql = p.lens[u], start = p.query_start_loc[u];
+            *seq = u;
+            *tok = static_cast<uint32_t>(start);
+            if (ql != 1) {
+                if (mark && blockIdx.x == 0) {
+                    for (int32_t r = 0; r < ql; r++) {
+                        reinterpret_cast<int4 *>(p.part_meta)[start + r] = make_int4(0, 0, 0, 0);
+                    }
+                }
+                *limit = 0;
+                return 0;
+            }
+            const int32_t lim = p.cached_lens[u] + 1;
+            *limit = static_cast<uint32_t>(lim > 1 ? lim : 1);
+            return ceil_div(*limit, static_cast<uint32_t>(kStep));
+        }
+        const uint32_t s = seq_of_row(u);
+        const int32_t lim = p.cached_lens[s] + (static_cast<int32_t>(u) - p.query_start_loc[s]) + 1;
         *limit = static_cast<uint32_t>(lim > 1 ? lim : 1);
         *seq = s;
+        *tok = u;
         return ceil_div(*limit, static_cast<uint32_t>(kStep));
     }
     // Exclusive prefix sums of the step counts. Up to 64 rows: every wave keeps them in its lanes
@@ -214,7 +237,7 @@ struct DecodeSplit {
     {
         if (in_lanes) {
             if (lane < R) {
-                ln_steps = steps_of(lane, &ln_limit, &ln_seq);
+                ln_steps = steps_of(lane, &ln_limit, &ln_seq, &ln_tok, true);
             }
             uint32_t incl = ln_steps;
 #pragma unroll
@@ -227,9 +250,9 @@ struct DecodeSplit {
         } else {
             const uint32_t ipt = ceil_div(R, static_cast<uint32_t>(kWaves * 64));
             const uint32_t i0 = min(R, threadIdx.x * ipt), i1 = min(R, i0 + ipt);
-            uint32_t mine = 0, limit, seq;
+            uint32_t mine = 0, limit, seq, tok;
             for (uint32_t i = i0; i < i1; i++) {
-                mine += steps_of(i, &limit, &seq);
+                mine += steps_of(i, &limit, &seq, &tok, true);
             }
             uint32_t incl = mine;
 #pragma unroll
@@ -247,7 +270,7 @@ struct DecodeSplit {
             }
             uint32_t run = before + incl - mine;
             for (uint32_t i = i0; i < i1; i++) {
-                const uint32_t n = steps_of(i, &limit, &seq);
+                const uint32_t n = steps_of(i, &limit, &seq, &tok, false);
                 pref[i] = (run << 4) | ((limit - 1) & 15u);
                 run += n;
             }
@@ -263,7 +286,7 @@ struct DecodeSplit {
             n_chunks = ceil_div(total, chunk);
         }
     }
-    // first step, step count and visible range of row i (every row has at least one step)
+    // first step, step count and visible range of unit i (*limit is meaningless when the unit has no steps)
     __device__ __forceinline__ void row_info(uint32_t i, uint32_t *first, uint32_t *n, uint32_t *limit) const
     {
         if (in_lanes) {
@@ -295,9 +318,19 @@ struct DecodeSplit {
         }
         return lo;
     }
-    __device__ __forceinline__ uint32_t seq_of(uint32_t row) const
+    __device__ __forceinline__ uint32_t seq_of(uint32_t unit) const
     {
-        return in_lanes ? uni(__shfl(ln_seq, static_cast<int>(row))) : uni(seq_of_row(uni(row)));
+        if (p.only_single) {
+            return uni(unit);
+        }
+        return in_lanes ? uni(__shfl(ln_seq, static_cast<int>(unit))) : uni(seq_of_row(uni(unit)));
+    }
+    __device__ __forceinline__ uint32_t tok_of(uint32_t unit) const
+    {
+        if (!p.only_single) {
+            return uni(unit);
+        }
+        return in_lanes ? uni(__shfl(ln_tok, static_cast<int>(unit))) : uni(static_cast<uint32_t>(p.query_start_loc[uni(unit)]));
     }
     // segment(seq, row, t0, t1, whole, partial slot, first piece of its row, meta of the row)
     template <typename F>
@@ -309,12 +342,16 @@ struct DecodeSplit {
             while (pos < end) {
                 uint32_t first, n, limit;
                 row_info(row, &first, &n, &limit);
+                if (n == 0) {   // a unit that takes no part (units without steps share their prefix with the next one)
+                    row++;
+                    continue;
+                }
                 const uint32_t a = pos - first, b = min(n, a + (end - pos));
                 const bool whole = a == 0 && b == n;
                 const bool first_seg = pos == start;
                 const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
                 const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
-                segment(seq_of(row), uni(row), uni(a * kStep), uni(min(limit, b * kStep)), whole,
+                segment(seq_of(row), tok_of(row), uni(a * kStep), uni(min(limit, b * kStep)), whole,
                         uni(2 * c + (first_seg ? 0u : 1u)), a == 0, meta);
                 pos += b - a;
                 row++;
@@ -994,7 +1031,7 @@ template <typename T>
 int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
-                       (kSplitLdsWords + p.total_rows + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + (p.only_single ? p.batch : p.total_rows) + 1) * sizeof(uint32_t);
     auto kernel = decode_dma_kernel<T>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
@@ -1010,7 +1047,7 @@ int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
-                       (kSplitLdsWords + p.total_rows + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + (p.only_single ? p.batch : p.total_rows) + 1) * sizeof(uint32_t);
     auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
@@ -1105,6 +1142,7 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     p.max_num_block = a.max_num_block;
     p.batch = a.batch;
     p.total_rows = a.total_tokens;
+    p.only_single = a.rows_mode == kOnlySingle ? 1u : 0u;
     DecodeSplitPlan pl{};
     decode_split_plan(a.total_tokens, a.n_heads, a.head_dim, a.block_size, a.max_num_block, &pl);
     const size_t need = pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;

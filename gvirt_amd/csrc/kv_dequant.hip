@@ -45,7 +45,7 @@ dequant_blocks_kernel(const unsigned char *__restrict__ k_cache, const unsigned 
                       const int32_t *__restrict__ block_tables, const int32_t *__restrict__ lens,
                       const int32_t *__restrict__ cached_lens, uint16_t *__restrict__ k_out, uint16_t *__restrict__ v_out,
                       int32_t *__restrict__ table_out, uint32_t block_size, uint32_t max_num_block, uint32_t n_kv_heads,
-                      uint32_t head_dim)
+                      uint32_t head_dim, uint32_t skip_single)
 {
     const uint32_t j = blockIdx.x, i = blockIdx.y;
     const bool is_v = blockIdx.z != 0;
@@ -53,7 +53,8 @@ dequant_blocks_kernel(const unsigned char *__restrict__ k_cache, const unsigned 
     if (!is_v && threadIdx.x == 0) {
         table_out[out_block] = static_cast<int32_t>(out_block);
     }
-    const int32_t visible = lens[i] > 0 ? cached_lens[i] + lens[i] : 0;
+    // sequences without rows need nothing; with skip_single those with one row read the bytes themselves
+    const int32_t visible = lens[i] > 0 && !(skip_single && lens[i] == 1) ? cached_lens[i] + lens[i] : 0;
     if (static_cast<int64_t>(j) * block_size >= visible) {
         return;
     }
@@ -122,7 +123,7 @@ int launch_kv_dequant(hipStream_t stream, AttentionArgs *a)
         dequant_blocks_kernel<T, decltype(kv)::value><<<grid, 256, 0, stream>>>(
             static_cast<const unsigned char *>(a->k_cache), static_cast<const unsigned char *>(a->v_cache), a->k_scale,
             a->v_scale, a->block_tables, a->lens, a->cached_lens, k_out, v_out, table, a->block_size, a->max_num_block,
-            a->n_kv_heads, a->head_dim);
+            a->n_kv_heads, a->head_dim, a->rows_mode == kSkipSingle ? 1u : 0u);
     };
     using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
     using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;

@@ -79,6 +79,7 @@ struct PrefillParams {
     uint32_t n_mtiles;         // grid.x
     uint32_t max_splits;       // grid.y: KV splits per M tile (1: none, results are final)
     uint32_t n_heads;
+    uint32_t skip_single;      // 1: sequences with exactly one query row are another kernel's
     int32_t *part_cnt;         // [token][head] number of partials to merge (0: the value is final)
     float *part_acc;           // [token][head][max_splits][D]
     float *part_ml;            // [token][head][max_splits][2]: reference maximum (log2 domain), normaliser
@@ -181,6 +182,13 @@ prefill_kernel(const PrefillParams p)
     }
     const uint32_t mt = tid - first_id(seq);
     const int32_t qlen = p.lens[seq];
+    if (p.skip_single && qlen == 1) {
+        // the decode kernel writes this row; the merge of this kernel's partials must leave it alone
+        if (p.part_cnt != nullptr && mt == 0 && blockIdx.y == 0 && threadIdx.x < G) {
+            p.part_cnt[static_cast<uint64_t>(p.query_start_loc[seq]) * p.n_heads + kvh * G + threadIdx.x] = 0;
+        }
+        return;
+    }
     if (qlen <= 0 || mt >= ceil_div(static_cast<uint32_t>(qlen) * G, static_cast<uint32_t>(kMTile))) {
         return;
     }
@@ -585,6 +593,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     // tile ids: every sequence may end with a ragged tile (see the kernel's numbering)
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
     p.n_heads = a.n_heads;
+    p.skip_single = a.rows_mode == kSkipSingle ? 1u : 0u;
     uint32_t splits = prefill_mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, a.max_num_block * a.block_size);
     if (a.workspace == nullptr || a.workspace_bytes < partial_bytes(a.total_tokens, a.n_heads, a.head_dim, splits)) {
         splits = 1;   // no scratch: every M tile walks its whole KV range

@@ -413,3 +413,32 @@ def test_block_tables_too_long_for_the_streaming_prefill_kernel(rt, model, lens)
     w = generic_case(19, lens, [131100], nH, nKV, d, bs, dtype, rms=True)
     assert w["max_num_block"] > 8191
     check(run_attention(rt, w), oracle_attention(w))
+
+
+def _mixed_lens(batch, prefills, seed):
+    """`batch` sequences, one query row each except the (index, rows) pairs of `prefills`; contexts 1..3000
+    (1..400 for the largest batches, which the CPU oracle would otherwise spend minutes on)."""
+    rng = np.random.default_rng(seed)
+    lens = [1] * batch
+    clens = [int(x) for x in rng.integers(1, 3000 if batch <= 130 else 400, size=batch)]
+    for i, n in prefills:
+        lens[i] = n
+        clens[i] = int(rng.integers(0, 2) * rng.integers(1, 700))
+    return clens, lens
+
+
+@pytest.mark.parametrize("kv_dtype", [None, torch.int8, torch.float8_e4m3fn])
+@pytest.mark.parametrize("model", [(32, 8, 128, 128, torch.bfloat16), (14, 2, 64, 16, torch.float16), (28, 4, 128, 64, torch.bfloat16)])
+@pytest.mark.parametrize("batch,prefills", [(21, [(0, 30)]), (40, [(39, 77), (5, 2)]), (130, [(64, 200), (3, 0), (129, 9)]),
+                                            (700, [(0, 300), (350, 0), (699, 130)])])
+def test_mixed_batch_split_between_decode_and_prefill_kernels(rt, kv_dtype, model, batch, prefills):
+    """Mostly decode rows with a few prefills (and sequences without rows) among them: the sequences with one
+    row go to the streaming decode kernel, the others to the prefill kernel, in one `attention` call; more than
+    64 sequences take the split's prefix sums through LDS."""
+    nH, nKV, d, bs, dtype = model
+    clens, lens = _mixed_lens(batch, prefills, batch)
+    assert batch < sum(lens) < 4 * batch
+    w = generic_case(81, lens, clens, nH, nKV, d, bs, dtype, rms=kv_dtype is None)
+    if kv_dtype is not None:
+        w = quantised(w, kv_dtype)
+    check(run_attention(rt, w), oracle_attention(w), max_abs=MAX_ABS if kv_dtype is None else MAX_ABS_INT8)
