@@ -48,7 +48,8 @@ size_t workspace_bytes_16(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv
 bool mixed_split(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
                  uint32_t batch)
 {
-    return !is_decode_batch(total_tokens, batch) && batch >= 16 && total_tokens > batch && total_tokens < 4 * batch &&
+    return !is_decode_batch(total_tokens, batch) && batch >= 16 && batch <= decode_mfma_slice_units() &&
+           total_tokens > batch && total_tokens < 4 * batch &&
            decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, batch);
 }
 

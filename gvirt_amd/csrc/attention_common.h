@@ -87,6 +87,7 @@ struct DecodeSplitPlan {
 size_t decode_mfma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint32_t block_size,
                                    uint32_t max_num_block);
 int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
+uint32_t decode_mfma_slice_units();   // units (rows, sequences) one launch of the decode kernels can split
 
 // mla_decode.hip
 struct MlaDecodeParams {

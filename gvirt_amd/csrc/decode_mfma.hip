@@ -87,6 +87,7 @@ struct DecodeMfmaParams {
     uint32_t batch;
     uint32_t total_rows;   // query rows of the batch (one per sequence in a plain decode step)
     uint32_t only_single;  // 1: the units of the split are the sequences, and only those with one query row take part
+    uint32_t unit0, n_units;   // this launch's slice of the units (rows or sequences): unit0 .. unit0 + n_units - 1
 };
 
 // 8 cache elements (uint4 = 16-bit, uint2 = int8) -> 8 x 16-bit in a uint4
@@ -176,8 +177,7 @@ struct DecodeSplit {
     __device__ __forceinline__ DecodeSplit(const DecodeMfmaParams &params, uint32_t *lds, uint32_t lane_, uint32_t wave_,
                                            bool lanes_ok = true)
         : p(params), wave_tot(lds), pref(lds + kWaves), lane(lane_), wave(wave_),
-          R(params.only_single ? params.batch : params.total_rows),
-          in_lanes(lanes_ok && (params.only_single ? params.batch : params.total_rows) <= 64)
+          R(params.n_units), in_lanes(lanes_ok && params.n_units <= 64)
     {
     }
     // The sequence that owns query row t. A batch of one row per sequence answers at once; otherwise (some
@@ -205,6 +205,7 @@ struct DecodeSplit {
     // kernel writes them.
     __device__ __forceinline__ uint32_t steps_of(uint32_t u, uint32_t *limit, uint32_t *seq, uint32_t *tok, bool mark) const
     {
+        u += p.unit0;   // units are numbered inside the launch's slice
         if (p.only_single) {
             const int32_t ql = p.lens[u], start = p.query_start_loc[u];
             *seq = u;
@@ -321,16 +322,16 @@ struct DecodeSplit {
     __device__ __forceinline__ uint32_t seq_of(uint32_t unit) const
     {
         if (p.only_single) {
-            return uni(unit);
+            return uni(unit + p.unit0);
         }
-        return in_lanes ? uni(__shfl(ln_seq, static_cast<int>(unit))) : uni(seq_of_row(uni(unit)));
+        return in_lanes ? uni(__shfl(ln_seq, static_cast<int>(unit))) : uni(seq_of_row(uni(unit + p.unit0)));
     }
     __device__ __forceinline__ uint32_t tok_of(uint32_t unit) const
     {
         if (!p.only_single) {
-            return uni(unit);
+            return uni(unit + p.unit0);
         }
-        return in_lanes ? uni(__shfl(ln_tok, static_cast<int>(unit))) : uni(static_cast<uint32_t>(p.query_start_loc[uni(unit)]));
+        return in_lanes ? uni(__shfl(ln_tok, static_cast<int>(unit))) : uni(static_cast<uint32_t>(p.query_start_loc[uni(unit + p.unit0)]));
     }
     // segment(seq, row, t0, t1, whole, partial slot, first piece of its row, meta of the row)
     template <typename F>
@@ -1031,7 +1032,7 @@ template <typename T>
 int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
-                       (kSplitLdsWords + (p.only_single ? p.batch : p.total_rows) + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
     auto kernel = decode_dma_kernel<T>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
@@ -1047,7 +1048,7 @@ int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
-                       (kSplitLdsWords + (p.only_single ? p.batch : p.total_rows) + 1) * sizeof(uint32_t);
+                       (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
     auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
@@ -1086,12 +1087,16 @@ bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_
                            uint32_t total_tokens)
 {
     const uint32_t group = n_heads / n_kv_heads;
-    // the work split keeps the prefix sums of the batch's rows in LDS
+    // (any number of rows: the work split keeps the prefix sums of up to kSplitSeqCap rows in LDS, larger batches
+    // run as several launches)
     (void)n_kv_heads;
-    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16 && total_tokens <= kSplitSeqCap;
+    (void)total_tokens;
+    return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16;
 }
 
 // decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8
+uint32_t decode_mfma_slice_units() { return kSplitSeqCap; }
+
 bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
 {
     return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0;
@@ -1164,19 +1169,36 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     p.part_acc = reinterpret_cast<float *>(ws + pl.meta_bytes + pl.ml_bytes);
     p.n_sub = a.n_kv_heads >= kWaves ? 1 : kWaves / a.n_kv_heads;
 
-    int rc;
-    if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
-        rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
-    } else if (a.head_dim == 128) {
-        rc = bf ? launch_fmt<BF16, 128>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 128>(stream, p, grid_x, a.kv_dtype);
-    } else {
-        rc = bf ? launch_fmt<BF16, 64>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 64>(stream, p, grid_x, a.kv_dtype);
+    // slices of at most kSplitSeqCap units, each with its own merge: the partial slots are reused from slice to
+    // slice. (Sequences' rows lie anywhere among the batch's rows, so a batch served by two kernels is one slice.)
+    const uint32_t units = p.only_single ? a.batch : a.total_tokens;
+    XL_REQUIRE(!p.only_single || units <= kSplitSeqCap, "too many sequences for a batch served by two kernels");
+    for (uint32_t u0 = 0; u0 < units; u0 += kSplitSeqCap) {
+        p.unit0 = u0;
+        p.n_units = min(kSplitSeqCap, units - u0);
+        int rc;
+        if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+            rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
+        } else if (a.head_dim == 128) {
+            rc = bf ? launch_fmt<BF16, 128>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 128>(stream, p, grid_x, a.kv_dtype);
+        } else {
+            rc = bf ? launch_fmt<BF16, 64>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 64>(stream, p, grid_x, a.kv_dtype);
+        }
+        if (rc != XLITE_HIP_OK) {
+            return rc;
+        }
+        if (!p.only_single) {
+            // the slice's rows are u0 .. u0 + n_units - 1
+            rc = launch_merge_meta(stream, a.dtype, static_cast<uint16_t *>(a.output) + static_cast<size_t>(u0) * a.n_heads * a.head_dim,
+                                   p.part_acc, p.part_ml, p.part_meta + static_cast<size_t>(u0) * 4, p.n_units, a.n_heads, a.head_dim);
+        } else {
+            rc = launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens, a.n_heads, a.head_dim);
+        }
+        if (rc != XLITE_HIP_OK) {
+            return rc;
+        }
     }
-    if (rc != XLITE_HIP_OK) {
-        return rc;
-    }
-    return launch_merge_meta(stream, a.dtype, a.output, p.part_acc, p.part_ml, p.part_meta, a.total_tokens, a.n_heads,
-                             a.head_dim);
+    return XLITE_HIP_OK;
 }
 
 }  // namespace xlite

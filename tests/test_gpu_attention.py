@@ -442,3 +442,43 @@ def test_mixed_batch_split_between_decode_and_prefill_kernels(rt, kv_dtype, mode
     if kv_dtype is not None:
         w = quantised(w, kv_dtype)
     check(run_attention(rt, w), oracle_attention(w), max_abs=MAX_ABS if kv_dtype is None else MAX_ABS_INT8)
+
+
+def compact_case(seed, lens, clens, nH, nKV, d, bs, dtype):
+    """generic_case with only the blocks the sequences need (a batch of thousands of short sequences and a few long
+    ones would otherwise reserve the longest sequence's block count for every one); table rows are padded with 0."""
+    g = torch.Generator().manual_seed(seed)
+    batch, T = len(lens), sum(lens)
+    need = [(l + c + bs - 1) // bs for l, c in zip(lens, clens)]
+    maxblk, NB = max(need), sum(need) + 1
+    rms = lambda x: x / x.pow(2).mean(-1, keepdim=True).add(1e-6).sqrt()
+    qkv = rms(torch.randn(T, nH + 2 * nKV, d, generator=g))
+    kc = rms(torch.randn(NB, bs, nKV, d, generator=g)).to(dtype)
+    vc = rms(torch.randn(NB, bs, nKV, d, generator=g)).to(dtype)
+    perm = torch.randperm(NB, generator=g).int()
+    tables = torch.zeros(batch, maxblk, dtype=torch.int32)
+    off = 0
+    for i, n in enumerate(need):
+        tables[i, :n] = perm[off:off + n]
+        off += n
+    shape = W.GqaShape("t", nH, nKV, d, bs, dtype)
+    return dict(shape=shape, batch=batch, qkv=qkv.reshape(T, -1).to(dtype), k_cache=kc, v_cache=vc,
+                output=torch.zeros(T, nH * d, dtype=dtype), query_start_loc=torch.tensor(np.cumsum([0] + lens[:-1]), dtype=torch.int32),
+                lens=torch.tensor(lens, dtype=torch.int32), cached_lens=torch.tensor(clens, dtype=torch.int32),
+                block_tables=tables.flatten(), max_num_block=maxblk)
+
+
+@pytest.mark.parametrize("model,batch", [((32, 8, 128, 128, torch.bfloat16), 4100), ((8, 2, 64, 16, torch.float16), 9000)])
+def test_decode_batches_beyond_one_launch_of_the_split(rt, model, batch):
+    """More rows than one launch of the decode kernel splits (4096): the batch runs as several launches over
+    slices of its rows, each followed by its merge. Short contexts, and a few long ones cut across workgroups."""
+    nH, nKV, d, bs, dtype = model
+    rng = np.random.default_rng(batch)
+    clens = [int(x) for x in rng.integers(1, 60, size=batch)]
+    for i in (7, 4095, 4096, batch - 1):
+        clens[i] = int(rng.integers(3000, 9000))
+    lens = [1] * batch
+    lens[4097], lens[4098] = 2, 0          # and the row / sequence numbering parts ways inside the second slice
+    w = compact_case(91, lens, clens, nH, nKV, d, bs, dtype)
+    assert w["k_cache"].numel() * 2 < 2 << 30
+    check(run_attention(rt, w), oracle_attention(w))
