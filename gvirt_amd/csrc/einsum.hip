@@ -2,9 +2,14 @@
 // (W_UK absorb and W_UV projection). Replaces XliteOpEinsumMhtHtdMhd / XliteOpEinsumMhtHdtMhd
 // (xlite/csrc/op.cpp:1872-1918, kernels/einsum_mht_htd_mhd.h:9-37).
 //
-// One wave computes a 32 x 32 output tile with v_mfma_f32_32x32x16, operands straight from
-// global memory (the left operand rows are k-contiguous; the [h,t,d] weight is read with
-// 2-byte loads that are contiguous across lanes). A workgroup covers 32 rows x 128 columns.
+// [h,d,t] weights (k-contiguous rows): one wave computes a 32 x 32 output tile with v_mfma_f32_32x32x16,
+// operands straight from global memory; a workgroup covers 32 rows x 128 columns.
+// [h,t,d] weights (the layout of both mla_v2 einsums): a workgroup covers 32 rows x 64 columns of one head and
+// its four waves split the reduction; a wave copies its slab of the weight (rows of 128 contiguous bytes) into
+// a region of LDS of its own with 16-byte loads, all of them in flight at once, and reads it back transposed
+// (ds_read_b64_tr_b16) as the B operand; the four partial tiles meet through LDS. With m <= 32 (a decode
+// step) every weight byte is read once, so the kernel is bound by streaming the weights: many small
+// workgroups (h * d / 64) keep every compute unit loading.
 #include "common.h"
 
 namespace xlite {
@@ -87,6 +92,117 @@ einsum_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__ w,
     }
 }
 
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+
+constexpr int kSlabCols = 64;                 // output columns of a workgroup
+constexpr int kSlabPitch = kSlabCols * 2 + 32;   // LDS bytes of a weight row: 128 + 32 keeps the transposing reads off each other's banks
+constexpr int kSlabRowsMax = 64;              // weight rows (k) a wave holds at a time
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+einsum_htd_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__ w, uint16_t *__restrict__ mhd,
+                  uint32_t m, uint32_t h, uint32_t t, uint32_t d, uint32_t t_stride)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char slab[4 * kSlabRowsMax * kSlabPitch];   // 40 KiB
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t col = lane & 31, half = lane >> 5;
+    const uint32_t head = blockIdx.z;
+    const uint32_t m0 = blockIdx.y * 32;
+    const uint32_t n0 = blockIdx.x * kSlabCols;
+    const uint32_t row = m0 + col;
+    const bool row_ok = row < m;
+    const uint16_t *a_ptr = mht + (static_cast<uint64_t>(row_ok ? row : 0) * h + head) * t_stride;
+    const uint16_t *w_head = w + static_cast<uint64_t>(head) * t * d + n0;
+    unsigned char *mine = slab + wave * (kSlabRowsMax * kSlabPitch);
+
+    // this wave's share of the reduction: a quarter of t, in multiples of 16
+    const uint32_t steps = t / 16, per = ceil_div(steps, 4u);
+    const uint32_t k_lo = min(steps, wave * per) * 16, k_hi = min(steps, (wave + 1) * per) * 16;
+
+    f32x16_t acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            acc[j][k] = 0.f;
+        }
+    }
+    // transposing read role: the 16-lane group g serves columns 16 (g % 2) .. + 15 of a 32-column tile and the
+    // rows 8 (g / 2) .. + 3 (+ 4 for the second read) of a 16-row step; lane 4 j' + q points at row j', columns 4 q .. + 3
+    const uint32_t gi = lane & 15, g = lane >> 4;
+    const uint32_t tr_off = (8 * (g >> 1) + (gi >> 2)) * kSlabPitch + (16 * (g & 1) + 4 * (gi & 3)) * 2;
+    typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+
+    for (uint32_t kb = k_lo; kb < k_hi; kb += kSlabRowsMax) {
+        const uint32_t rows = min(static_cast<uint32_t>(kSlabRowsMax), k_hi - kb);
+        // the slab: `rows` weight rows of 128 bytes = 8 lanes of 16 bytes; 8 rows per wave-wide load
+        uint4 v[kSlabRowsMax / 8];
+#pragma unroll
+        for (int i = 0; i < kSlabRowsMax / 8; i++) {
+            const uint32_t r = min(i * 8 + (lane >> 3), rows - 1);   // rows past the slab re-read its last row
+            v[i] = *reinterpret_cast<const uint4 *>(w_head + static_cast<uint64_t>(kb + r) * d + (lane & 7) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < kSlabRowsMax / 8; i++) {
+            const uint32_t r = i * 8 + (lane >> 3);
+            if (r < rows) {
+                *reinterpret_cast<uint4 *>(mine + r * kSlabPitch + (lane & 7) * 16) = v[i];
+            }
+        }
+        // wave-private region: the LDS counter wait the compiler inserts between the writes and the reads is all
+        // the ordering needed
+        for (uint32_t k0 = 0; k0 < rows; k0 += 16) {
+            uint4 a = make_uint4(0, 0, 0, 0);
+            if (row_ok) {
+                a = *reinterpret_cast<const uint4 *>(a_ptr + kb + k0 + half * 8);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                unsigned char *src = mine + k0 * kSlabPitch + tr_off + j * 64;
+                const uint2 b0 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)src));
+                const uint2 b1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(src + 4 * kSlabPitch)));
+                acc[j] = Mma<T>::run(a, make_uint4(b0.x, b0.y, b1.x, b1.y), acc[j]);
+            }
+        }
+    }
+    // the four partial tiles meet in LDS (the slabs are done with): [wave][32 rows][64 columns] fp32
+    __syncthreads();
+    float *part = reinterpret_cast<float *>(slab);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const uint32_t r = (k / 4) * 8 + half * 4 + (k % 4);
+            part[(wave * 32 + r) * kSlabCols + j * 32 + col] = acc[j][k];
+        }
+    }
+    __syncthreads();
+    // thread = (row, 8 columns): sums the four partials and stores 16 bytes
+    {
+        const uint32_t r = threadIdx.x >> 3, c8 = (threadIdx.x & 7) * 8;
+        if (m0 + r < m) {
+            float sum[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                sum[i] = 0.f;
+            }
+#pragma unroll
+            for (int wv = 0; wv < 4; wv++) {
+                const float4 x = *reinterpret_cast<const float4 *>(part + (wv * 32 + r) * kSlabCols + c8);
+                const float4 y = *reinterpret_cast<const float4 *>(part + (wv * 32 + r) * kSlabCols + c8 + 4);
+                sum[0] += x.x; sum[1] += x.y; sum[2] += x.z; sum[3] += x.w;
+                sum[4] += y.x; sum[5] += y.y; sum[6] += y.z; sum[7] += y.w;
+            }
+            uint4 o;
+            o.x = T::pack(sum[0], sum[1]);
+            o.y = T::pack(sum[2], sum[3]);
+            o.z = T::pack(sum[4], sum[5]);
+            o.w = T::pack(sum[6], sum[7]);
+            *reinterpret_cast<uint4 *>(mhd + (static_cast<uint64_t>(m0 + r) * h + head) * d + n0 + c8) = o;
+        }
+    }
+}
+
 }  // namespace
 }  // namespace xlite
 
@@ -113,6 +229,17 @@ extern "C" int xlite_hip_einsum_mht_mhd(void *stream, const void *mht, const voi
     const uint16_t *a = static_cast<const uint16_t *>(mht);
     const uint16_t *b = static_cast<const uint16_t *>(w);
     uint16_t *c = static_cast<uint16_t *>(mhd);
+    if (!w_is_hdt && d % kSlabCols == 0) {
+        // [h,t,d] weights: the LDS-transposing kernel
+        dim3 g2(d / kSlabCols, ceil_div(m, 32), h);
+        if (dtype == XLITE_HIP_BF16) {
+            einsum_htd_kernel<BF16><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
+        } else {
+            einsum_htd_kernel<FP16><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
+        }
+        XL_LAUNCH_CHECK();
+        return XLITE_HIP_OK;
+    }
     if (dtype == XLITE_HIP_BF16) {
         if (w_is_hdt) {
             einsum_kernel<BF16, true><<<grid, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);

@@ -113,7 +113,9 @@ def test_einsum(rt, m, h, t, d, dtype):
     torch.testing.assert_close(out.float().cpu(), ref, atol=2e-2, rtol=1e-2)
     out2 = torch.zeros(m, h, d, dtype=dtype, device=DEV)
     einsum_mht_hdt_mhd(rt, a.to(DEV), w.transpose(1, 2).contiguous().to(DEV), out2, m, h, t, d)
-    assert torch.equal(out.cpu().view(torch.int16), out2.cpu().view(torch.int16))
+    torch.testing.assert_close(out2.float().cpu(), ref, atol=2e-2, rtol=1e-2)
+    # the two layouts sum the products in different orders: equal up to a rounding step of the 16-bit result
+    torch.testing.assert_close(out.float().cpu(), out2.float().cpu(), atol=2e-3, rtol=2 ** -6)
 
 
 @pytest.mark.parametrize("nH,nope,vd", [(16, 128, 128), (8, 192, 256)])
