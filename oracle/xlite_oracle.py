@@ -68,8 +68,9 @@ tests/test_oracle_pins.py):
       q . k; with no intermediate rounding the weighted sum equals (sum_h w_h q_h) . k (linearity).
   indexer_topk_ref: numpy argsort on the same scores; every selected score >= every unselected one.
   get_tile_size_of_cached_kv_ref, prepare_attn_ref: hand-computed cases.
-  int8 KV: parity unpinned by the reference (feature absent there); pinned only by
-      the round-trip bound |x - dequant(quant(x))| <= scale/2.
+  int8 / fp8 KV: parity unpinned by the reference (feature absent there). int8 is pinned by the round-trip bound
+      |x - dequant(quant(x))| <= scale/2; fp8 by brute force over all 256 codes of OCP e4m3 (decoded values from
+      the format's definition, quantisation = nearest code, ties to even, against a search over the code table).
 """
 from __future__ import annotations
 
