@@ -1043,6 +1043,362 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
     return XLITE_HIP_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The direct-to-LDS kernel for 8-bit caches (head_dim 128, kv heads a multiple of 8). The cache bytes
+// travel as they are: one copy instruction moves 1 KiB = one position of the pass's 8 kv heads, and the
+// per-position scales follow by 4-byte copies. Bytes become fp16 (exactly) between the LDS read and the
+// matrix product, so a wave reads half the LDS bytes of the 16-bit kernel and writes none.
+// A step is 32 positions = two score tiles of 16. Stage: [K | V][32 positions][8 kv heads][128 bytes], then
+// the scales [K | V][kv head][32 positions]. The 256-byte bank window of LDS holds two kv heads' rows of a
+// position, so the XOR pattern of a position covers the 16-byte chunk (3 bits) and the kv head's low bit;
+// it is chosen so that the 16 positions of a score tile (K rows as the A operand, ds_read_b128) and the
+// 16 positions one half of the wave gathers for the second product (ds_read_b64_tr_b8) both land in 16
+// different 16-byte slots.
+//   K: lane (position = lane % 16, j = lane / 16) reads chunks j and j + 4 of its row; the 16 bytes of a
+//      chunk feed two k steps, and the query registers hold the head's elements in that same order.
+//   V: ds_read_b64_tr_b8 hands lane (column = lane % 16, j) the bytes of eight positions of one column:
+//      rows 0-3 = positions 4j .. 4j+3 of the first tile, rows 4-7 = the same of the second, which is the
+//      order in which the lane holds the probabilities after the first product (k = 32 positions).
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void dma_4b(uint32_t lds_addr, const void *src)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off\n\t"
+                 :: "s"(lds_addr), "v"(src) : "memory", "m0");
+}
+
+// four cache bytes -> four fp16 values (two registers), exactly
+template <int KVF>
+__device__ __forceinline__ void widen4(uint32_t w, uint32_t *lo, uint32_t *hi)
+{
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    if constexpr (KVF == XLITE_HIP_KV_FP8) {
+        *lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(static_cast<int>(w), 1.0f, false));
+        *hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(static_cast<int>(w), 1.0f, true));
+    } else {
+        // byte b ^ 0x80 = b + 128 as an unsigned byte u; 0x6400 | u reads as 1024 + u in fp16; minus 1152 leaves b
+        const h2_t bias = {static_cast<_Float16>(-1152.0f), static_cast<_Float16>(-1152.0f)};
+        const uint32_t x = w ^ 0x80808080u;
+        *lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u)) + bias);
+        *hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u)) + bias);
+    }
+}
+
+template <typename T, int KVF>
+__global__ void __launch_bounds__(kWaves * 64)
+decode_dma8_kernel(const DecodeMfmaParams p)
+{
+    constexpr int D = 128;
+    constexpr int MT = D / 16;
+    constexpr int STEP = 32;                     // positions per step
+    constexpr int HEADB = D;                     // bytes of one (position, kv head) row
+    constexpr int POSB = kWaves * HEADB;         // LDS bytes of one position: the 8 kv heads of the pass
+    constexpr int KBYTES = STEP * POSB;          // 32 KiB: the K half of a stage
+    constexpr int SCALEB = kWaves * STEP * 4;    // 1 KiB: the K scales of a stage
+    constexpr int STAGE = 2 * KBYTES + 2 * SCALEB;
+    constexpr int PER_WAVE = 9;                  // copies per wave and step: 4 K rows, 4 V rows, 64 scales
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE);
+    const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
+        static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t col = lane & 15;
+    const uint32_t jq = lane >> 4;
+
+    // XOR pattern of position `pos` of a step: chunk bits, kv-head bit
+    auto pat_chunk = [](uint32_t pos) { return pos & 7u; };
+    auto pat_head = [](uint32_t pos) { return ((pos >> 3) ^ (pos >> 4)) & 1u; };
+    auto slot_off = [&](uint32_t pos, uint32_t head, uint32_t chunk) {
+        return pos * POSB + (((head ^ pat_head(pos)) << 3 | (chunk ^ pat_chunk(pos))) << 4);
+    };
+    // read roles (this wave's kv head = `wave` inside the pass)
+    uint32_t kr_off[2][2];
+#pragma unroll
+    for (int tl = 0; tl < 2; tl++) {
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            kr_off[tl][r] = slot_off(16 * tl + col, wave, jq + 4 * r);
+        }
+    }
+    uint32_t vr_off[MT];
+    {
+        const uint32_t row = col >> 1;   // row of the 8 x 16 byte block this lane points at
+        const uint32_t pos = row < 4 ? 4 * jq + row : 16 + 4 * jq + (row - 4);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            vr_off[mt] = KBYTES + slot_off(pos, wave, mt) + ((lane & 1) << 3);
+        }
+    }
+    const uint32_t sc_off = 2 * KBYTES + (wave * STEP + 4 * jq) * 4;   // K scales of the first tile's rows
+    // copy roles: wave w moves positions 4w .. 4w+3 (K and V). Lane = slot (kv head, chunk) of the position's
+    // 1 KiB; the slot receives the chunk the pattern assigns to it.
+    uint32_t c_voff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t pos = 4 * wave + i;
+        c_voff[i] = ((lane >> 3) ^ pat_head(pos)) * HEADB + (((lane & 7u) ^ pat_chunk(pos)) << 4);
+    }
+    // scale copies: waves 0-3 the K scales, 4-7 the V scales; a wave moves two kv heads x 32 positions
+    const uint32_t sc_head = 2 * (wave & 3) + (lane >> 5);
+    const uint32_t sc_pos = lane & 31;
+    const float *sc_src = wave < 4 ? p.k_scale : p.v_scale;
+    const uint32_t sc_dst = 2 * KBYTES + (wave >> 2) * SCALEB + (wave & 3) * 256;
+
+    const uint32_t g_valid = p.group < 16 ? p.group : 16;
+    const uint32_t row_bytes = p.n_kv_heads * HEADB;
+
+    DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
+    split.scan();
+    if (split.total == 0) {
+        return;
+    }
+
+    auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool whole, uint32_t pslot, bool first_piece,
+                           int4 meta) {
+        const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
+        const uint32_t n_steps = ceil_div(t1 - t0, static_cast<uint32_t>(STEP));
+        const uint32_t blk0 = t0 / p.block_size;
+        // Q^T as the B operand, as fp16: k step 2r + h of the first product covers the elements
+        // [16 (j + 4r) + 8h, + 8) of the head
+        uint4 qreg[4];
+        auto load_q = [&](uint32_t kv0) {
+            const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
+                                   static_cast<uint64_t>((kv0 + wave) * p.group + col) * D;
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + 16 * (jq + 4 * (ks >> 1)) + 8 * (ks & 1))
+                                         : make_uint4(0, 0, 0, 0);
+            }
+        };
+        auto q_to_fp16 = [&]() {
+            if constexpr (!std::is_same<T, FP16>::value) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) {
+                    uint32_t *w = reinterpret_cast<uint32_t *>(&qreg[ks]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        w[j] = FP16::pack(T::to_f32(static_cast<uint16_t>(w[j] & 0xffff)), T::to_f32(static_cast<uint16_t>(w[j] >> 16)));
+                    }
+                }
+            }
+        };
+        load_q(0);
+        {
+            const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
+            for (uint32_t i = threadIdx.x; i < nblk; i += kWaves * 64) {
+                tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
+            }
+            if (first_piece && threadIdx.x == 0) {
+                reinterpret_cast<int4 *>(p.part_meta)[tok] = meta;
+            }
+            __syncthreads();
+        }
+
+        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += kWaves) {
+            const uint32_t kvh = kv0 + wave;
+            const uint32_t head0 = kvh * p.group;
+
+            if (kv0 > 0) {
+                load_q(kv0);
+            }
+            // complete these loads before any copy is issued: memory operations finish in order
+            q_to_fp16();
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+            }
+            f32x4_t O[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                O[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            }
+            float m_run = -INFINITY, l_run = 0.f;
+
+            // copies of one step into stage step % 2. Each half of a step (16 positions from a multiple of 16)
+            // lies in one block (block_size % 16 == 0). Positions at or beyond the end re-read the last valid one.
+            auto issue = [&](uint32_t step) {
+                const uint32_t ts = t0 + step * STEP;   // <= t1 - 1
+                const uint32_t tl = t1 - 1;
+                const uint32_t st = smem_addr + (step & 1) * STAGE;
+                uint64_t row0[2];
+                uint32_t max_i[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const uint32_t hs = min(ts + 16 * h, tl);
+                    const uint32_t blk = hs / p.block_size, off = hs % p.block_size;
+                    const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
+                    row0[h] = static_cast<uint64_t>(phys) * p.block_size + off;
+                    max_i[h] = ts + 16 * h > tl ? 0u : min(tl - (ts + 16 * h), 15u);
+                }
+                const uint32_t half = wave >> 2;
+                const uint64_t my_row0 = half ? row0[1] : row0[0];
+                const uint32_t my_max = half ? max_i[1] : max_i[0];
+                const char *kb = static_cast<const char *>(p.k_cache) + my_row0 * row_bytes + kv0 * HEADB;
+                const char *vb = static_cast<const char *>(p.v_cache) + my_row0 * row_bytes + kv0 * HEADB;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t pos = 4 * wave + i;
+                    const uint32_t src = min(pos & 15u, my_max) * row_bytes;   // uniform
+                    dma_1k(st + pos * POSB, c_voff[i], kb + src);
+                    dma_1k(st + KBYTES + pos * POSB, c_voff[i], vb + src);
+                }
+                {
+                    const bool hi = sc_pos >= 16;
+                    const uint64_t r0 = hi ? row0[1] : row0[0];
+                    const uint32_t mi = hi ? max_i[1] : max_i[0];
+                    const float *src = sc_src + (r0 + min(sc_pos & 15u, mi)) * p.n_kv_heads + kv0 + sc_head;
+                    dma_4b(st + sc_dst, src);
+                }
+            };
+            auto compute = [&](uint32_t step) {
+                const uint32_t t = t0 + step * STEP;
+                const unsigned char *stage = smem + (step & 1) * STAGE;
+                // ---- S^T = K . Q^T: two tiles of 16 positions x 16 heads ------------------------------------
+                f32x4_t S[2];
+#pragma unroll
+                for (int tl = 0; tl < 2; tl++) {
+                    S[tl] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int r = 0; r < 2; r++) {
+                        const uint4 raw = *reinterpret_cast<const uint4 *>(stage + kr_off[tl][r]);
+                        uint4 a0, a1;
+                        widen4<KVF>(raw.x, &a0.x, &a0.y);
+                        widen4<KVF>(raw.y, &a0.z, &a0.w);
+                        widen4<KVF>(raw.z, &a1.x, &a1.y);
+                        widen4<KVF>(raw.w, &a1.z, &a1.w);
+                        S[tl] = Mfma16<FP16>::run(a0, qreg[2 * r], S[tl]);
+                        S[tl] = Mfma16<FP16>::run(a1, qreg[2 * r + 1], S[tl]);
+                    }
+                }
+                // V^T bytes do not depend on the softmax: fetch them now
+                typedef int v2i_t __attribute__((ext_vector_type(2)));
+                v2i_t vraw[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    typedef v2i_t __attribute__((address_space(3))) * lds_tr_ptr;
+                    vraw[mt] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_tr_ptr)(const_cast<unsigned char *>(stage) + vr_off[mt]));
+                }
+                float ksc[8], vsc[8];
+                {
+                    const float4 k0 = *reinterpret_cast<const float4 *>(stage + sc_off);
+                    const float4 k1 = *reinterpret_cast<const float4 *>(stage + sc_off + 64);
+                    const float4 v0 = *reinterpret_cast<const float4 *>(stage + sc_off + SCALEB);
+                    const float4 v1 = *reinterpret_cast<const float4 *>(stage + sc_off + SCALEB + 64);
+                    ksc[0] = k0.x, ksc[1] = k0.y, ksc[2] = k0.z, ksc[3] = k0.w;
+                    ksc[4] = k1.x, ksc[5] = k1.y, ksc[6] = k1.z, ksc[7] = k1.w;
+                    vsc[0] = v0.x, vsc[1] = v0.y, vsc[2] = v0.z, vsc[3] = v0.w;
+                    vsc[4] = v1.x, vsc[5] = v1.y, vsc[6] = v1.z, vsc[7] = v1.w;
+                }
+                // ---- online softmax; lane holds positions t + 16 tl + 4 jq + e of head `col` ------------------
+                float sv[8];
+                bool ok[8];
+                float mx = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    ok[i] = (t + 16 * (i >> 2) + 4 * jq + (i & 3)) < t1;
+                    const float v = ok[i] ? S[i >> 2][i & 3] * kLog2e * ksc[i] : -INFINITY;   // also drops the padding's NaN
+                    sv[i] = v;
+                    mx = fmaxf(mx, v);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                const float m_new = fmaxf(m_run, mx);
+                const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = fast_exp2(m_run - m_safe);
+                m_run = m_new;
+                float pe[8];
+                float psum = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float x = fast_exp2(sv[i] - m_safe);
+                    psum += x;
+                    pe[i] = ok[i] ? x * vsc[i] : 0.f;
+                }
+                l_run = l_run * alpha + psum;
+                const uint4 pb = make_uint4(FP16::pack(pe[0], pe[1]), FP16::pack(pe[2], pe[3]),
+                                            FP16::pack(pe[4], pe[5]), FP16::pack(pe[6], pe[7]));
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        O[mt][0] *= alpha;
+                        O[mt][1] *= alpha;
+                        O[mt][2] *= alpha;
+                        O[mt][3] *= alpha;
+                    }
+                }
+                // ---- O^T += V^T . P^T (k = the 32 positions) -------------------------------------------------
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    uint4 a;
+                    widen4<KVF>(static_cast<uint32_t>(vraw[mt].x), &a.x, &a.y);
+                    widen4<KVF>(static_cast<uint32_t>(vraw[mt].y), &a.z, &a.w);
+                    O[mt] = Mfma16<FP16>::run(a, pb, O[mt]);
+                }
+            };
+
+            // every copy is unconditional (steps past the end copy the last step again, into the stage
+            // nobody reads any more), so the wait counts are exact
+            const uint32_t last = n_steps - 1;
+            issue(0);
+            issue(min(1u, last));
+            for (uint32_t step = 0; step < n_steps; step++) {
+                dma_wait<PER_WAVE>();   // this wave's share of `step` has landed
+                __syncthreads();        // ... and everybody else's
+                compute(step);
+                __syncthreads();        // the stage is free again
+                issue(min(step + 2, last));
+            }
+            dma_wait<0>();
+            __syncthreads();
+
+            float l_tot = l_run + __shfl_xor(l_run, 16);
+            l_tot += __shfl_xor(l_tot, 32);
+            if (col < g_valid) {
+                if (whole) {
+                    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+                    uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        uint2 o;
+                        o.x = T::pack(O[mt][0] * inv, O[mt][1] * inv);
+                        o.y = T::pack(O[mt][2] * inv, O[mt][3] * inv);
+                        *reinterpret_cast<uint2 *>(dst + mt * 16 + jq * 4) = o;
+                    }
+                } else {
+                    const uint64_t slot = static_cast<uint64_t>(pslot) * p.n_heads + head0 + col;
+                    float *dst = p.part_acc + slot * D;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
+                    }
+                    if (jq == 0) {
+                        *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
+                    }
+                }
+            }
+        }
+    };
+
+    split.for_each_segment(run_segment);
+}
+
+template <typename T, int KVF>
+int launch_dma8(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
+{
+    const size_t lds = 2 * static_cast<size_t>(2 * 32 * kWaves * 128 + 2 * kWaves * 32 * 4) +
+                       (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
+    auto kernel = decode_dma8_kernel<T, KVF>;
+    if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
+        return rc;
+    }
+    dim3 grid(n_workgroups, 1, 1);
+    kernel<<<grid, kWaves * 64, lds, stream>>>(p);
+    XL_LAUNCH_CHECK();
+    return XLITE_HIP_OK;
+}
+
 template <typename T, int D, int KVF, bool MULTI_SUB>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
@@ -1100,6 +1456,12 @@ uint32_t decode_mfma_slice_units() { return kSplitSeqCap; }
 bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
 {
     return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0;
+}
+
+// decode_dma8_kernel: head_dim 128, 8-bit cache, kv heads a multiple of 8
+bool decode_dma8_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
+{
+    return head_dim == 128 && kv_dtype != XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0;
 }
 
 // The chunk the kernel really uses is the batch's total step count over the number of workgroups, which the
@@ -1179,6 +1541,12 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
         int rc;
         if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
+        } else if (decode_dma8_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+            if (a.kv_dtype == XLITE_HIP_KV_FP8) {
+                rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_FP8>(stream, p, grid_x) : launch_dma8<FP16, XLITE_HIP_KV_FP8>(stream, p, grid_x);
+            } else {
+                rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_INT8>(stream, p, grid_x) : launch_dma8<FP16, XLITE_HIP_KV_INT8>(stream, p, grid_x);
+            }
         } else if (a.head_dim == 128) {
             rc = bf ? launch_fmt<BF16, 128>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 128>(stream, p, grid_x, a.kv_dtype);
         } else {

@@ -214,6 +214,20 @@ def test_decode_quantised_kv_ragged_batch(rt, kv_dtype):
 
 
 @pytest.mark.parametrize("kv_dtype", KV_DTYPES)
+@pytest.mark.parametrize("model", [(32, 8, 16, torch.float16), (16, 16, 32, torch.bfloat16), (128, 8, 128, torch.bfloat16),
+                                   (8, 8, 48, torch.float16), (24, 8, 16, torch.bfloat16)])
+def test_decode_quantised_kv_byte_streaming_kernel_shapes(rt, kv_dtype, model):
+    """Decode batches on the kernel that copies the cache bytes straight into LDS (head_dim 128, kv heads a multiple
+    of 8): both activation types, one and two passes over the kv heads, groups of 1, 3, 4 and 16 query heads, blocks
+    of 16, 32 and 48 positions (a step of 32 positions then spans two blocks), and visible ranges around every
+    multiple of 16 and 32 (the padding rows of the last step re-read the last position)."""
+    nH, nKV, bs, dtype = model
+    ctx = [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 96, 97, 1000, 4097]
+    w = quantised(generic_case(62, [1] * len(ctx), [c - 1 for c in ctx], nH, nKV, 128, bs, dtype), kv_dtype)
+    check(run_attention(rt, w), oracle_attention(w), max_abs=MAX_ABS_INT8)
+
+
+@pytest.mark.parametrize("kv_dtype", KV_DTYPES)
 @pytest.mark.parametrize("model", [(32, 8, 128, 128, torch.bfloat16), (14, 2, 64, 128, torch.float16), (28, 4, 128, 16, torch.bfloat16),
                                    (64, 2, 128, 128, torch.bfloat16), (8, 2, 128, 20, torch.float16)])
 @pytest.mark.parametrize("work", [([0], [77]), ([128], [300]), ([0] * 4, [189, 65, 13, 545]), ([2047, 1500, 0, 900], [1, 1, 300, 1]),
