@@ -30,12 +30,12 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
-MEASURED_TRAFFIC_BYTES = {"c2": 1080255515, "c3": 302359634, "c4": 313334697, "c5": 1623923510}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080255515, "c3": 302359634, "c4": 313334697, "c5": 1623764049}
 # where each constant comes from: the committed counter summary whose "HBM traffic per launch" line holds it
 TRAFFIC_SOURCE = {"c2": "profiles/decode_dma_kernel_c2_llama3_8b_b64_ctx4096.md",
                   "c3": "profiles/prefill_kernel_c3_qwen25_7b_chunked.md",
                   "c4": "profiles/mla_decode_kernel_c4_deepseek_r1_b32.md",
-                  "c5": "profiles/decode_mfma_kernel_int8_c5_llama3_8b_b128_ragged.md"}
+                  "c5": "profiles/decode_dma8_kernel_int8_c5_llama3_8b_b128_ragged.md"}
 
 
 def _traffic(key):
@@ -232,7 +232,7 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
         "attention_ms_dist": _launch_dist(torch, attn),
-        "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_mfma_kernel (+ merge_meta_kernel)", "achieved": round(achieved, 2),
+        "roofline": {"bound": "hbm", "kernel": "decode_dma_kernel / decode_dma8_kernel / decode_mfma_kernel (+ merge_meta_kernel)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      **_traffic(name.split()[0]), "algorithmic_bytes_per_launch": int(alg_bytes)},
         "cpu_baseline": cpu,

@@ -325,9 +325,10 @@ prefill_kernel(const PrefillParams p)
         }
     };
 
-    // The matrix pipe and the vector ALU of a SIMD do not run at the same time, so what can be hidden is
-    // LDS latency: a step's K operands are fetched during the previous step's second product, its V^T
-    // operands during its own softmax.
+    // A wave issues in order, so its own softmax does not overlap its own products; what the wave itself can
+    // hide is LDS latency: a step's K operands are fetched during the previous step's second product, its V^T
+    // operands during its own softmax. (The SIMD's other wave overlaps the rest: its products run while this
+    // wave's vector instructions issue.)
     uint4 kop[KS];
     auto fetch_k = [&](uint32_t stage_off, int h) {
         const unsigned char *base = smem + stage_off + h * 32 * ROWB + k_row;
@@ -343,8 +344,7 @@ prefill_kernel(const PrefillParams p)
     auto step = [&](uint32_t stage_off, int h, uint32_t j0, uint32_t next_stage_off, int next_h, auto mask_tag) {
         constexpr bool MASK = decltype(mask_tag)::value;
         // ---- S^T = K . Q^T (one accumulation chain: the SIMD's other wave fills the issue gaps between
-        // dependent products, and a second chain would cost 16 additions on the vector ALU, which the matrix
-        // pipe cannot overlap)
+        // dependent products, and a second chain would cost 16 more vector instructions of this wave's issue time)
         f32x16_t S;
 #pragma unroll
         for (int k = 0; k < 16; k++) {
