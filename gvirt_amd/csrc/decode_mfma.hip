@@ -131,16 +131,25 @@ __device__ __forceinline__ uint4 widen(const uint2 &raw, Fp8Tag)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// XOR pattern applied to the 16-byte chunk index of LDS row `row`. One pattern serves both read
-// shapes: 16 lanes reading the same chunk of 16 consecutive rows (K as MFMA A operand) land in 16
-// different chunk slots, and 8 consecutive rows read as 32-byte pieces (transposing V read) land
-// in 8 different 32-byte slots of the 256-byte bank window.
+// XOR pattern applied to the 16-byte chunk index of LDS row `row`. One pattern serves both read shapes of a
+// step's 16 rows. K as the MFMA A operand (ds_read_b128, lane = 16 j + row reads chunk 4 ks + j of its row): the
+// hardware serves the instruction in four passes of 16 lanes, and a pass is lanes 0-3, 12-15, 20-23 and 24-27, then
+// 4-11, 16-19 and 28-31 (the upper half of the wave likewise) - rows 0-3 and 12-15 of one chunk next to rows 4-11
+// of its neighbour -, so those two row sets must own complete pairs of slots (2k, 2k + 1) of the 256-byte bank
+// window. (Measured: with a pattern that only gives 16 consecutive lanes 16 different slots every such read took 8
+// cycles instead of 4.) The transposing V read (ds_read_b64_tr_b16, passes of 32 lanes = 8 consecutive rows read as
+// 32-byte pieces) needs those 8 rows in 8 different 32-byte slots. head_dim 64: two rows share a bank window and the
+// pattern has three bits.
 template <int D>
 __device__ __forceinline__ uint32_t swizzle(uint32_t row)
 {
-    constexpr uint32_t CH = D / 8, R256 = 256 / (D * 2);
-    const uint32_t rr = row / R256;
-    return ((rr & (CH / 2 - 1)) << 1) | ((rr / (CH / 2)) & 1);
+    if constexpr (D == 128) {
+        const uint32_t hi = (row >> 3) & 1;
+        return (((row & 7) ^ (hi << 2)) << 1) | hi;
+    } else {
+        static_assert(D == 64, "patterns exist for head_dim 128 and 64");
+        return row & 6;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -51,10 +51,18 @@ constexpr uint32_t kTblCap = 3000;     // block-table entries of a segment stage
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 
 // XOR patterns for the 16-byte chunk index inside a row.
-// Latent rows (1024 bytes, every row starts at bank 0): low four chunk bits. The 16 rows that one
-// ds_read_b128 pass touches get 16 different chunk slots, and the 8 rows that one transposing pass touches
-// get 8 different 32-byte groups.
-__device__ __forceinline__ uint32_t swz_kc(uint32_t row) { return ((row & 7) << 1) | ((row >> 3) & 1); }
+// Latent rows (1024 bytes, every row starts at bank 0): low four chunk bits. The hardware serves a ds_read_b128
+// in four passes of 16 lanes, and a pass is not 16 consecutive lanes: lanes 0-3, 12-15, 20-23 and 24-27 go together,
+// then 4-11, 16-19 and 28-31 (the upper half of the wave likewise). With lane = 16 j + row that is rows 0-3 and 12-15
+// of one 16-byte column group next to rows 4-11 of its neighbour, so the rows 0-3 and 12-15 must own complete pairs
+// of slots (2k, 2k + 1): measured with the pattern ((row & 7) << 1) | (row >> 3), which gives 16 consecutive lanes
+// 16 different slots, every K read took 8 cycles instead of 4. The 8 rows that one transposing pass (32 lanes)
+// touches get 8 different 32-byte groups.
+__device__ __forceinline__ uint32_t swz_kc(uint32_t row)
+{
+    const uint32_t hi = (row >> 3) & 1;
+    return (((row & 7) ^ (hi << 2)) << 1) | hi;
+}
 // Rotary rows (128 bytes, two per bank window): low three chunk bits; rows of equal parity differ.
 __device__ __forceinline__ uint32_t swz_pe(uint32_t row) { return (row >> 1) & 7; }
 
@@ -117,7 +125,7 @@ mla_decode_kernel(const MlaDecodeParams p)
     auto set_roles = [&](uint32_t ln) {
         const uint32_t c4 = ln & 15, g = ln >> 4;
         gi4 = g * 4;
-        kc_voff = ((ln & ~15u) | ((ln & 15u) ^ (8 * (wave & 1) + ((wave >> 1) & 1)))) << 4;
+        kc_voff = ((ln & ~15u) | ((ln & 15u) ^ swz_kc(4 * wave))) << 4;   // (row 4 wave + i: this ^ (i << 5))
         pe_row = (wave & (PE_WAVES - 1)) * 8 + (ln >> 3);
         pe_voff = ((ln & 7u) ^ swz_pe(pe_row)) << 4;
         kx = (g ^ swz_kc(c4)) << 4;
