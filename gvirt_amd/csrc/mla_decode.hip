@@ -286,29 +286,27 @@ mla_decode_kernel(const MlaDecodeParams p)
 
             // ---- S^T = K . Q^T of one step: two tiles of 16 positions x 16 heads, 18 k-steps of 32 elements.
             // The two accumulation chains alternate; operands are fetched kAhead products ahead.
-            auto qk = [&](uint32_t step, f32x4_t (&S)[2]) {
+            // The first kAhead operands are fetched by `qk_fetch`, which the loop calls right behind the step's barrier:
+            // their latency then overlaps the address arithmetic of the copies issued in between.
+            auto rd_k = [&](uint32_t soff, int i) {
+                const int ks = i >> 1, mt = i & 1;
+                return ks < KS_C
+                           ? *reinterpret_cast<const uint4 *>(smem + soff + k_row + (((ks & 3) << 6) ^ kx) + ((ks >> 2) << 8) + mt * 16 * KC_ROWB)
+                           : *reinterpret_cast<const uint4 *>(smem + soff + p_row + (((ks - KS_C) << 6) ^ px) + mt * 16 * PE_ROWB);
+            };
+            auto qk_fetch = [&](uint32_t step, uint4 (&a)[kAhead]) {
                 const uint32_t soff = (step % kStages) * STAGE_BYTES;
-                uint32_t xk[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    xk[j] = soff + k_row + ((j << 6) ^ kx);
+                for (int i = 0; i < kAhead; i++) {
+                    a[i] = rd_k(soff, i);
                 }
-                const uint32_t xp = soff + p_row;
-                auto rd_k = [&](int i) {
-                    const int ks = i >> 1, mt = i & 1;
-                    return ks < KS_C
-                               ? *reinterpret_cast<const uint4 *>(smem + xk[ks & 3] + ((ks >> 2) << 8) + mt * 16 * KC_ROWB)
-                               : *reinterpret_cast<const uint4 *>(smem + xp + (((ks - KS_C) << 6) ^ px) + mt * 16 * PE_ROWB);
-                };
+            };
+            auto qk = [&](uint32_t step, f32x4_t (&S)[2], uint4 (&a)[kAhead]) {
+                const uint32_t soff = (step % kStages) * STAGE_BYTES;
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
                     S[0][k] = 0.f;
                     S[1][k] = 0.f;
-                }
-                uint4 a[kAhead];
-#pragma unroll
-                for (int i = 0; i < kAhead; i++) {
-                    a[i] = rd_k(i);
                 }
 #pragma unroll
                 for (int i = 0; i < 2 * (KS_C + KS_R); i++) {
@@ -316,7 +314,7 @@ mla_decode_kernel(const MlaDecodeParams p)
                                                                      __builtin_bit_cast(bf16x8_t, qreg[i >> 1]),
                                                                      S[i & 1], 0, 0, 0);
                     if (i + kAhead < 2 * (KS_C + KS_R)) {
-                        a[i % kAhead] = rd_k(i + kAhead);
+                        a[i % kAhead] = rd_k(soff, i + kAhead);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -331,6 +329,24 @@ mla_decode_kernel(const MlaDecodeParams p)
                 const uint32_t soff = (step % kStages) * STAGE_BYTES;
                 const uint32_t lane_pos = t + gi4;
                 float mx = -INFINITY;
+                // the first transposed operands of the second product do not depend on the softmax: in flight during it
+                typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+                uint32_t xv[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    xv[j] = soff + (vr_off ^ (j << 5));
+                }
+                auto rd_v = [&](int dt, int rd) {
+                    unsigned char *ptr = smem + xv[dt & 7] + ((dt >> 3) << 8) + rd * 16 * KC_ROWB;
+                    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
+                };
+                uint2 v[VB][2];
+#pragma unroll
+                for (int d = 0; d < VB - 1; d++) {
+                    v[d][0] = rd_v(d, 0);
+                    v[d][1] = rd_v(d, 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
                 // the softmax runs at a raised wave priority: its vector instructions go ahead of the products of
                 // the SIMD's other wave (1-2 % on the step; raising it around the products instead gains nothing)
                 __builtin_amdgcn_s_setprio(2);
@@ -408,22 +424,6 @@ mla_decode_kernel(const MlaDecodeParams p)
                 // which is the order the lane's own probabilities already have
                 const uint4 pb = make_uint4(pw[0], pw[1], pw[2], pw[3]);
                 __builtin_amdgcn_s_setprio(0);
-                typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
-                uint32_t xv[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    xv[j] = soff + (vr_off ^ (j << 5));
-                }
-                auto rd_v = [&](int dt, int rd) {
-                    unsigned char *ptr = smem + xv[dt & 7] + ((dt >> 3) << 8) + rd * 16 * KC_ROWB;
-                    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
-                };
-                uint2 v[VB][2];
-#pragma unroll
-                for (int d = 0; d < VB - 1; d++) {
-                    v[d][0] = rd_v(d, 0);
-                    v[d][1] = rd_v(d, 1);
-                }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++) {
@@ -472,8 +472,11 @@ mla_decode_kernel(const MlaDecodeParams p)
                     dma_wait<(kDepth - 1) * 4>();
                 }
                 __syncthreads();            // ... and everybody else's; the stage issued into below is free
+                uint4 a[kAhead];
+                qk_fetch(it, a);
+                __builtin_amdgcn_sched_barrier(0);
                 issue(min(it + kDepth, last));
-                qk(it, S);
+                qk(it, S, a);
                 softmax_pv(it, S);
             }
             dma_wait<0>();
