@@ -538,26 +538,38 @@ bool prefill_mfma_supported(const AttentionArgs &a)
            a.n_heads % a.n_kv_heads == 0;
 }
 
-// KV splits per M tile: with fewer workgroups than compute units, the split count that minimises
-// (rounds of workgroups over the chip) / splits, each split keeping at least kMinSplitTiles tiles of the
-// longest possible context.
+// KV splits per M tile. The cost of s splits, in units of one workgroup walking the longest possible context:
+//     (rounds of workgroups over the chip) x (1 / s of the walk + a workgroup's set-up and drain, about four KV
+//     tiles' time) + s x (the partials' trip through memory: fp32 O per row and head, written and read back)
+// With fewer workgroups than compute units that is the old rule (rounds / s); it also cuts the last round of a
+// batch that fills the chip once and a bit (a chunk's tail: 292 workgroups on 256 compute units run two rounds,
+// three splits run four rounds of a third each). Each split keeps at least kMinSplitTiles tiles of the longest context.
 uint32_t prefill_mfma_pick_splits(uint32_t total_tokens, uint32_t group, uint32_t batch, uint32_t n_kv_heads,
-                                  uint32_t max_ctx)
+                                  uint32_t max_ctx, uint32_t head_dim)
 {
     const uint64_t base = (static_cast<uint64_t>(ceil_div(total_tokens * group, static_cast<uint32_t>(kMTile))) + batch) *
                           n_kv_heads;
     const uint64_t n_cu = 256;
     const uint32_t cap = min(64u, max_ctx / (kMinSplitTiles * BN));
-    if (base >= n_cu || cap <= 1) {
+    if (cap <= 1) {
         return 1;
     }
+    constexpr double kTileUs = 2.2;         // one KV tile of 64 positions, measured on the chunked-prefill shape
+    constexpr double kPartialGBs = 4000.0;  // what the partials' round trip sustains
+    const double walk_us = static_cast<double>(max_ctx) / BN * kTileUs;
+    const double setup = 4.0 * kTileUs / walk_us;
+    const double part = static_cast<double>(total_tokens) * group * n_kv_heads * head_dim * 8.0 / (kPartialGBs * 1e3) / walk_us;
+    auto cost = [&](uint32_t n) {
+        const double rounds = static_cast<double>((base * n + n_cu - 1) / n_cu);
+        return rounds * (1.0 / n + setup) + (n > 1 ? part * n : 0.0);
+    };
     uint32_t best = 1;
-    double best_cost = 1.0;   // base < n_cu: one round
-    for (uint32_t s = 2; s <= cap; s++) {
-        const double cost = static_cast<double>((base * s + n_cu - 1) / n_cu) / s;
-        if (cost < best_cost * 0.95) {
-            best = s;
-            best_cost = cost;
+    double best_cost = cost(1);
+    for (uint32_t n = 2; n <= cap; n++) {
+        const double c = cost(n);
+        if (c < best_cost * (best == 1 ? 0.95 : 1.0)) {   // splitting at all has to pay clearly
+            best = n;
+            best_cost = c;
         }
     }
     return best;
@@ -566,7 +578,7 @@ uint32_t prefill_mfma_pick_splits(uint32_t total_tokens, uint32_t group, uint32_
 size_t prefill_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                     uint32_t batch, uint32_t max_ctx)
 {
-    const uint32_t splits = prefill_mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx);
+    const uint32_t splits = prefill_mfma_pick_splits(total_tokens, n_heads / n_kv_heads, batch, n_kv_heads, max_ctx, head_dim);
     return splits <= 1 ? 0 : partial_bytes(total_tokens, n_heads, head_dim, splits);
 }
 
@@ -594,7 +606,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
     p.n_heads = a.n_heads;
     p.skip_single = a.rows_mode == kSkipSingle ? 1u : 0u;
-    uint32_t splits = prefill_mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, a.max_num_block * a.block_size);
+    uint32_t splits = prefill_mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, a.max_num_block * a.block_size, a.head_dim);
     if (a.workspace == nullptr || a.workspace_bytes < partial_bytes(a.total_tokens, a.n_heads, a.head_dim, splits)) {
         splits = 1;   // no scratch: every M tile walks its whole KV range
     }
