@@ -169,7 +169,26 @@ prefill_kernel(const PrefillParams p)
         return static_cast<uint32_t>((static_cast<uint64_t>(p.query_start_loc[i]) * G) / kMTile) + i;
     };
     uint32_t seq = 0;
-    {
+    int32_t qlen, clen, qstart;
+    uint32_t mt;
+    // (the condition goes through readfirstlane: left to itself the compiler folds it into the per-lane `lane < batch`
+    // below and then treats everything behind the join as divergent)
+    if (__builtin_amdgcn_readfirstlane(p.batch <= 64 ? 1 : 0)) {
+        // one round of loads instead of a chain of them: lane i fetches what the batch says about sequence i. The ids
+        // are nondecreasing, so the sequences that start at or before `tid` are a prefix of the batch, and the owner
+        // is its last one; its lengths are then read from the owner's lane.
+        const bool in_batch = lane < p.batch;
+        const int32_t my_start = in_batch ? p.query_start_loc[lane] : 0;
+        const int32_t my_len = in_batch ? p.lens[lane] : 0;
+        const int32_t my_cached = in_batch ? p.cached_lens[lane] : 0;
+        const uint32_t fid = in_batch ? static_cast<uint32_t>((static_cast<uint64_t>(my_start) * G) / kMTile) + lane : 0xffffffffu;
+        const uint64_t started = __ballot(fid <= tid);
+        seq = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(__builtin_popcountll(started))) - 1;
+        qstart = __builtin_amdgcn_readlane(my_start, static_cast<int>(seq));
+        qlen = __builtin_amdgcn_readlane(my_len, static_cast<int>(seq));
+        clen = __builtin_amdgcn_readlane(my_cached, static_cast<int>(seq));
+        mt = tid - static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(fid), static_cast<int>(seq)));
+    } else {
         uint32_t hi = p.batch;   // first_id(seq) <= tid < first_id(hi); first_id(0) == 0
         while (hi - seq > 1) {
             const uint32_t mid = (seq + hi) >> 1;
@@ -179,21 +198,22 @@ prefill_kernel(const PrefillParams p)
                 hi = mid;
             }
         }
+        seq = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(seq)));   // the same in every lane, said so
+        mt = tid - first_id(seq);
+        qlen = p.lens[seq];
+        clen = p.cached_lens[seq];
+        qstart = p.query_start_loc[seq];
     }
-    const uint32_t mt = tid - first_id(seq);
-    const int32_t qlen = p.lens[seq];
     if (p.skip_single && qlen == 1) {
         // the decode kernel writes this row; the merge of this kernel's partials must leave it alone
         if (p.part_cnt != nullptr && mt == 0 && blockIdx.y == 0 && threadIdx.x < G) {
-            p.part_cnt[static_cast<uint64_t>(p.query_start_loc[seq]) * p.n_heads + kvh * G + threadIdx.x] = 0;
+            p.part_cnt[static_cast<uint64_t>(qstart) * p.n_heads + kvh * G + threadIdx.x] = 0;
         }
         return;
     }
     if (qlen <= 0 || mt >= ceil_div(static_cast<uint32_t>(qlen) * G, static_cast<uint32_t>(kMTile))) {
         return;
     }
-    const int32_t clen = p.cached_lens[seq];
-    const int32_t qstart = p.query_start_loc[seq];
     const uint32_t m_rows = static_cast<uint32_t>(qlen) * G;
     const uint32_t m_first = mt * kMTile;
     const uint32_t m_last = min(m_rows, m_first + kMTile) - 1;
@@ -217,11 +237,6 @@ prefill_kernel(const PrefillParams p)
     const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
     const uint32_t row_bytes = p.n_kv_heads * ROWB;
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE);
-    for (uint32_t i = __umulhi(first_tile * BN, p.block_magic) + threadIdx.x;
-         i <= __umulhi(min(n_tiles * BN, range_end) - 1, p.block_magic); i += kThreads) {
-        tbl_lds[i] = static_cast<uint32_t>(table[i]);
-    }
-    __syncthreads();
 
     // ---- this lane's M row ---------------------------------------------------------------------------
     const uint32_t m = m_first + wave * 32 + col;
@@ -240,6 +255,12 @@ prefill_kernel(const PrefillParams p)
         for (int ks = 0; ks < KS; ks++) {
             qreg[ks] = m_valid ? *reinterpret_cast<const uint4 *>(src + ks * 16 + half * 8) : make_uint4(0, 0, 0, 0);
         }
+        // the block-table entries of this workgroup's range go to LDS while the query loads are in flight
+        for (uint32_t i = __umulhi(first_tile * BN, p.block_magic) + threadIdx.x;
+             i <= __umulhi(min(n_tiles * BN, range_end) - 1, p.block_magic); i += kThreads) {
+            tbl_lds[i] = static_cast<uint32_t>(table[i]);
+        }
+        __syncthreads();
         // complete these loads before any copy is issued: memory operations finish in order, and their
         // first use is inside the streaming loop
 #pragma unroll
@@ -484,23 +505,45 @@ prefill_kernel(const PrefillParams p)
     dma_wait<0>();
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if (m_valid) {
-        // O^T lane layout: column = M row, register k of tile dt = element 32 dt + 8 (k / 4) + 4 half + k % 4
-        const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head;
-        if (n_splits == 1) {
-            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-            uint16_t *dst = p.out + static_cast<uint64_t>(tok) * p.out_tok_stride + static_cast<uint64_t>(head) * D;
+    // O^T lane layout: column = M row, register k of tile dt = element 32 dt + 8 (k / 4) + 4 half + k % 4
+    if (n_splits == 1) {
+        // Final values leave through LDS (stored straight from this layout a lane writes 8 bytes of its own row per
+        // instruction, 64 scattered pieces: 4 us per workgroup): every wave lays its 32 rows out row-major in its
+        // own part of the stage memory and stores them 16 bytes per lane, a row by consecutive lanes.
+        constexpr int PITCH = ROWB + 8;     // rows 8 bytes apart in the bank window: the 32 lanes of a write pass differ
+        constexpr int LPR = ROWB / 16;      // lanes per row of the store
+        constexpr int RPI = 64 / LPR;       // rows per store instruction
+        __syncthreads();   // every wave has left the loop and nothing is in flight: the stages are free
+        unsigned char *mine = smem + wave * (32 * PITCH);
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
+        for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
-                for (int kg = 0; kg < 4; kg++) {
-                    uint2 o;
-                    o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
-                    o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
-                    *reinterpret_cast<uint2 *>(dst + dt * 32 + kg * 8 + half * 4) = o;
-                }
+            for (int kg = 0; kg < 4; kg++) {
+                uint2 o;
+                o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
+                o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
+                *reinterpret_cast<uint2 *>(mine + col * PITCH + (dt * 32 + kg * 8 + half * 4) * 2) = o;
             }
-        } else {
+        }
+        // lane `col` knows where row `col` goes (0: the row does not exist)
+        const uint64_t my_dst = m_valid ? reinterpret_cast<uint64_t>(p.out + static_cast<uint64_t>(tok) * p.out_tok_stride +
+                                                                     static_cast<uint64_t>(head) * D)
+                                        : 0;
+#pragma unroll
+        for (int i = 0; i < 32 / RPI; i++) {
+            const uint32_t r = lane / LPR + RPI * i;
+            const uint64_t dst = __shfl(my_dst, static_cast<int>(r));
+            const unsigned char *src = mine + r * PITCH + (lane % LPR) * 16;
+            const uint2 lo = *reinterpret_cast<const uint2 *>(src), hi = *reinterpret_cast<const uint2 *>(src + 8);
+            if (dst != 0) {
+                *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(dst) + (lane % LPR) * 16) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            }
+        }
+    }
+    if (m_valid) {
+        const uint64_t rh = static_cast<uint64_t>(tok) * p.n_heads + head;
+        if (n_splits > 1) {
             // this run's partial: a row that sees none of the run's positions leaves (-inf, 0, zeros)
             const uint64_t slot = rh * p.max_splits + split;
             float *dst = p.part_acc + slot * D;
