@@ -1009,20 +1009,26 @@ decode_dma_kernel(const DecodeMfmaParams p)
                 }
             };
 
-            // every copy is unconditional (steps past the end copy the last step again, into the stage
-            // nobody reads any more), so the wait counts are exact
+            // Two steps in flight. No copy is issued twice (the hint above sends a repeated one to memory
+            // again: two of a segment's 66 steps), so the wait before the last step is for everything.
             const uint32_t last = n_steps - 1;
             issue(0);
-            issue(min(1u, last));
+            if (last >= 1) {
+                issue(1);
+            }
             for (uint32_t step = 0; step < n_steps; step++) {
-                dma_wait<PER_WAVE>();   // this wave's share of `step` has landed
+                if (step < last) {
+                    dma_wait<PER_WAVE>();   // this wave's share of `step` has landed: only the next step's is out
+                } else {
+                    dma_wait<0>();
+                }
                 __syncthreads();        // ... and everybody else's
                 compute(step);
                 __syncthreads();        // the stage is free again
-                issue(min(step + 2, last));
+                if (step + 2 <= last) {
+                    issue(step + 2);
+                }
             }
-            dma_wait<0>();
-            __syncthreads();
 
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
@@ -1365,20 +1371,26 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 }
             };
 
-            // every copy is unconditional (steps past the end copy the last step again, into the stage
-            // nobody reads any more), so the wait counts are exact
+            // Two steps in flight. No copy is issued twice (the hint above sends a repeated one to memory
+            // again: two of a segment's 66 steps), so the wait before the last step is for everything.
             const uint32_t last = n_steps - 1;
             issue(0);
-            issue(min(1u, last));
+            if (last >= 1) {
+                issue(1);
+            }
             for (uint32_t step = 0; step < n_steps; step++) {
-                dma_wait<PER_WAVE>();   // this wave's share of `step` has landed
+                if (step < last) {
+                    dma_wait<PER_WAVE>();   // this wave's share of `step` has landed: only the next step's is out
+                } else {
+                    dma_wait<0>();
+                }
                 __syncthreads();        // ... and everybody else's
                 compute(step);
                 __syncthreads();        // the stage is free again
-                issue(min(step + 2, last));
+                if (step + 2 <= last) {
+                    issue(step + 2);
+                }
             }
-            dma_wait<0>();
-            __syncthreads();
 
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
