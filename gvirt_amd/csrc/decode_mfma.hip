@@ -88,6 +88,7 @@ struct DecodeMfmaParams {
     uint32_t total_rows;   // query rows of the batch (one per sequence in a plain decode step)
     uint32_t only_single;  // 1: the units of the split are the sequences, and only those with one query row take part
     uint32_t unit0, n_units;   // this launch's slice of the units (rows or sequences): unit0 .. unit0 + n_units - 1
+    uint32_t step_mult;    // steps (of 16 positions) the kernel takes at a time: chunks are multiples of it
 };
 
 // A cache row is read once per decode step: the non-temporal hint keeps it from displacing other lines
@@ -309,7 +310,8 @@ struct DecodeSplit {
         }
         if (total != 0) {
             chunk = max(ceil_div(total, gridDim.x), kSplitMinChunk);
-            chunk = min(chunk, (kSplitTblCap - 2) * p.block_size / kStep);
+            chunk = ceil_div(chunk, p.step_mult) * p.step_mult;
+            chunk = min(chunk, (kSplitTblCap - 2) * p.block_size / kStep / p.step_mult * p.step_mult);
             n_chunks = ceil_div(total, chunk);
         }
     }
@@ -833,17 +835,23 @@ __device__ __forceinline__ void dma_wait()
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-template <typename T>
+// NKV: kv heads of a pass. 8, or all of a model's 4, 2 or 1: then 8 / NKV waves share a kv head, a step is
+// 16 positions for each of them (wave w: kv head w % NKV, positions 16 (w / NKV) .. + 15 of the step), and
+// their results meet in the head's first wave at the end of the segment.
+template <typename T, int NKV>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_dma_kernel(const DecodeMfmaParams p)
 {
     constexpr int D = 128;
     constexpr int KS = D / 32, MT = D / 16;
     constexpr int HEADB = D * 2;                 // bytes of one (position, kv head) row
-    constexpr int POSB = kWaves * HEADB;         // LDS bytes of one position: the 8 kv heads of the pass
-    constexpr int KBYTES = kStep * POSB;         // 32 KiB: the K half of a stage
+    constexpr int NSUB = kWaves / NKV;           // 16-position groups of a step
+    constexpr int POSB = NKV * HEADB;            // LDS bytes of one position: the kv heads of the pass
+    constexpr int WSTEP = kStep * NSUB;          // positions of a step
+    constexpr int KBYTES = WSTEP * POSB;         // 32 KiB: the K half of a stage
     constexpr int STAGE = 2 * KBYTES;
     constexpr int PER_WAVE = 8;                  // copies per wave and step
+    constexpr int XS = D + 16;                   // floats of one head's (O, m, l) on its way to the head's first wave
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + 2 * STAGE);
@@ -855,11 +863,12 @@ decode_dma_kernel(const DecodeMfmaParams p)
     const uint32_t col = lane & 15;
     const uint32_t jq = lane >> 4;
 
-    // read roles (this wave's kv head = `wave` inside the pass)
+    // read roles: this wave's kv head inside the pass and its group of 16 positions inside the step
+    const uint32_t kvl = wave % NKV, sub = wave / NKV;
     uint32_t kr_off[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-        kr_off[ks] = col * POSB + wave * HEADB + (((4 * ks + jq) ^ swizzle<D>(col)) << 4);
+        kr_off[ks] = (16 * sub + col) * POSB + kvl * HEADB + (((4 * ks + jq) ^ swizzle<D>(col)) << 4);
     }
     uint32_t vr_off[MT];
     {
@@ -867,15 +876,23 @@ decode_dma_kernel(const DecodeMfmaParams p)
         const uint32_t q4 = lane & 3;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            vr_off[mt] = KBYTES + pos * POSB + wave * HEADB + (((2 * mt + (q4 >> 1)) ^ swizzle<D>(pos)) << 4) + ((q4 & 1) << 3);
+            vr_off[mt] = KBYTES + (16 * sub + pos) * POSB + kvl * HEADB + (((2 * mt + (q4 >> 1)) ^ swizzle<D>(pos)) << 4) + ((q4 & 1) << 3);
         }
     }
-    // copy roles: wave w moves positions 2w and 2w+1, each as two copies of four kv heads, for K and V.
-    // Lane = (kv head inside the four) * 16 + chunk slot; the slot receives chunk slot ^ pattern(position).
-    uint32_t c_voff[2];
+    // copy roles: wave w fills bytes 4096 w .. + 4095 of the K and of the V half of a stage with four copies each:
+    // 8 kv heads: two positions, each as two copies of four kv heads; 4: four positions; 2: eight; 1: sixteen.
+    // They are positions of the wave's own group. Lane = (256-byte row inside the KiB) * 16 + chunk slot; the slot
+    // receives chunk slot ^ pattern(position). c_rel: the lane's position inside the group, c_voff: its offset
+    // inside the position's cache row.
+    uint32_t c_rel[4], c_voff[4];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        c_voff[i] = (lane >> 4) * HEADB + (((lane & 15u) ^ swizzle<D>(2 * wave + i)) << 4);
+    for (int i = 0; i < 4; i++) {
+        const uint32_t byte = (4 * wave + i) * 1024 + 16 * lane;
+        c_rel[i] = (byte / POSB) & 15u;
+        c_voff[i] = ((byte % POSB) & ~255u) + (((lane & 15u) ^ swizzle<D>(c_rel[i])) << 4);
+        if constexpr (NKV >= 4) {
+            c_rel[i] = uni(c_rel[i]);   // a copy is one position
+        }
     }
 
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
@@ -891,13 +908,13 @@ decode_dma_kernel(const DecodeMfmaParams p)
     auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool whole, uint32_t pslot, bool first_piece,
                            int4 meta) {
         const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
-        const uint32_t n_steps = ceil_div(t1 - t0, kStep);
+        const uint32_t n_steps = ceil_div(t1 - t0, static_cast<uint32_t>(WSTEP));
         const uint32_t blk0 = t0 / p.block_size;
         // the query rows of the first pass travel together with the block-table entries
         uint4 qreg[KS];
         auto load_q = [&](uint32_t kv0) {
             const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
-                                   static_cast<uint64_t>((kv0 + wave) * p.group + col) * D;
+                                   static_cast<uint64_t>((kv0 + kvl) * p.group + col) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8) : make_uint4(0, 0, 0, 0);
@@ -915,8 +932,8 @@ decode_dma_kernel(const DecodeMfmaParams p)
             __syncthreads();
         }
 
-        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += kWaves) {
-            const uint32_t kvh = kv0 + wave;
+        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += NKV) {
+            const uint32_t kvh = kv0 + kvl;
             const uint32_t head0 = kvh * p.group;
 
             if (kv0 > 0) {
@@ -934,30 +951,34 @@ decode_dma_kernel(const DecodeMfmaParams p)
             }
             float m_run = -INFINITY, l_run = 0.f;
 
-            // copies of one step into stage step % 2. The 16 positions of a step share one block
-            // (block_size % 16 == 0). Positions at or beyond the end re-read the last valid one.
+            // copies of one step into stage step % 2. The 16 positions of a group share one block
+            // (block_size % 16 == 0, segments start at multiples of 16). Positions at or beyond the end re-read
+            // the last valid one, a group beyond the end the last valid group.
             auto issue = [&](uint32_t step) {
-                const uint32_t ts = t0 + step * kStep;
-                const uint32_t blk = ts / p.block_size, off = ts % p.block_size;
+                const uint32_t ts = t0 + step * WSTEP;
+                const uint32_t gs = NSUB == 1 ? ts : min(ts + 16 * sub, (t1 - 1) & ~15u);
+                const uint32_t blk = gs / p.block_size, off = gs % p.block_size;
                 const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
                 const uint64_t row0 = static_cast<uint64_t>(phys) * p.block_size + off;
-                const uint32_t last_pos = min(t1 - 1 - ts, static_cast<uint32_t>(kStep - 1));
-                const uint32_t st = smem_addr + (step & 1) * STAGE;
+                const uint32_t last_rel = min(t1 - 1 - gs, 15u);
+                const uint32_t st = smem_addr + (step & 1) * STAGE + wave * 4096;
                 const char *kb = static_cast<const char *>(p.k_cache) + row0 * row_bytes + kv0 * HEADB;
                 const char *vb = static_cast<const char *>(p.v_cache) + row0 * row_bytes + kv0 * HEADB;
 #pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    const uint32_t pos = 2 * wave + i;
-                    const uint32_t src = min(pos, last_pos) * row_bytes;   // uniform
-#pragma unroll
-                    for (int j = 0; j < 2; j++) {
-                        dma_1k(st + pos * POSB + j * 1024, c_voff[i], kb + src + j * 1024);
-                        dma_1k(st + KBYTES + pos * POSB + j * 1024, c_voff[i], vb + src + j * 1024);
+                for (int i = 0; i < 4; i++) {
+                    if constexpr (NKV >= 4) {
+                        const uint32_t src = uni(min(c_rel[i], last_rel) * row_bytes);
+                        dma_1k(st + i * 1024, c_voff[i], kb + src);
+                        dma_1k(st + KBYTES + i * 1024, c_voff[i], vb + src);
+                    } else {
+                        const uint32_t voff = min(c_rel[i], last_rel) * POSB + c_voff[i];   // the cache row is the pass
+                        dma_1k(st + i * 1024, voff, kb);
+                        dma_1k(st + KBYTES + i * 1024, voff, vb);
                     }
                 }
             };
             auto compute = [&](uint32_t step) {
-                const uint32_t t = t0 + step * kStep;
+                const uint32_t t = t0 + step * WSTEP + 16 * sub;
                 const unsigned char *stage = smem + (step & 1) * STAGE;
                 f32x4_t S = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1032,7 +1053,45 @@ decode_dma_kernel(const DecodeMfmaParams p)
 
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
-            if (col < g_valid) {
+            if constexpr (NSUB > 1) {
+                // the groups of a kv head meet in its first wave: (O, m, l) of the others through the stage memory,
+                // which nobody reads any more (every wave has passed the loop's last barrier)
+                float *xch = reinterpret_cast<float *>(smem);
+                if (sub != 0) {
+                    float *dst = xch + (wave * 16 + col) * XS;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
+                    }
+                    if (jq == 0) {
+                        dst[D] = m_run;
+                        dst[D + 1] = l_tot;
+                    }
+                }
+                __syncthreads();
+                if (sub == 0) {
+#pragma unroll
+                    for (int s2 = 1; s2 < NSUB; s2++) {
+                        const float *src = xch + ((s2 * NKV + kvl) * 16 + col) * XS;
+                        const float m2 = src[D], l2 = src[D + 1];
+                        const float m_new = fmaxf(m_run, m2);
+                        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                        const float a1 = fast_exp2(m_run - m_safe), a2 = fast_exp2(m2 - m_safe);
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++) {
+                            const float4 o2 = *reinterpret_cast<const float4 *>(src + mt * 16 + jq * 4);
+                            O[mt][0] = O[mt][0] * a1 + o2.x * a2;
+                            O[mt][1] = O[mt][1] * a1 + o2.y * a2;
+                            O[mt][2] = O[mt][2] * a1 + o2.z * a2;
+                            O[mt][3] = O[mt][3] * a1 + o2.w * a2;
+                        }
+                        l_tot = l_tot * a1 + l2 * a2;
+                        m_run = m_new;
+                    }
+                }
+                __syncthreads();   // the next segment refills the stages
+            }
+            if (col < g_valid && sub == 0) {
                 if (whole) {
                     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
                     uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
@@ -1061,12 +1120,12 @@ decode_dma_kernel(const DecodeMfmaParams p)
     split.for_each_segment(run_segment);
 }
 
-template <typename T>
-int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
+template <typename T, int NKV>
+int launch_dma_nkv(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
                        (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
-    auto kernel = decode_dma_kernel<T>;
+    auto kernel = decode_dma_kernel<T, NKV>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
     }
@@ -1074,6 +1133,16 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
+}
+template <typename T>
+int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
+{
+    switch (p.n_kv_heads) {
+    case 1: return launch_dma_nkv<T, 1>(stream, p, n_workgroups);
+    case 2: return launch_dma_nkv<T, 2>(stream, p, n_workgroups);
+    case 4: return launch_dma_nkv<T, 4>(stream, p, n_workgroups);
+    default: return launch_dma_nkv<T, 8>(stream, p, n_workgroups);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -1489,12 +1558,13 @@ bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_
     return (head_dim == 64 || head_dim == 128) && block_size % kStep == 0 && group <= 16;
 }
 
-// decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8
 uint32_t decode_mfma_slice_units() { return kSplitSeqCap; }
 
+// decode_dma_kernel: head_dim 128, 16-bit cache, kv heads a multiple of 8, or 4, 2 or 1 of them
 bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
 {
-    return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0;
+    return head_dim == 128 && kv_dtype == XLITE_HIP_KV_SAME &&
+           (n_kv_heads % kWaves == 0 || n_kv_heads == 4 || n_kv_heads == 2 || n_kv_heads == 1);
 }
 
 // decode_dma8_kernel: head_dim 128, 8-bit cache, kv heads a multiple of 8
@@ -1578,7 +1648,9 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
         p.unit0 = u0;
         p.n_units = min(kSplitSeqCap, units - u0);
         int rc;
+        p.step_mult = 1;
         if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+            p.step_mult = a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1;
             rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
         } else if (decode_dma8_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             if (a.kv_dtype == XLITE_HIP_KV_FP8) {

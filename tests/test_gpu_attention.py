@@ -117,6 +117,24 @@ def test_decode_wide_groups_and_small_blocks(rt, model, work):
     check(run_attention(rt, w), oracle_attention(w))
 
 
+@pytest.mark.parametrize("model", [(28, 4, 128, torch.bfloat16), (16, 4, 16, torch.float16), (64, 4, 48, torch.bfloat16),
+                                   (14, 2, 128, torch.bfloat16), (32, 2, 16, torch.float16), (6, 2, 32, torch.bfloat16),
+                                   (16, 1, 128, torch.bfloat16), (7, 1, 16, torch.float16), (1, 1, 48, torch.bfloat16)])
+def test_decode_few_kv_heads_position_groups_share_a_workgroup(rt, model):
+    """Decode batches with 4, 2 or 1 kv heads of 128 elements (a model's share under tensor parallelism): 2, 4 or 8
+    waves share a kv head, each with its own 16 positions of a step of 32, 64 or 128, and their results meet inside
+    the workgroup. Visible ranges around every multiple of 16 up to two steps and around block ends (whole groups
+    beyond the end re-read the last valid group), blocks of 16, 32, 48 and 128 positions, groups of 1 to 16 heads."""
+    nH, nKV, bs, dtype = model
+    ctx = [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 79, 80, 81, 96, 97, 111, 112, 113, 127, 128, 129, 143, 144, 145,
+           160, 191, 192, 193, 255, 256, 257, 1000, 4097, 9000]
+    w = generic_case(63, [1] * len(ctx), [c - 1 for c in ctx], nH, nKV, 128, bs, dtype)
+    check(run_attention(rt, w), oracle_attention(w))
+    # a handful of long sequences: every workgroup gets a slice of one, partials merged by the second kernel
+    w = generic_case(64, [1] * 3, [20000, 7001, 12345], nH, nKV, 128, bs, dtype)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 @pytest.mark.parametrize("model,batch,lo,hi,long_ones", [((32, 8, 128, 128, torch.bfloat16), 100, 1, 3000, [9000, 5000]),
                                                         ((32, 8, 128, 128, torch.bfloat16), 700, 1, 200, [2500]),
                                                         ((16, 8, 128, 16, torch.float16), 70, 1, 900, []),
