@@ -1185,17 +1185,23 @@ __device__ __forceinline__ void widen4(uint32_t w, uint32_t *lo, uint32_t *hi)
     }
 }
 
-template <typename T, int KVF>
+// NKV: kv heads of a pass. 8, or all of a model's 4 or 2: then 8 / NKV waves share a kv head, a step is 32 positions
+// for each of them (wave w: kv head w % NKV, positions 32 (w / NKV) .. + 31 of the step), and their results meet in
+// the head's first wave at the end of the segment.
+template <typename T, int KVF, int NKV>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_dma8_kernel(const DecodeMfmaParams p)
 {
     constexpr int D = 128;
     constexpr int MT = D / 16;
-    constexpr int STEP = 32;                     // positions per step
+    constexpr int STEP = 32;                     // positions per step and wave
+    constexpr int NSUB = kWaves / NKV;           // 32-position groups of a step
+    constexpr int WSTEP = STEP * NSUB;           // positions per step
     constexpr int HEADB = D;                     // bytes of one (position, kv head) row
-    constexpr int POSB = kWaves * HEADB;         // LDS bytes of one position: the 8 kv heads of the pass
-    constexpr int KBYTES = STEP * POSB;          // 32 KiB: the K half of a stage
-    constexpr int SCALEB = kWaves * STEP * 4;    // 1 KiB: the K scales of a stage
+    constexpr int POSB = NKV * HEADB;            // LDS bytes of one position: the kv heads of the pass
+    constexpr int KBYTES = WSTEP * POSB;         // 32 KiB: the K half of a stage
+    constexpr int SCALEB = kWaves * STEP * 4;    // 1 KiB: the K scales of a stage, [wave][32 positions]
+    constexpr int XS = D + 16;                   // floats of one head's (O, m, l) on its way to the head's first wave
     constexpr int STAGE = 2 * KBYTES + 2 * SCALEB;
     constexpr int PER_WAVE = 9;                  // copies per wave and step: 4 K rows, 4 V rows, 64 scales
 
@@ -1209,19 +1215,20 @@ decode_dma8_kernel(const DecodeMfmaParams p)
     const uint32_t col = lane & 15;
     const uint32_t jq = lane >> 4;
 
-    // XOR pattern of position `pos` of a step: chunk bits, kv-head bit
+    // XOR pattern of position `pos` of a wave's 32: chunk bits, kv-head bit
     auto pat_chunk = [](uint32_t pos) { return pos & 7u; };
     auto pat_head = [](uint32_t pos) { return ((pos >> 3) ^ (pos >> 4)) & 1u; };
-    auto slot_off = [&](uint32_t pos, uint32_t head, uint32_t chunk) {
-        return pos * POSB + (((head ^ pat_head(pos)) << 3 | (chunk ^ pat_chunk(pos))) << 4);
+    auto slot_off = [&](uint32_t pos, uint32_t head, uint32_t chunk) {   // pos: inside the whole step
+        return pos * POSB + head / 2 * 256 + ((((head & 1u) ^ pat_head(pos & 31u)) << 3 | (chunk ^ pat_chunk(pos & 31u))) << 4);
     };
-    // read roles (this wave's kv head = `wave` inside the pass)
+    // read roles: this wave's kv head inside the pass and its group of 32 positions inside the step
+    const uint32_t kvl = wave % NKV, sub = wave / NKV;
     uint32_t kr_off[2][2];
 #pragma unroll
     for (int tl = 0; tl < 2; tl++) {
 #pragma unroll
         for (int r = 0; r < 2; r++) {
-            kr_off[tl][r] = slot_off(16 * tl + col, wave, jq + 4 * r);
+            kr_off[tl][r] = slot_off(STEP * sub + 16 * tl + col, kvl, jq + 4 * r);
         }
     }
     uint32_t vr_off[MT];
@@ -1230,23 +1237,34 @@ decode_dma8_kernel(const DecodeMfmaParams p)
         const uint32_t pos = row < 4 ? 4 * jq + row : 16 + 4 * jq + (row - 4);
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            vr_off[mt] = KBYTES + slot_off(pos, wave, mt) + ((lane & 1) << 3);
+            vr_off[mt] = KBYTES + slot_off(STEP * sub + pos, kvl, mt) + ((lane & 1) << 3);
         }
     }
     const uint32_t sc_off = 2 * KBYTES + (wave * STEP + 4 * jq) * 4;   // K scales of the first tile's rows
-    // copy roles: wave w moves positions 4w .. 4w+3 (K and V). Lane = slot (kv head, chunk) of the position's
-    // 1 KiB; the slot receives the chunk the pattern assigns to it.
-    uint32_t c_voff[4];
+    // copy roles: wave w fills bytes 4096 w .. + 4095 of the K and of the V half of a stage with four copies each:
+    // 8 kv heads: four positions; 4: eight; 2: sixteen. They are positions of one 16-position half of the wave's own
+    // group. Lane = slot (position inside the KiB, kv head, chunk); the slot receives the (kv head, chunk) the
+    // position's pattern assigns to it. c_rel: the lane's position inside the half, c_voff: its offset inside the
+    // position's cache row.
+    uint32_t c_rel[4], c_voff[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t pos = 4 * wave + i;
-        c_voff[i] = ((lane >> 3) ^ pat_head(pos)) * HEADB + (((lane & 7u) ^ pat_chunk(pos)) << 4);
+        const uint32_t byte = (4 * wave + i) * 1024 + 16 * lane;
+        const uint32_t pos = (byte / POSB) & 31u, in_pos = byte % POSB;
+        c_rel[i] = pos & 15u;
+        c_voff[i] = (in_pos / 256 * 2 + (((in_pos >> 7) & 1u) ^ pat_head(pos))) * HEADB + (((lane & 7u) ^ pat_chunk(pos)) << 4);
+        if constexpr (NKV == 8) {
+            c_rel[i] = uni(c_rel[i]);   // a copy is one position
+        }
     }
-    // scale copies: waves 0-3 the K scales, 4-7 the V scales; a wave moves two kv heads x 32 positions
-    const uint32_t sc_head = 2 * (wave & 3) + (lane >> 5);
+    const uint32_t c_half = ((4 * wave * 1024 / POSB) >> 4) & 1u;   // the half of the group this wave's copies lie in
+    // scale copies: a wave moves the scales of two kv heads of its own group x 32 positions: the K scales if its kv
+    // head is even, the V scales of the same two heads if it is odd
+    const uint32_t sc_wave = (wave & ~1u) + (lane >> 5);   // the wave that reads these scales
+    const uint32_t sc_head = sc_wave % NKV;
     const uint32_t sc_pos = lane & 31;
-    const float *sc_src = wave < 4 ? p.k_scale : p.v_scale;
-    const uint32_t sc_dst = 2 * KBYTES + (wave >> 2) * SCALEB + (wave & 3) * 256;
+    const float *sc_src = (wave & 1u) ? p.v_scale : p.k_scale;
+    const uint32_t sc_dst = 2 * KBYTES + (wave & 1u) * SCALEB + (wave & ~1u) * STEP * 4;
 
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t row_bytes = p.n_kv_heads * HEADB;
@@ -1260,14 +1278,14 @@ decode_dma8_kernel(const DecodeMfmaParams p)
     auto run_segment = [&](uint32_t seq, uint32_t tok, uint32_t t0, uint32_t t1, bool whole, uint32_t pslot, bool first_piece,
                            int4 meta) {
         const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
-        const uint32_t n_steps = ceil_div(t1 - t0, static_cast<uint32_t>(STEP));
+        const uint32_t n_steps = ceil_div(t1 - t0, static_cast<uint32_t>(WSTEP));
         const uint32_t blk0 = t0 / p.block_size;
         // Q^T as the B operand, as fp16: k step 2r + h of the first product covers the elements
         // [16 (j + 4r) + 8h, + 8) of the head
         uint4 qreg[4];
         auto load_q = [&](uint32_t kv0) {
             const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
-                                   static_cast<uint64_t>((kv0 + wave) * p.group + col) * D;
+                                   static_cast<uint64_t>((kv0 + kvl) * p.group + col) * D;
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + 16 * (jq + 4 * (ks >> 1)) + 8 * (ks & 1))
@@ -1298,8 +1316,8 @@ decode_dma8_kernel(const DecodeMfmaParams p)
             __syncthreads();
         }
 
-        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += kWaves) {
-            const uint32_t kvh = kv0 + wave;
+        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += NKV) {
+            const uint32_t kvh = kv0 + kvl;
             const uint32_t head0 = kvh * p.group;
 
             if (kv0 > 0) {
@@ -1321,7 +1339,7 @@ decode_dma8_kernel(const DecodeMfmaParams p)
             // copies of one step into stage step % 2. Each half of a step (16 positions from a multiple of 16)
             // lies in one block (block_size % 16 == 0). Positions at or beyond the end re-read the last valid one.
             auto issue = [&](uint32_t step) {
-                const uint32_t ts = t0 + step * STEP;   // <= t1 - 1
+                const uint32_t ts = t0 + step * WSTEP + STEP * sub;   // this wave's group; beyond the end: see below
                 const uint32_t tl = t1 - 1;
                 const uint32_t st = smem_addr + (step & 1) * STAGE;
                 uint64_t row0[2];
@@ -1334,17 +1352,21 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                     row0[h] = static_cast<uint64_t>(phys) * p.block_size + off;
                     max_i[h] = ts + 16 * h > tl ? 0u : min(tl - (ts + 16 * h), 15u);
                 }
-                const uint32_t half = wave >> 2;
-                const uint64_t my_row0 = half ? row0[1] : row0[0];
-                const uint32_t my_max = half ? max_i[1] : max_i[0];
+                const uint64_t my_row0 = c_half ? row0[1] : row0[0];
+                const uint32_t my_max = c_half ? max_i[1] : max_i[0];
                 const char *kb = static_cast<const char *>(p.k_cache) + my_row0 * row_bytes + kv0 * HEADB;
                 const char *vb = static_cast<const char *>(p.v_cache) + my_row0 * row_bytes + kv0 * HEADB;
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const uint32_t pos = 4 * wave + i;
-                    const uint32_t src = min(pos & 15u, my_max) * row_bytes;   // uniform
-                    dma_1k(st + pos * POSB, c_voff[i], kb + src);
-                    dma_1k(st + KBYTES + pos * POSB, c_voff[i], vb + src);
+                    if constexpr (NKV == 8) {
+                        const uint32_t src = uni(min(c_rel[i], my_max) * row_bytes);
+                        dma_1k(st + (4 * wave + i) * 1024, c_voff[i], kb + src);
+                        dma_1k(st + KBYTES + (4 * wave + i) * 1024, c_voff[i], vb + src);
+                    } else {
+                        const uint32_t voff = min(c_rel[i], my_max) * POSB + c_voff[i];   // the cache row is the pass
+                        dma_1k(st + (4 * wave + i) * 1024, voff, kb);
+                        dma_1k(st + KBYTES + (4 * wave + i) * 1024, voff, vb);
+                    }
                 }
                 {
                     const bool hi = sc_pos >= 16;
@@ -1355,7 +1377,7 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 }
             };
             auto compute = [&](uint32_t step) {
-                const uint32_t t = t0 + step * STEP;
+                const uint32_t t = t0 + step * WSTEP + STEP * sub;
                 const unsigned char *stage = smem + (step & 1) * STAGE;
                 // ---- S^T = K . Q^T: two tiles of 16 positions x 16 heads ------------------------------------
                 f32x4_t S[2];
@@ -1463,7 +1485,45 @@ decode_dma8_kernel(const DecodeMfmaParams p)
 
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
-            if (col < g_valid) {
+            if constexpr (NSUB > 1) {
+                // the groups of a kv head meet in its first wave: (O, m, l) of the others through the stage memory,
+                // which nobody reads any more (every wave has passed the loop's last barrier)
+                float *xch = reinterpret_cast<float *>(smem);
+                if (sub != 0) {
+                    float *dst = xch + (wave * 16 + col) * XS;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
+                    }
+                    if (jq == 0) {
+                        dst[D] = m_run;
+                        dst[D + 1] = l_tot;
+                    }
+                }
+                __syncthreads();
+                if (sub == 0) {
+#pragma unroll
+                    for (int s2 = 1; s2 < NSUB; s2++) {
+                        const float *src = xch + ((s2 * NKV + kvl) * 16 + col) * XS;
+                        const float m2 = src[D], l2 = src[D + 1];
+                        const float m_new = fmaxf(m_run, m2);
+                        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                        const float a1 = fast_exp2(m_run - m_safe), a2 = fast_exp2(m2 - m_safe);
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++) {
+                            const float4 o2 = *reinterpret_cast<const float4 *>(src + mt * 16 + jq * 4);
+                            O[mt][0] = O[mt][0] * a1 + o2.x * a2;
+                            O[mt][1] = O[mt][1] * a1 + o2.y * a2;
+                            O[mt][2] = O[mt][2] * a1 + o2.z * a2;
+                            O[mt][3] = O[mt][3] * a1 + o2.w * a2;
+                        }
+                        l_tot = l_tot * a1 + l2 * a2;
+                        m_run = m_new;
+                    }
+                }
+                __syncthreads();   // the next segment refills the stages
+            }
+            if (col < g_valid && sub == 0) {
                 if (whole) {
                     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
                     uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
@@ -1492,12 +1552,12 @@ decode_dma8_kernel(const DecodeMfmaParams p)
     split.for_each_segment(run_segment);
 }
 
-template <typename T, int KVF>
-int launch_dma8(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
+template <typename T, int KVF, int NKV>
+int launch_dma8_nkv(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * 32 * kWaves * 128 + 2 * kWaves * 32 * 4) +
                        (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
-    auto kernel = decode_dma8_kernel<T, KVF>;
+    auto kernel = decode_dma8_kernel<T, KVF, NKV>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
     }
@@ -1505,6 +1565,15 @@ int launch_dma8(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgr
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
+}
+template <typename T, int KVF>
+int launch_dma8(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
+{
+    switch (p.n_kv_heads) {
+    case 2: return launch_dma8_nkv<T, KVF, 2>(stream, p, n_workgroups);
+    case 4: return launch_dma8_nkv<T, KVF, 4>(stream, p, n_workgroups);
+    default: return launch_dma8_nkv<T, KVF, 8>(stream, p, n_workgroups);
+    }
 }
 
 template <typename T, int D, int KVF, bool MULTI_SUB>
@@ -1567,10 +1636,11 @@ bool decode_dma_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
            (n_kv_heads % kWaves == 0 || n_kv_heads == 4 || n_kv_heads == 2 || n_kv_heads == 1);
 }
 
-// decode_dma8_kernel: head_dim 128, 8-bit cache, kv heads a multiple of 8
+// decode_dma8_kernel: head_dim 128, 8-bit cache, kv heads a multiple of 8, or 4 or 2 of them
 bool decode_dma8_supported(uint32_t n_kv_heads, uint32_t head_dim, int kv_dtype)
 {
-    return head_dim == 128 && kv_dtype != XLITE_HIP_KV_SAME && n_kv_heads % kWaves == 0;
+    return head_dim == 128 && kv_dtype != XLITE_HIP_KV_SAME &&
+           (n_kv_heads % kWaves == 0 || n_kv_heads == 4 || n_kv_heads == 2);
 }
 
 // The chunk the kernel really uses is the batch's total step count over the number of workgroups, which the
@@ -1653,6 +1723,7 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
             p.step_mult = a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1;
             rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
         } else if (decode_dma8_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+            p.step_mult = 2 * (a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1);   // a wave takes 32 positions at a time
             if (a.kv_dtype == XLITE_HIP_KV_FP8) {
                 rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_FP8>(stream, p, grid_x) : launch_dma8<FP16, XLITE_HIP_KV_FP8>(stream, p, grid_x);
             } else {

@@ -246,6 +246,23 @@ def test_decode_quantised_kv_byte_streaming_kernel_shapes(rt, kv_dtype, model):
 
 
 @pytest.mark.parametrize("kv_dtype", KV_DTYPES)
+@pytest.mark.parametrize("model", [(28, 4, 128, torch.bfloat16), (16, 4, 16, torch.float16), (64, 4, 48, torch.bfloat16),
+                                   (14, 2, 128, torch.float16), (32, 2, 16, torch.bfloat16), (2, 2, 32, torch.bfloat16)])
+def test_decode_quantised_kv_few_kv_heads_position_groups_share_a_workgroup(rt, kv_dtype, model):
+    """8-bit caches with 4 or 2 kv heads of 128 elements on the kernel that copies the cache bytes straight into LDS:
+    2 or 4 waves share a kv head, each with its own 32 positions of a step of 64 or 128 (a copy instruction is then 2
+    or 4 positions, the scales of a wave's group travel with it), and their results meet inside the workgroup. Visible
+    ranges around every multiple of 16 up to two steps, block sizes of 16, 32, 48 and 128, groups of 1 to 16 heads."""
+    nH, nKV, bs, dtype = model
+    ctx = [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 79, 80, 81, 96, 97, 111, 112, 113, 127, 128, 129, 143, 144, 145,
+           160, 191, 192, 193, 255, 256, 257, 1000, 4097, 9000]
+    w = quantised(generic_case(65, [1] * len(ctx), [c - 1 for c in ctx], nH, nKV, 128, bs, dtype), kv_dtype)
+    check(run_attention(rt, w), oracle_attention(w), max_abs=MAX_ABS_INT8)
+    w = quantised(generic_case(66, [1] * 3, [20000, 7001, 12345], nH, nKV, 128, bs, dtype), kv_dtype)
+    check(run_attention(rt, w), oracle_attention(w), max_abs=MAX_ABS_INT8)
+
+
+@pytest.mark.parametrize("kv_dtype", KV_DTYPES)
 @pytest.mark.parametrize("model", [(32, 8, 128, 128, torch.bfloat16), (14, 2, 64, 128, torch.float16), (28, 4, 128, 16, torch.bfloat16),
                                    (64, 2, 128, 128, torch.bfloat16), (8, 2, 128, 20, torch.float16)])
 @pytest.mark.parametrize("work", [([0], [77]), ([128], [300]), ([0] * 4, [189, 65, 13, 545]), ([2047, 1500, 0, 900], [1, 1, 300, 1]),
