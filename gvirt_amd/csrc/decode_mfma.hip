@@ -559,9 +559,14 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 return (static_cast<uint64_t>(tbl_lds[blk - blk0]) * p.block_size + off) * p.n_kv_heads;
             };
             auto sub_end = [&](uint32_t sub) { return min(t1, t0 + (sub + 1) * sub_len); };
-            auto issue = [&](uint32_t step, auto slot_tag) {
+            // `raw_step` may lie beyond the last step (the pipeline's loads are unconditional): then every lane reads
+            // the first 16 bytes of the last step, one cache line per instruction (the same rows again would be fetched
+            // from memory again under the non-temporal hint)
+            auto issue = [&](uint32_t raw_step, auto slot_tag) {
                 constexpr int SL = decltype(slot_tag)::value;
+                const uint32_t step = min(raw_step, n_steps - 1);
                 const bool last_step = step + 1 == n_steps;
+                const uint32_t keep = raw_step >= n_steps ? 0u : ~0u;
                 if constexpr (!MULTI_SUB) {
                     const uint32_t ts = step_start(0, step);
                     const uint64_t row0 = row_of(ts);   // uniform: scalar address arithmetic
@@ -583,13 +588,13 @@ decode_mfma_kernel(const DecodeMfmaParams p)
 #pragma unroll
                         for (int i = 0; i < NV; i++) {
                             const uint32_t back = vec_pos(i) > last_pos ? (vec_pos(i) - last_pos) * row_bytes : 0u;
-                            kreg[SL][i] = ld_stream<gvec_t>(kb + (g_off[i] - back));
-                            vreg[SL][i] = ld_stream<gvec_t>(vb + (g_off[i] - back));
+                            kreg[SL][i] = ld_stream<gvec_t>(kb + ((g_off[i] - back) & keep));
+                            vreg[SL][i] = ld_stream<gvec_t>(vb + ((g_off[i] - back) & keep));
                         }
                         if constexpr (KV8) {
                             if (s_active) {
                                 const uint32_t back = s_pos > last_pos ? (s_pos - last_pos) * p.n_kv_heads : 0u;
-                                sreg[SL] = s_src[row0 + s_off - back];
+                                sreg[SL] = s_src[row0 + ((s_off - back) & keep)];
                             }
                         }
                     }
@@ -601,8 +606,8 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                         const uint32_t last_pos = min(end - 1 - ts, static_cast<uint32_t>(kStep - 1));
                         const uint32_t back = vec_pos(i) > last_pos ? (vec_pos(i) - last_pos) * row_bytes : 0u;
                         const uint64_t row0 = row_of(ts);
-                        kreg[SL][i] = ld_stream<gvec_t>(reinterpret_cast<const char *>(kc) + row0 * CH * VB + (g_off[i] - back));
-                        vreg[SL][i] = ld_stream<gvec_t>(reinterpret_cast<const char *>(vc) + row0 * CH * VB + (g_off[i] - back));
+                        kreg[SL][i] = ld_stream<gvec_t>(reinterpret_cast<const char *>(kc) + row0 * CH * VB + ((g_off[i] - back) & keep));
+                        vreg[SL][i] = ld_stream<gvec_t>(reinterpret_cast<const char *>(vc) + row0 * CH * VB + ((g_off[i] - back) & keep));
                     }
                     if constexpr (KV8) {
                         if (s_active) {
@@ -719,18 +724,18 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             // for everything in flight.
             const uint32_t last = n_steps - 1;   // n_steps >= 1: the tile is not empty
             issue(0, S0{});
-            issue(min(1u, last), S1{});
+            issue(1u, S1{});
             stage_write(S0{});
-            issue(min(2u, last), S0{});
+            issue(2u, S0{});
             __syncthreads();
             for (uint32_t step = 0; step < n_steps; step += 2) {
                 compute(step, S0{});
                 stage_write(S1{});
-                issue(min(step + 3, last), S1{});
+                issue(step + 3, S1{});
                 __syncthreads();
                 compute(step + 1, S1{});
                 stage_write(S0{});
-                issue(min(step + 4, last), S0{});
+                issue(step + 4, S0{});
                 __syncthreads();
             }
 
