@@ -1173,20 +1173,23 @@ __device__ __forceinline__ void dma_4b(uint32_t lds_addr, const void *src)
                  :: "s"(lds_addr), "v"(src) : "memory", "m0");
 }
 
-// four cache bytes -> four fp16 values (two registers), exactly
+// four cache bytes -> four fp16 values (two registers), exactly. fp8: the values themselves. int8: the values plus
+// kInt8Bias: byte b ^ 0x80 = b + 128 as an unsigned byte u, and 0x6400 | u reads as 1024 + u in fp16. The constant does
+// not have to be subtracted element by element (two packed subtractions per four values, a sixth of the kernel's
+// vector instructions): a product over biased operands is the product wanted plus the constant times the sum of the
+// other operand, which the caller takes off once - sum_d (k_d + c) q_d = sum_d k_d q_d + c sum_d q_d. Everything
+// stays exact: 1024 + u and its products with an fp16 value fit fp32.
+constexpr float kInt8Bias = 1152.0f;
 template <int KVF>
 __device__ __forceinline__ void widen4(uint32_t w, uint32_t *lo, uint32_t *hi)
 {
-    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
     if constexpr (KVF == XLITE_HIP_KV_FP8) {
         *lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(static_cast<int>(w), 1.0f, false));
         *hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(static_cast<int>(w), 1.0f, true));
     } else {
-        // byte b ^ 0x80 = b + 128 as an unsigned byte u; 0x6400 | u reads as 1024 + u in fp16; minus 1152 leaves b
-        const h2_t bias = {static_cast<_Float16>(-1152.0f), static_cast<_Float16>(-1152.0f)};
         const uint32_t x = w ^ 0x80808080u;
-        *lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u)) + bias);
-        *hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u)) + bias);
+        *lo = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
+        *hi = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
     }
 }
 
@@ -1340,6 +1343,23 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 O[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             }
             float m_run = -INFINITY, l_run = 0.f;
+            // int8: what the bias of the K operand adds to every score of head `col` (the score accumulators start from
+            // its negative), and the running sum of the probabilities as the second product sees them, for the bias
+            // of the V operand
+            float s_init = 0.f, pv_run = 0.f;
+            if constexpr (KVF == XLITE_HIP_KV_INT8) {
+                float qs = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) {
+                    qs = FP16::dot2(qreg[ks].x, 0x3c003c00u, qs);
+                    qs = FP16::dot2(qreg[ks].y, 0x3c003c00u, qs);
+                    qs = FP16::dot2(qreg[ks].z, 0x3c003c00u, qs);
+                    qs = FP16::dot2(qreg[ks].w, 0x3c003c00u, qs);
+                }
+                qs += __shfl_xor(qs, 16);
+                qs += __shfl_xor(qs, 32);
+                s_init = -kInt8Bias * qs;
+            }
 
             // copies of one step into stage step % 2. Each half of a step (16 positions from a multiple of 16)
             // lies in one block (block_size % 16 == 0). Positions at or beyond the end re-read the last valid one.
@@ -1388,7 +1408,7 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 f32x4_t S[2];
 #pragma unroll
                 for (int tl = 0; tl < 2; tl++) {
-                    S[tl] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    S[tl] = f32x4_t{s_init, s_init, s_init, s_init};
 #pragma unroll
                     for (int r = 0; r < 2; r++) {
                         const uint4 raw = *reinterpret_cast<const uint4 *>(stage + kr_off[tl][r]);
@@ -1448,6 +1468,13 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 l_run = l_run * alpha + psum;
                 const uint4 pb = make_uint4(FP16::pack(pe[0], pe[1]), FP16::pack(pe[2], pe[3]),
                                             FP16::pack(pe[4], pe[5]), FP16::pack(pe[6], pe[7]));
+                if constexpr (KVF == XLITE_HIP_KV_INT8) {
+                    float ps = FP16::dot2(pb.x, 0x3c003c00u, 0.f);
+                    ps = FP16::dot2(pb.y, 0x3c003c00u, ps);
+                    ps = FP16::dot2(pb.z, 0x3c003c00u, ps);
+                    ps = FP16::dot2(pb.w, 0x3c003c00u, ps);
+                    pv_run = pv_run * alpha + ps;
+                }
                 if (__any(alpha != 1.0f)) {
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
@@ -1490,6 +1517,19 @@ decode_dma8_kernel(const DecodeMfmaParams p)
 
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
+            if constexpr (KVF == XLITE_HIP_KV_INT8) {
+                // O^T of head `col` carries the bias of V times the probabilities summed over every position
+                float pv_tot = pv_run + __shfl_xor(pv_run, 16);
+                pv_tot += __shfl_xor(pv_tot, 32);
+                const float corr = kInt8Bias * pv_tot;
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    O[mt][0] -= corr;
+                    O[mt][1] -= corr;
+                    O[mt][2] -= corr;
+                    O[mt][3] -= corr;
+                }
+            }
             if constexpr (NSUB > 1) {
                 // the groups of a kv head meet in its first wave: (O, m, l) of the others through the stage memory,
                 // which nobody reads any more (every wave has passed the loop's last barrier)
