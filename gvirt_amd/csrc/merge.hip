@@ -118,6 +118,80 @@ merge_mla_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ part_a
         const uint32_t ps = s == 0 ? 2 * c0 + (1 - first_flag) : 2 * (c0 + s);
         return static_cast<uint64_t>(ps) * n_heads + head;
     };
+    if (n <= 64 && dv <= 512) {
+        // The common case in one round trip after the meta entry: lane s fetches (maximum, sum) of segment s and, without
+        // waiting for it, the first four segments' rows; the weights are worked out while those are on their way.
+        // (The general loop below waits for the maxima, then for the sums, then for every round of rows in turn.)
+        const uint32_t c = lane;
+        const bool c_ok = c < dv / 8;
+        auto load_round = [&](uint32_t j, uint4 (&x)[4]) {
+#pragma unroll
+            for (uint32_t u = 0; u < 4; u++) {
+                const uint32_t idx = min(j + u * WPR + stream, n - 1);
+                x[u] = c_ok ? *reinterpret_cast<const uint4 *>(part_acc + slot_of(idx) * dv + c * 8) : make_uint4(0, 0, 0, 0);
+            }
+        };
+        const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(min(lane, n - 1)) * 2);
+        uint4 x[4];
+        load_round(0, x);
+        float mm = lane < n ? ml.x : -INFINITY;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            mm = fmaxf(mm, __shfl_xor(mm, d));
+        }
+        const float ms = mm == -INFINITY ? 0.f : mm;
+        const float w_lane = lane < n ? fast_exp2(ml.x - ms) * ml.y : 0.f;
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float wsum = 0.f;
+        for (uint32_t j = 0; j < n; j += 4 * WPR) {
+            if (j > 0) {
+                load_round(j, x);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 4; u++) {
+                const uint32_t want = j + u * WPR + stream;
+                float w = __shfl(w_lane, static_cast<int>(min(want, n - 1)));
+                w = want < n ? w : 0.f;
+                const uint32_t xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+                wsum += w;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    acc[2 * k] += T::lo(xs[k]) * w;
+                    acc[2 * k + 1] += T::hi(xs[k]) * w;
+                }
+            }
+        }
+        if constexpr (WPR > 1) {
+            if (wave != 0) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    xch[((wave - 1) * 9 + k) * 64 + lane] = acc[k];
+                }
+                xch[((wave - 1) * 9 + 8) * 64 + lane] = wsum;
+            }
+            __syncthreads();
+            if (wave != 0) {
+                return;
+            }
+            for (uint32_t w = 0; w + 1 < WPR; w++) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    acc[k] += xch[(w * 9 + k) * 64 + lane];
+                }
+                wsum += xch[(w * 9 + 8) * 64 + lane];
+            }
+        }
+        const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+        if (c_ok) {
+            uint4 o;
+            o.x = T::pack(acc[0] * inv, acc[1] * inv);
+            o.y = T::pack(acc[2] * inv, acc[3] * inv);
+            o.z = T::pack(acc[4] * inv, acc[5] * inv);
+            o.w = T::pack(acc[6] * inv, acc[7] * inv);
+            *reinterpret_cast<uint4 *>(out + rh * dv + c * 8) = o;
+        }
+        return;
+    }
     float mm = -INFINITY;
     for (uint32_t s = lane; s < n; s += 64) {
         mm = fmaxf(mm, part_ml[slot_of(s) * 2]);
@@ -222,51 +296,95 @@ merge_meta_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc
         const uint32_t ps = s == 0 ? 2 * c0 + (1 - first_flag) : 2 * (c0 + s);
         return static_cast<uint64_t>(ps) * n_heads + head;
     };
-    float mm = -INFINITY;
-    for (uint32_t s = lane; s < n; s += 64) {
-        mm = fmaxf(mm, part_ml[slot_of(s) * 2]);
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        mm = fmaxf(mm, __shfl_xor(mm, d));
-    }
-    const float ms = mm == -INFINITY ? 0.f : mm;
     const uint32_t lanes_per = dv / 4;                 // 16 or 32
     const uint32_t c = lane % lanes_per;
     const uint32_t streams = 64 / lanes_per * WPR;     // slots summed side by side
     const uint32_t stream = (wave % WPR) * (64 / lanes_per) + lane / lanes_per;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     float lsum = 0.f;
-    for (uint32_t s0 = 0; s0 < n; s0 += 64) {
-        const uint32_t cnt = min(64u, n - s0);
-        float w_lane = 0.f, l_lane = 0.f;
-        if (lane < cnt) {
-            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
-            w_lane = fast_exp2(ml.x - ms);
-            l_lane = ml.y * w_lane;
+    float ms = 0.f;
+    if (n <= 64) {
+        // The common case in one round trip after the meta entry: lane s fetches (maximum, normaliser) of slot s and,
+        // without waiting for it, the first round of rows; the weights are worked out while those are on their way.
+        auto load_round = [&](uint32_t j, float4 (&x)[4]) {
+#pragma unroll
+            for (uint32_t u = 0; u < 4; u++) {
+                const uint32_t safe = min(j + u * streams + stream, n - 1);
+                x[u] = *reinterpret_cast<const float4 *>(part_acc + slot_of(safe) * dv + c * 4);
+            }
+        };
+        const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(min(lane, n - 1)) * 2);
+        float4 x[4];
+        load_round(0, x);
+        float mm = lane < n ? ml.x : -INFINITY;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            mm = fmaxf(mm, __shfl_xor(mm, d));
         }
+        ms = mm == -INFINITY ? 0.f : mm;
+        const float w_lane = lane < n ? fast_exp2(ml.x - ms) : 0.f;
+        float l_lane = lane < n ? ml.y * w_lane : 0.f;
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) {
             l_lane += __shfl_xor(l_lane, d);
         }
-        lsum += l_lane;
-        for (uint32_t j = 0; j < cnt; j += 4 * streams) {   // uniform trip count: every lane takes part in the exchanges
-            float4 x[4];
-            float w[4];
-#pragma unroll
-            for (uint32_t u = 0; u < 4; u++) {
-                const uint32_t idx = j + u * streams + stream;
-                const uint32_t safe = min(idx, cnt - 1);
-                x[u] = *reinterpret_cast<const float4 *>(part_acc + slot_of(s0 + safe) * dv + c * 4);
-                w[u] = __shfl(w_lane, static_cast<int>(safe));
-                w[u] = idx < cnt ? w[u] : 0.f;
+        lsum = l_lane;
+        for (uint32_t j = 0; j < n; j += 4 * streams) {   // uniform trip count: every lane takes part in the exchanges
+            if (j > 0) {
+                load_round(j, x);
             }
 #pragma unroll
             for (uint32_t u = 0; u < 4; u++) {
-                acc.x += x[u].x * w[u];
-                acc.y += x[u].y * w[u];
-                acc.z += x[u].z * w[u];
-                acc.w += x[u].w * w[u];
+                const uint32_t idx = j + u * streams + stream;
+                float w = __shfl(w_lane, static_cast<int>(min(idx, n - 1)));
+                w = idx < n ? w : 0.f;
+                acc.x += x[u].x * w;
+                acc.y += x[u].y * w;
+                acc.z += x[u].z * w;
+                acc.w += x[u].w * w;
+            }
+        }
+    } else {
+        float mm = -INFINITY;
+        for (uint32_t s = lane; s < n; s += 64) {
+            mm = fmaxf(mm, part_ml[slot_of(s) * 2]);
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            mm = fmaxf(mm, __shfl_xor(mm, d));
+        }
+        ms = mm == -INFINITY ? 0.f : mm;
+        for (uint32_t s0 = 0; s0 < n; s0 += 64) {
+            const uint32_t cnt = min(64u, n - s0);
+            float w_lane = 0.f, l_lane = 0.f;
+            if (lane < cnt) {
+                const float2 ml = *reinterpret_cast<const float2 *>(part_ml + slot_of(s0 + lane) * 2);
+                w_lane = fast_exp2(ml.x - ms);
+                l_lane = ml.y * w_lane;
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                l_lane += __shfl_xor(l_lane, d);
+            }
+            lsum += l_lane;
+            for (uint32_t j = 0; j < cnt; j += 4 * streams) {   // uniform trip count: every lane takes part in the exchanges
+                float4 x[4];
+                float w[4];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    const uint32_t idx = j + u * streams + stream;
+                    const uint32_t safe = min(idx, cnt - 1);
+                    x[u] = *reinterpret_cast<const float4 *>(part_acc + slot_of(s0 + safe) * dv + c * 4);
+                    w[u] = __shfl(w_lane, static_cast<int>(safe));
+                    w[u] = idx < cnt ? w[u] : 0.f;
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    acc.x += x[u].x * w[u];
+                    acc.y += x[u].y * w[u];
+                    acc.z += x[u].z * w[u];
+                    acc.w += x[u].w * w[u];
+                }
             }
         }
     }
