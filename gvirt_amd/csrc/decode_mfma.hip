@@ -89,7 +89,17 @@ struct DecodeMfmaParams {
     uint32_t only_single;  // 1: the units of the split are the sequences, and only those with one query row take part
     uint32_t unit0, n_units;   // this launch's slice of the units (rows or sequences): unit0 .. unit0 + n_units - 1
     uint32_t step_mult;    // steps (of 16 positions) the kernel takes at a time: chunks are multiples of it
+    uint32_t block_magic;  // floor(2^32 / block_size) + 1: position / block_size == mulhi(position, magic) for positions
+                           // below 2^32 / block_size; 0 when a table reaches further (then the kernels divide)
 };
+
+// block and offset inside it of position t (a division by a run-time block size is some twenty instructions)
+__device__ __forceinline__ uint32_t block_of(const DecodeMfmaParams &p, uint32_t t, uint32_t *off)
+{
+    const uint32_t blk = p.block_magic != 0 ? __umulhi(t, p.block_magic) : t / p.block_size;
+    *off = t - blk * p.block_size;
+    return blk;
+}
 
 // A cache row is read once per decode step: the non-temporal hint keeps it from displacing other lines
 // on its way through the caches. Measured on batch 64 x 4096 positions: the LDS copies of the streaming
@@ -555,7 +565,8 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 return t < t1 ? t : t0;   // exhausted sub range: any valid rows, nobody consumes them
             };
             auto row_of = [&](uint32_t t) -> uint64_t {
-                const uint32_t blk = t / p.block_size, off = t % p.block_size;
+                uint32_t off;
+                const uint32_t blk = block_of(p, t, &off);
                 return (static_cast<uint64_t>(tbl_lds[blk - blk0]) * p.block_size + off) * p.n_kv_heads;
             };
             auto sub_end = [&](uint32_t sub) { return min(t1, t0 + (sub + 1) * sub_len); };
@@ -962,7 +973,8 @@ decode_dma_kernel(const DecodeMfmaParams p)
             auto issue = [&](uint32_t step) {
                 const uint32_t ts = t0 + step * WSTEP;
                 const uint32_t gs = NSUB == 1 ? ts : min(ts + 16 * sub, (t1 - 1) & ~15u);
-                const uint32_t blk = gs / p.block_size, off = gs % p.block_size;
+                uint32_t off;
+                const uint32_t blk = block_of(p, gs, &off);
                 const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
                 const uint64_t row0 = static_cast<uint64_t>(phys) * p.block_size + off;
                 const uint32_t last_rel = min(t1 - 1 - gs, 15u);
@@ -1250,34 +1262,35 @@ decode_dma8_kernel(const DecodeMfmaParams p)
             vr_off[mt] = KBYTES + slot_off(STEP * sub + pos, kvl, mt) + ((lane & 1) << 3);
         }
     }
-    const uint32_t sc_off = 2 * KBYTES + (wave * STEP + 4 * jq) * 4;   // K scales of the first tile's rows
+    // scales of this wave's kv head: block (group, half, head pair) of the scale area, then [K | V][head of the pair][16]
+    const uint32_t sc_off = 2 * KBYTES + (sub * NKV + kvl / 2) * 256 + (kvl & 1u) * 64 + 4 * jq * 4;   // K, first tile
+    constexpr uint32_t kScHalf = (NKV / 2) * 256;   // the second tile's block
     // copy roles: wave w fills bytes 4096 w .. + 4095 of the K and of the V half of a stage with four copies each:
     // 8 kv heads: four positions; 4: eight; 2: sixteen. They are positions of one 16-position half of the wave's own
     // group. Lane = slot (position inside the KiB, kv head, chunk); the slot receives the (kv head, chunk) the
     // position's pattern assigns to it. c_rel: the lane's position inside the half, c_voff: its offset inside the
     // position's cache row.
-    uint32_t c_rel[4], c_voff[4];
+    const uint32_t row_bytes = p.n_kv_heads * HEADB;
+    uint32_t c_rel[4], c_voff[4], c_full[4];   // c_full: the lane's offset from the half's first row when no row is clamped
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t byte = (4 * wave + i) * 1024 + 16 * lane;
         const uint32_t pos = (byte / POSB) & 31u, in_pos = byte % POSB;
         c_rel[i] = pos & 15u;
         c_voff[i] = (in_pos / 256 * 2 + (((in_pos >> 7) & 1u) ^ pat_head(pos))) * HEADB + (((lane & 7u) ^ pat_chunk(pos)) << 4);
-        if constexpr (NKV == 8) {
-            c_rel[i] = uni(c_rel[i]);   // a copy is one position
-        }
+        c_full[i] = c_rel[i] * row_bytes + c_voff[i];
     }
     const uint32_t c_half = ((4 * wave * 1024 / POSB) >> 4) & 1u;   // the half of the group this wave's copies lie in
-    // scale copies: a wave moves the scales of two kv heads of its own group x 32 positions: the K scales if its kv
-    // head is even, the V scales of the same two heads if it is odd
-    const uint32_t sc_wave = (wave & ~1u) + (lane >> 5);   // the wave that reads these scales
-    const uint32_t sc_head = sc_wave % NKV;
-    const uint32_t sc_pos = lane & 31;
-    const float *sc_src = (wave & 1u) ? p.v_scale : p.k_scale;
-    const uint32_t sc_dst = 2 * KBYTES + (wave & 1u) * SCALEB + (wave & ~1u) * STEP * 4;
+    // scale copies: every wave moves the scales it can address with the block lookup of its own half: those of the
+    // half's 16 positions for two kv heads of its group, K and V. Lane = (tensor, head of the pair, position); the 256
+    // bytes land in the wave's own block of the scale area, [tensor][head of the pair][16 positions].
+    const uint32_t sc_pair = (wave % NKV) % (NKV / 2);           // which two kv heads of the group
+    const uint32_t sc_head = 2 * sc_pair + ((lane >> 4) & 1u);
+    const uint32_t sc_pos = lane & 15;
+    const float *sc_src = (lane >> 5) ? p.v_scale : p.k_scale;
+    const uint32_t sc_dst = 2 * KBYTES + wave * 256;
 
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
-    const uint32_t row_bytes = p.n_kv_heads * HEADB;
 
     DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
     split.scan();
@@ -1369,39 +1382,32 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 const uint32_t ts = t0 + step * WSTEP + STEP * sub;   // this wave's group; beyond the end: see below
                 const uint32_t tl = t1 - 1;
                 const uint32_t st = smem_addr + (step & 1) * STAGE;
-                uint64_t row0[2];
-                uint32_t max_i[2];
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const uint32_t hs = min(ts + 16 * h, tl);
-                    const uint32_t blk = hs / p.block_size, off = hs % p.block_size;
-                    const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
-                    row0[h] = static_cast<uint64_t>(phys) * p.block_size + off;
-                    max_i[h] = ts + 16 * h > tl ? 0u : min(tl - (ts + 16 * h), 15u);
-                }
-                const uint64_t my_row0 = c_half ? row0[1] : row0[0];
-                const uint32_t my_max = c_half ? max_i[1] : max_i[0];
+                // one block lookup: everything this wave copies lies in its half of its group
+                const uint32_t hs0 = ts + 16 * c_half;
+                const uint32_t hs = min(hs0, tl);
+                uint32_t off;
+                const uint32_t blk = block_of(p, hs, &off);
+                const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk - blk0]);
+                const uint64_t my_row0 = static_cast<uint64_t>(phys) * p.block_size + off;
+                const uint32_t my_max = hs0 > tl ? 0u : min(tl - hs0, 15u);
                 const char *kb = static_cast<const char *>(p.k_cache) + my_row0 * row_bytes + kv0 * HEADB;
                 const char *vb = static_cast<const char *>(p.v_cache) + my_row0 * row_bytes + kv0 * HEADB;
+                if (my_max == 15) {
+                    // every row of the half exists: the rows' offsets are part of the lanes' precomputed ones
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    if constexpr (NKV == 8) {
-                        const uint32_t src = uni(min(c_rel[i], my_max) * row_bytes);
-                        dma_1k(st + (4 * wave + i) * 1024, c_voff[i], kb + src);
-                        dma_1k(st + KBYTES + (4 * wave + i) * 1024, c_voff[i], vb + src);
-                    } else {
-                        const uint32_t voff = min(c_rel[i], my_max) * POSB + c_voff[i];   // the cache row is the pass
+                    for (int i = 0; i < 4; i++) {
+                        dma_1k(st + (4 * wave + i) * 1024, c_full[i], kb);
+                        dma_1k(st + KBYTES + (4 * wave + i) * 1024, c_full[i], vb);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const uint32_t voff = min(c_rel[i], my_max) * row_bytes + c_voff[i];
                         dma_1k(st + (4 * wave + i) * 1024, voff, kb);
                         dma_1k(st + KBYTES + (4 * wave + i) * 1024, voff, vb);
                     }
                 }
-                {
-                    const bool hi = sc_pos >= 16;
-                    const uint64_t r0 = hi ? row0[1] : row0[0];
-                    const uint32_t mi = hi ? max_i[1] : max_i[0];
-                    const float *src = sc_src + (r0 + min(sc_pos & 15u, mi)) * p.n_kv_heads + kv0 + sc_head;
-                    dma_4b(st + sc_dst, src);
-                }
+                dma_4b(st + sc_dst, sc_src + (my_row0 + min(sc_pos, my_max)) * p.n_kv_heads + kv0 + sc_head);
             };
             auto compute = [&](uint32_t step) {
                 const uint32_t t = t0 + step * WSTEP + STEP * sub;
@@ -1434,9 +1440,9 @@ decode_dma8_kernel(const DecodeMfmaParams p)
                 float ksc[8], vsc[8];
                 {
                     const float4 k0 = *reinterpret_cast<const float4 *>(stage + sc_off);
-                    const float4 k1 = *reinterpret_cast<const float4 *>(stage + sc_off + 64);
-                    const float4 v0 = *reinterpret_cast<const float4 *>(stage + sc_off + SCALEB);
-                    const float4 v1 = *reinterpret_cast<const float4 *>(stage + sc_off + SCALEB + 64);
+                    const float4 k1 = *reinterpret_cast<const float4 *>(stage + sc_off + kScHalf);
+                    const float4 v0 = *reinterpret_cast<const float4 *>(stage + sc_off + 128);
+                    const float4 v1 = *reinterpret_cast<const float4 *>(stage + sc_off + kScHalf + 128);
                     ksc[0] = k0.x, ksc[1] = k0.y, ksc[2] = k0.z, ksc[3] = k0.w;
                     ksc[4] = k1.x, ksc[5] = k1.y, ksc[6] = k1.z, ksc[7] = k1.w;
                     vsc[0] = v0.x, vsc[1] = v0.y, vsc[2] = v0.z, vsc[3] = v0.w;
@@ -1766,6 +1772,9 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
         p.n_units = min(kSplitSeqCap, units - u0);
         int rc;
         p.step_mult = 1;
+        p.block_magic = static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32)
+                            ? static_cast<uint32_t>((1ull << 32) / a.block_size) + 1
+                            : 0u;
         if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             p.step_mult = a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1;
             rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
