@@ -1168,7 +1168,8 @@ int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgro
 // per-position scales follow by 4-byte copies. Bytes become fp16 (exactly) between the LDS read and the
 // matrix product, so a wave reads half the LDS bytes of the 16-bit kernel and writes none.
 // A step is 32 positions = two score tiles of 16. Stage: [K | V][32 positions][8 kv heads][128 bytes], then
-// the scales [K | V][kv head][32 positions]. The 256-byte bank window of LDS holds two kv heads' rows of a
+// the scales in one 256-byte block per copying wave, [16-position half][pair of kv heads][K | V][head of the pair][16
+// positions], so that a lane reads its eight scales of a tensor with two ds_read_b128. The 256-byte bank window of LDS holds two kv heads' rows of a
 // position, so the XOR pattern of a position covers the 16-byte chunk (3 bits) and the kv head's low bit;
 // it is chosen so that the 16 positions of a score tile (K rows as the A operand, ds_read_b128) and the
 // 16 positions one half of the wave gathers for the second product (ds_read_b64_tr_b8) both land in 16
@@ -1222,7 +1223,7 @@ decode_dma8_kernel(const DecodeMfmaParams p)
     constexpr int HEADB = D;                     // bytes of one (position, kv head) row
     constexpr int POSB = NKV * HEADB;            // LDS bytes of one position: the kv heads of the pass
     constexpr int KBYTES = WSTEP * POSB;         // 32 KiB: the K half of a stage
-    constexpr int SCALEB = kWaves * STEP * 4;    // 1 KiB: the K scales of a stage, [wave][32 positions]
+    constexpr int SCALEB = kWaves * STEP * 4;    // 1 KiB: half of a stage's scale area (eight blocks of 256 bytes in all)
     constexpr int XS = D + 16;                   // floats of one head's (O, m, l) on its way to the head's first wave
     constexpr int STAGE = 2 * KBYTES + 2 * SCALEB;
     constexpr int PER_WAVE = 9;                  // copies per wave and step: 4 K rows, 4 V rows, 64 scales
