@@ -30,7 +30,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
-MEASURED_TRAFFIC_BYTES = {"c2": 1080254815, "c3": 335262040, "c4": 306641667, "c5": 1623753891}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080257123, "c3": 335345883, "c4": 306642776, "c5": 1623782068}
 # where each constant comes from: the committed counter summary whose "HBM traffic per launch" line holds it
 TRAFFIC_SOURCE = {"c2": "profiles/decode_dma_kernel_c2_llama3_8b_b64_ctx4096.md",
                   "c3": "profiles/prefill_kernel_c3_qwen25_7b_chunked.md",
