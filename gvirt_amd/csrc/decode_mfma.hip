@@ -1704,7 +1704,8 @@ void decode_split_plan(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint
                        DecodeSplitPlan *pl)
 {
     const uint64_t max_steps = ceil_div(max_num_block * block_size, static_cast<uint32_t>(kStep));
-    const uint64_t chunk_cap = static_cast<uint64_t>(kSplitTblCap - 2) * block_size / kStep;
+    // (the kernels round the cap down to a multiple of the steps they take at a time, at most 16: the bound uses 16)
+    const uint64_t chunk_cap = static_cast<uint64_t>(kSplitTblCap - 2) * block_size / kStep / 16 * 16;
     const uint64_t by_cap = (static_cast<uint64_t>(batch) * max_steps + chunk_cap - 1) / chunk_cap;
     pl->max_chunks = static_cast<uint32_t>(by_cap > kSplitMaxWorkgroups ? by_cap : kSplitMaxWorkgroups);
     pl->meta_bytes = ((static_cast<size_t>(batch) * sizeof(int4) + 255) / 256) * 256;
