@@ -729,11 +729,10 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             using S0 = std::integral_constant<int, 0>;
             using S1 = std::integral_constant<int, 1>;
             // Software pipeline: registers hold steps n+1 and n+2 while step n is computed from LDS.
-            // Every load and LDS write below is unconditional (steps past the end re-read the last
+            // Every load and LDS write below is unconditional (steps past the end read one line of the last
             // step and land in a stage nobody consumes): a conditional prefetch would force the
             // wait for the older batch to assume that the newer one was never issued, i.e. to wait
-            // for everything in flight.
-            const uint32_t last = n_steps - 1;   // n_steps >= 1: the tile is not empty
+            // for everything in flight. (n_steps >= 1: the tile is not empty.)
             issue(0, S0{});
             issue(1u, S1{});
             stage_write(S0{});

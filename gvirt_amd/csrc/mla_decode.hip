@@ -359,7 +359,7 @@ mla_decode_kernel(const MlaDecodeParams p)
                 }
                 if (listed) {
                     const uint32_t valid = __builtin_amdgcn_readfirstlane(mask_lds[step]) >> gi4;
-                    if (__builtin_amdgcn_readfirstlane(mask_lds[step]) != 0xffffffffu) {
+                    if (static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(mask_lds[step])) != 0xffffffffu) {
 #pragma unroll
                         for (int mt = 0; mt < 2; mt++) {
 #pragma unroll

@@ -35,7 +35,6 @@ constexpr int kMTile = kWaves * 32;
 constexpr int BN = 64;                    // positions per KV tile
 constexpr int kStages = 4;
 constexpr size_t kLdsLimit = 160 * 1024;   // LDS of a compute unit: the stages plus the staged block-table row must fit
-constexpr int NT = BN / 32;               // 32-position sub tiles
 constexpr uint32_t kMinSplitTiles = 8;          // a KV split walks at least 512 positions
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
