@@ -135,6 +135,28 @@ def test_decode_few_kv_heads_position_groups_share_a_workgroup(rt, model):
     check(run_attention(rt, w), oracle_attention(w))
 
 
+@pytest.mark.parametrize("model", [(32, 8, 128, torch.bfloat16), (28, 4, 128, torch.bfloat16), (6, 3, 128, torch.float16),
+                                   (14, 2, 64, torch.bfloat16)])
+@pytest.mark.parametrize("kv_dtype", [None, torch.int8])
+def test_decode_block_tables_beyond_the_multiply_high_lookup(rt, model, kv_dtype):
+    """Positions become (block, offset) by a multiply-high with floor(2^32 / block_size) + 1, which is exact below
+    2^32 / block_size positions; a block table that reaches further (here 4096 blocks of 1024 positions) makes the
+    kernels divide instead. The same batch with the table cut to what the contexts need takes the multiply-high path
+    and must give the same bits."""
+    nH, nKV, d, dtype = model
+    w = generic_case(67, [1] * 3, [2999, 1024, 17], nH, nKV, d, 1024, dtype)
+    if kv_dtype is not None:
+        w = quantised(w, kv_dtype)
+    ref = oracle_attention(w)
+    narrow = run_attention(rt, w)
+    check(narrow, ref, max_abs=MAX_ABS if kv_dtype is None else MAX_ABS_INT8)
+    wide = dict(w)
+    rows = w["block_tables"].reshape(w["batch"], w["max_num_block"])
+    wide["block_tables"] = torch.cat([rows, torch.zeros(w["batch"], 4096 - w["max_num_block"], dtype=torch.int32)], 1).reshape(-1)
+    wide["max_num_block"] = 4096
+    assert torch.equal(run_attention(rt, wide), narrow)
+
+
 @pytest.mark.parametrize("model,batch,lo,hi,long_ones", [((32, 8, 128, 128, torch.bfloat16), 100, 1, 3000, [9000, 5000]),
                                                         ((32, 8, 128, 128, torch.bfloat16), 700, 1, 200, [2500]),
                                                         ((16, 8, 128, 16, torch.float16), 70, 1, 900, []),
