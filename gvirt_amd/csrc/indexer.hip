@@ -25,6 +25,11 @@ namespace {
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 constexpr int kWavesPerWg = 4;
 constexpr int kRange = 256;          // positions per wave
+// the kernel for batches with several rows per sequence: 8 rows share the K rows of 1024 positions through LDS
+constexpr int kShWaves = 8;
+constexpr int kShRange = 1024;       // positions per workgroup
+constexpr int kShStage = 64;         // positions per LDS stage (16 KiB)
+constexpr int kShStages = 3;
 constexpr int kSelThreads = 1024;
 constexpr uint32_t kSelStage = 24576;   // scores of a row kept in LDS between the passes (48 KiB)
 
@@ -85,33 +90,18 @@ __device__ __forceinline__ bool find_row(uint32_t t, const int32_t *query_start_
     return true;
 }
 
-// NT = n_heads / 16, head_dim = 128.
+// Scores of query row t (of sequence `seq`, `total` candidate positions) for the positions [p0, p1), by one wave,
+// K rows straight from the cache. NT = n_heads / 16, head_dim = 128.
 template <typename T, int NT>
-__global__ void __launch_bounds__(kWavesPerWg * 64)
-indexer_scores_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
-                      const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
-                      const int32_t *__restrict__ query_start_loc, const int32_t *__restrict__ lens,
-                      const int32_t *__restrict__ cached_lens, const int32_t *__restrict__ block_tables,
-                      uint32_t total_tokens, uint32_t batch, uint32_t block_size, uint32_t max_num_block,
-                      uint32_t ld_scores)
+__device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
+                                                  const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
+                                                  const int32_t *__restrict__ block_tables, uint32_t t, uint32_t seq,
+                                                  uint32_t total, uint32_t p0, uint32_t p1, uint32_t block_size,
+                                                  uint32_t max_num_block, uint32_t ld_scores, uint32_t lane)
 {
     constexpr int D = 128;
     constexpr int KS = D / 32;
     constexpr int H = NT * 16;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t t = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
-    if (t >= total_tokens) {
-        return;
-    }
-    uint32_t seq = 0, total = 0;
-    if (!find_row(t, query_start_loc, lens, cached_lens, batch, &seq, &total)) {
-        return;
-    }
-    const uint32_t p0 = blockIdx.y * kRange;
-    if (p0 >= total) {
-        return;
-    }
-    const uint32_t p1 = min(total, p0 + kRange);
     const uint32_t col = lane & 15, kg = lane >> 4;
 
     // A operands: Q of head 16 nt + col, dims 32 ks + 8 kg .. +8; weights of heads 16 nt + 4 kg .. +4 in the
@@ -190,6 +180,214 @@ indexer_scores_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict
         if (pos0 + 32 < p1) {
             tile(pos0 + 32, kb[2], kb[1]);
         }
+    }
+}
+
+// One wavefront per (query row, range of 256 positions): decode batches, where no two rows share a sequence.
+template <typename T, int NT>
+__global__ void __launch_bounds__(kWavesPerWg * 64)
+indexer_scores_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
+                      const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
+                      const int32_t *__restrict__ query_start_loc, const int32_t *__restrict__ lens,
+                      const int32_t *__restrict__ cached_lens, const int32_t *__restrict__ block_tables,
+                      uint32_t total_tokens, uint32_t batch, uint32_t block_size, uint32_t max_num_block,
+                      uint32_t ld_scores)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t t = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    if (t >= total_tokens) {
+        return;
+    }
+    uint32_t seq = 0, total = 0;
+    if (!find_row(t, query_start_loc, lens, cached_lens, batch, &seq, &total)) {
+        return;
+    }
+    const uint32_t p0 = blockIdx.y * kRange;
+    if (p0 >= total) {
+        return;
+    }
+    indexer_row_range<T, NT>(q, k_cache, weight, scores, block_tables, t, seq, total, p0, min(total, p0 + kRange),
+                             block_size, max_num_block, ld_scores, lane);
+}
+
+// XOR pattern of the 16-byte chunk index of LDS row `row` (256 bytes = one bank window): the rows that one pass of a
+// ds_read_b128 touches (not 16 consecutive lanes: lanes 0-3, 12-15, 20-23, 24-27 go together) get different slots
+__device__ __forceinline__ uint32_t idx_swz(uint32_t row)
+{
+    const uint32_t hi = (row >> 3) & 1;
+    return (((row & 7) ^ (hi << 2)) << 1) | hi;
+}
+// one wave-wide copy of 64 x 16 bytes from per-lane global addresses into 1 KiB of LDS at `lds_addr` + 16 * lane
+__device__ __forceinline__ void idx_dma_1k(uint32_t lds_addr, const void *lane_ptr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\t"
+                 :: "s"(lds_addr), "v"(lane_ptr) : "memory", "m0");
+}
+
+// Batches with several rows per sequence (prefill): the 8 waves of a workgroup take 8 consecutive query rows and,
+// when these belong to one sequence, share its K rows: 64 positions at a time are copied straight into LDS (a ring
+// of three 16 KiB stages, chunks XOR-swizzled by the copy's per-lane addresses) and every wave reads them from
+// there as its B operands, so a K row crosses the L2 once per 8 query rows instead of once per row. A wave's
+// scores of the range collect in LDS and leave 16 bytes per lane at the end. Workgroups whose rows do not all
+// belong to one sequence (its first or last rows, a decode row among them) run the per-row code above.
+template <typename T, int NT>
+__global__ void __launch_bounds__(kShWaves * 64)
+indexer_scores_shared_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
+                             const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
+                             const int32_t *__restrict__ query_start_loc, const int32_t *__restrict__ lens,
+                             const int32_t *__restrict__ cached_lens, const int32_t *__restrict__ block_tables,
+                             uint32_t total_tokens, uint32_t batch, uint32_t block_size, uint32_t max_num_block,
+                             uint32_t ld_scores)
+{
+    constexpr int D = 128;
+    constexpr int KS = D / 32;
+    constexpr int H = NT * 16;
+    constexpr int ROWB = D * 2;
+    constexpr int STAGEB = kShStage * ROWB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint16_t *out_lds = reinterpret_cast<uint16_t *>(smem + kShStages * STAGEB);          // [wave][kShRange]
+    int32_t *row_seq = reinterpret_cast<int32_t *>(smem + kShStages * STAGEB + kShWaves * kShRange * 2);
+    const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
+        static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)));
+    const uint32_t t = blockIdx.x * kShWaves + wave;
+    uint32_t seq = 0, total = 0;
+    const bool valid = t < total_tokens && find_row(t, query_start_loc, lens, cached_lens, batch, &seq, &total);
+    if (lane == 0) {
+        row_seq[wave] = valid ? static_cast<int32_t>(seq) : -1 - static_cast<int32_t>(wave);
+    }
+    __syncthreads();
+    bool same = row_seq[0] >= 0;
+#pragma unroll
+    for (int w = 1; w < kShWaves; w++) {
+        same = same && row_seq[w] == row_seq[0];
+    }
+    const uint32_t p0 = blockIdx.y * kShRange;
+    const uint32_t blk0 = p0 / block_size;
+    // (the block-table entries of the range sit in the lanes of one register: at most 64 of them)
+    const bool shared = __builtin_amdgcn_readfirstlane(
+        same && p0 < total && (min(total, p0 + kShRange) - 1) / block_size - blk0 + 1 <= 64 ? 1 : 0);
+    if (!shared) {
+        if (valid && p0 < total) {
+            indexer_row_range<T, NT>(q, k_cache, weight, scores, block_tables, t, seq, total, p0,
+                                     min(total, p0 + kShRange), block_size, max_num_block, ld_scores, lane);
+        }
+        return;
+    }
+    const uint32_t p1 = min(total, p0 + kShRange);
+    const uint32_t col = lane & 15, kg = lane >> 4;
+
+    // A operands and weights, as in the per-row code
+    uint4 qa[NT][KS];
+    uint2 wa[NT];
+    const uint16_t *qrow = q + static_cast<uint64_t>(t) * H * D;
+    const uint16_t *wrow = weight + static_cast<uint64_t>(t) * (D + H) + D;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            qa[nt][ks] = *reinterpret_cast<const uint4 *>(qrow + (16 * nt + col) * D + 32 * ks + 8 * kg);
+        }
+        uint2 w = make_uint2(0u, 0u);
+        if (col == 0) {
+            const uint16_t *wp = wrow + 16 * nt + 4 * kg;
+            w.x = static_cast<uint32_t>(wp[0]) | (static_cast<uint32_t>(wp[1]) << 16);
+            w.y = static_cast<uint32_t>(wp[2]) | (static_cast<uint32_t>(wp[3]) << 16);
+        }
+        wa[nt] = w;
+    }
+    const int32_t *table = block_tables + static_cast<uint64_t>(seq) * max_num_block;
+    const uint32_t nblk = (p1 - 1) / block_size - blk0 + 1;
+    const int32_t tbl_reg = lane < nblk ? table[blk0 + lane] : 0;
+    // complete these loads before any copy is issued: the copies' completion is counted, and memory operations finish
+    // in order
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            asm volatile("" : "+v"(qa[nt][ks].x), "+v"(qa[nt][ks].y), "+v"(qa[nt][ks].z), "+v"(qa[nt][ks].w));
+        }
+        asm volatile("" : "+v"(wa[nt].x), "+v"(wa[nt].y));
+    }
+    int32_t tbl_pinned = tbl_reg;
+    asm volatile("" : "+v"(tbl_pinned));
+
+    // copy role: wave w moves rows 8 w .. 8 w + 7 of a stage as two copies of four rows; lane = (row of the four, chunk
+    // slot), and the slot receives the chunk the row's pattern assigns to it. Positions beyond the end repeat the last.
+    auto issue = [&](uint32_t s) {
+        const uint32_t st = smem_addr + (s % kShStages) * STAGEB;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t r = 8 * wave + 4 * i + (lane >> 4);
+            const uint32_t pos = min(p0 + s * kShStage + r, total - 1);
+            const uint32_t blk = pos / block_size;
+            const uint32_t phys = static_cast<uint32_t>(__shfl(tbl_pinned, static_cast<int>(blk - blk0)));
+            const unsigned char *src = reinterpret_cast<const unsigned char *>(k_cache) +
+                                       (static_cast<uint64_t>(phys) * block_size + pos % block_size) * ROWB +
+                                       (((lane & 15u) ^ idx_swz(r)) << 4);
+            idx_dma_1k(st + (8 * wave + 4 * i) * ROWB, src);
+        }
+    };
+    // read role: position 16 tile + col of the stage, dims 32 ks + 8 kg .. + 8
+    uint32_t rd_off[4][KS];
+#pragma unroll
+    for (int tl = 0; tl < 4; tl++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            rd_off[tl][ks] = (16 * tl + col) * ROWB + (((4 * ks + kg) ^ idx_swz(16 * tl + col)) << 4);
+        }
+    }
+    uint16_t *my_out = out_lds + wave * kShRange;
+    const uint32_t n_st = ceil_div(p1 - p0, static_cast<uint32_t>(kShStage));
+    issue(0);
+    if (n_st > 1) {
+        issue(1);
+    }
+    for (uint32_t s = 0; s < n_st; s++) {
+        // every copy of this wave so far has landed (those of stage s + 1 were issued a stage's arithmetic ago) ...
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();   // ... and everybody else's; stage s - 1 is free
+        if (s + 2 < n_st) {
+            issue(s + 2);
+        }
+        const unsigned char *stage = smem + (s % kShStages) * STAGEB;
+#pragma unroll
+        for (int tl = 0; tl < 4; tl++) {
+            const uint32_t pos0 = p0 + s * kShStage + 16 * tl;
+            if (pos0 < p1) {
+                f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                uint4 kt[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    kt[ks] = *reinterpret_cast<const uint4 *>(stage + rd_off[tl][ks]);
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) {
+                    f32x4_t sc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ks++) {
+                        sc = Mma<T>::k32(qa[nt][ks], kt[ks], sc);
+                    }
+                    const uint2 sb = make_uint2(T::pack(sc[0], sc[1]), T::pack(sc[2], sc[3]));
+                    acc = Mma<T>::k16(wa[nt], sb, acc);
+                }
+                if (kg == 0) {
+                    my_out[pos0 - p0 + col] = T::from_f32(acc[0]);
+                }
+            }
+        }
+    }
+    // the wave's scores of [p0, p1) leave LDS (written and read by this wave only: the compiler's LDS counter waits
+    // order them): 16 bytes per lane where the row pitch allows, 2-byte pieces for the rest
+    uint16_t *out = scores + static_cast<uint64_t>(t) * ld_scores + p0;
+    const uint32_t n = p1 - p0;
+    const uint32_t n8 = (ld_scores % 8 == 0 && (reinterpret_cast<uint64_t>(scores) & 15u) == 0) ? n & ~7u : 0u;
+    for (uint32_t j = lane * 8; j < n8; j += 64 * 8) {
+        *reinterpret_cast<uint4 *>(out + j) = *reinterpret_cast<const uint4 *>(my_out + j);
+    }
+    for (uint32_t j = n8 + lane; j < n; j += 64) {
+        out[j] = my_out[j];
     }
 }
 
@@ -370,20 +568,35 @@ int launch_scores(hipStream_t stream, const void *q, const void *k_cache, const 
                   const int32_t *block_tables, uint32_t total_tokens, uint32_t n_heads, uint32_t block_size,
                   uint32_t batch, uint32_t max_num_block, uint32_t ld_scores)
 {
+    // several rows per sequence (more rows than sequences): the kernel whose workgroups share K rows through LDS.
+    // 128 heads keep Q in 128 registers per lane, too many for it next to its staging: the per-row kernel.
+    const bool shared = total_tokens > batch && n_heads <= 64;
     const dim3 grid(ceil_div(total_tokens, kWavesPerWg), ceil_div(max_num_block * block_size, kRange), 1);
-#define XL_IDX(NT)                                                                                                    \
-    indexer_scores_kernel<T, NT><<<grid, kWavesPerWg * 64, 0, stream>>>(                                              \
-        static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k_cache), static_cast<const uint16_t *>(weight), \
+    const dim3 grid_sh(ceil_div(total_tokens, kShWaves), ceil_div(max_num_block * block_size, kShRange), 1);
+    const size_t lds_sh = static_cast<size_t>(kShStages) * kShStage * 256 + kShWaves * kShRange * 2 + kShWaves * 4;
+#define XL_IDX_ARGS                                                                                                   \
+    static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k_cache), static_cast<const uint16_t *>(weight), \
         static_cast<uint16_t *>(scores), query_start_loc, lens, cached_lens, block_tables, total_tokens, batch,      \
-        block_size, max_num_block, ld_scores)
+        block_size, max_num_block, ld_scores
+#define XL_IDX(NT) indexer_scores_kernel<T, NT><<<grid, kWavesPerWg * 64, 0, stream>>>(XL_IDX_ARGS)
+#define XL_IDX_SH(NT)                                                                                                 \
+    do {                                                                                                              \
+        auto kernel = indexer_scores_shared_kernel<T, NT>;                                                            \
+        if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds_sh)) {                      \
+            return rc;                                                                                                \
+        }                                                                                                             \
+        kernel<<<grid_sh, kShWaves * 64, lds_sh, stream>>>(XL_IDX_ARGS);                                              \
+    } while (0)
     switch (n_heads / 16) {
-    case 1: XL_IDX(1); break;
-    case 2: XL_IDX(2); break;
-    case 4: XL_IDX(4); break;
+    case 1: if (shared) { XL_IDX_SH(1); } else { XL_IDX(1); } break;
+    case 2: if (shared) { XL_IDX_SH(2); } else { XL_IDX(2); } break;
+    case 4: if (shared) { XL_IDX_SH(4); } else { XL_IDX(4); } break;
     case 8: XL_IDX(8); break;
     default: return fail(XLITE_HIP_EINVAL, __func__, "n_heads must be 16, 32, 64 or 128");
     }
 #undef XL_IDX
+#undef XL_IDX_SH
+#undef XL_IDX_ARGS
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
 }

@@ -92,6 +92,25 @@ def test_indexer_scores_shapes_and_permuted_tables(rt, nH, bs, dtype):
     assert torch.equal(run_scores(rt, ident), got)
 
 
+@pytest.mark.parametrize("nH,bs,dtype", [(64, 64, torch.bfloat16), (16, 16, torch.float16), (32, 48, torch.bfloat16),
+                                         (64, 8, torch.bfloat16), (64, 1, torch.float16), (128, 128, torch.bfloat16)])
+def test_indexer_scores_prefill_rows_share_key_rows(rt, nH, bs, dtype):
+    """Batches with several rows per sequence: workgroups of 8 consecutive rows of one sequence share its K rows through
+    LDS, 1024 positions per workgroup in stages of 64. Three sequences whose row counts leave whole workgroups, a
+    workgroup across a sequence boundary and a partial last one; ranges that end inside a stage, at its end and after
+    one position of the next; blocks of 8 positions and of one (more than 64 table entries per range: the per-row code
+    serves those, as it does 128 heads). The bits must not depend on the block permutation."""
+    c = indexer_case(43, [40, 9, 23], [2500, 1015, 0], nH, bs=bs, dtype=dtype)
+    got = run_scores(rt, c)
+    check_scores(c, got, oracle_scores(c))
+    ident = dict(c)
+    nb = c["batch"] * c["maxblk"]
+    kc2 = torch.zeros_like(c["kc"])
+    kc2[torch.arange(nb)] = c["kc"][c["tables"].long()]
+    ident["kc"], ident["tables"] = kc2, torch.arange(nb).int()
+    assert torch.equal(run_scores(rt, ident), got)
+
+
 def test_indexer_rejects_unsupported_shapes(rt):
     c = indexer_case(43, [1], [10], 24)
     with pytest.raises(RuntimeError):
