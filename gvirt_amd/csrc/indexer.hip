@@ -231,7 +231,7 @@ __device__ __forceinline__ void idx_dma_1k(uint32_t lds_addr, const void *lane_p
 // scores of the range collect in LDS and leave 16 bytes per lane at the end. Workgroups whose rows do not all
 // belong to one sequence (its first or last rows, a decode row among them) run the per-row code above.
 template <typename T, int NT>
-__global__ void __launch_bounds__(kShWaves * 64)
+__global__ void __launch_bounds__(kShWaves * 64, NT <= 4 ? 4 : 2)
 indexer_scores_shared_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
                              const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
                              const int32_t *__restrict__ query_start_loc, const int32_t *__restrict__ lens,
@@ -568,9 +568,8 @@ int launch_scores(hipStream_t stream, const void *q, const void *k_cache, const 
                   const int32_t *block_tables, uint32_t total_tokens, uint32_t n_heads, uint32_t block_size,
                   uint32_t batch, uint32_t max_num_block, uint32_t ld_scores)
 {
-    // several rows per sequence (more rows than sequences): the kernel whose workgroups share K rows through LDS.
-    // 128 heads keep Q in 128 registers per lane, too many for it next to its staging: the per-row kernel.
-    const bool shared = total_tokens > batch && n_heads <= 64;
+    // several rows per sequence (more rows than sequences): the kernel whose workgroups share K rows through LDS
+    const bool shared = total_tokens > batch;
     const dim3 grid(ceil_div(total_tokens, kWavesPerWg), ceil_div(max_num_block * block_size, kRange), 1);
     const dim3 grid_sh(ceil_div(total_tokens, kShWaves), ceil_div(max_num_block * block_size, kShRange), 1);
     const size_t lds_sh = static_cast<size_t>(kShStages) * kShStage * 256 + kShWaves * kShRange * 2 + kShWaves * 4;
@@ -591,7 +590,7 @@ int launch_scores(hipStream_t stream, const void *q, const void *k_cache, const 
     case 1: if (shared) { XL_IDX_SH(1); } else { XL_IDX(1); } break;
     case 2: if (shared) { XL_IDX_SH(2); } else { XL_IDX(2); } break;
     case 4: if (shared) { XL_IDX_SH(4); } else { XL_IDX(4); } break;
-    case 8: XL_IDX(8); break;
+    case 8: if (shared) { XL_IDX_SH(8); } else { XL_IDX(8); } break;
     default: return fail(XLITE_HIP_EINVAL, __func__, "n_heads must be 16, 32, 64 or 128");
     }
 #undef XL_IDX
