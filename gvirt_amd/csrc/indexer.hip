@@ -6,9 +6,10 @@
 // the weights); there is no causal limit inside a sequence and no activation function. Golden:
 // xlite/tests/kernels/indexer_scores.py:96-118.
 //
-// One wavefront owns one query row and a range of 256 positions. Q sits in registers as the A operand of
-// v_mfma_f32_16x16x32 (16 heads x 32 dims per tile), K rows are loaded straight from the paged cache as
-// the B operand (a lane holds 8 dims of one position), so a result tile holds 16 heads x 16 positions
+// A wavefront owns one query row (and, in decode batches, a range of 256 positions; in batches with several rows per
+// sequence eight such waves share the K rows of 1024 positions through LDS). Q sits in registers as the A operand of
+// v_mfma_f32_16x16x32 (16 heads x 32 dims per tile), K rows are the B operand, loaded straight from the paged cache
+// or read from the shared stage (a lane holds 8 dims of one position), so a result tile holds 16 heads x 16 positions
 // with one position per lane column: rounded and packed, it is already the B operand of the second
 // product, whose A operand carries the 16 weights in row 0.
 //
