@@ -251,9 +251,12 @@ mla_decode_kernel(const MlaDecodeParams p)
                 if (listed) {
                     const uint32_t stage = smem_addr + (step % kStages) * STAGE_BYTES;
                     const uint32_t e0 = step * kStep;
+                    // the wave's four entries in one LDS read (a lookup is awaited with every operand read pending)
+                    const uint4 rows = *reinterpret_cast<const uint4 *>(tbl_lds + e0 + r0);
+                    const uint32_t row_of[4] = {rows.x, rows.y, rows.z, rows.w};
 #pragma unroll
                     for (uint32_t i = 0; i < 4; i++) {
-                        const uint64_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[e0 + r0 + i]);
+                        const uint64_t phys = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row_of[i])));
                         dma_1k(stage + (r0 + i) * KC_ROWB, kc_voff ^ (i << 5),
                                reinterpret_cast<const char *>(p.k_cache) + phys * KC_ROWB);
                     }
@@ -776,12 +779,12 @@ int mla_decode_plan(const MlaArgs &a, MlaPlan *pl)
     }
     // half of what one workgroup per compute unit would get if every row were as long as allowed, between 128
     // and 512 positions
-    uint64_t tok = max_ctx * a.total_tokens / static_cast<uint64_t>(n_cu) / 2;
+    // with position lists no row walks more than top_k positions, and a chunk stages one entry per position
+    const uint64_t max_len = a.top_k != 0 && a.top_k < max_ctx ? a.top_k : max_ctx;
+    uint64_t tok = max_len * a.total_tokens / static_cast<uint64_t>(n_cu) / 2;
     tok = tok > 512 ? 512 : (tok < 128 ? 128 : tok);
     pl->chunk_min_steps = static_cast<uint32_t>(tok / kStep);
     pl->n_workgroups = static_cast<uint32_t>(n_cu);
-    // with position lists no row walks more than top_k positions, and a chunk stages one entry per position
-    const uint64_t max_len = a.top_k != 0 && a.top_k < max_ctx ? a.top_k : max_ctx;
     const uint64_t max_steps = (max_len + kStep - 1) / kStep;
     uint64_t chunk_cap = static_cast<uint64_t>(kTblCap - 2) * (dense ? kStep : a.block_size) / kStep;
     if (a.top_k != 0 && chunk_cap > kTblCap / kStep) {
