@@ -569,8 +569,10 @@ int launch_scores(hipStream_t stream, const void *q, const void *k_cache, const 
                   const int32_t *block_tables, uint32_t total_tokens, uint32_t n_heads, uint32_t block_size,
                   uint32_t batch, uint32_t max_num_block, uint32_t ld_scores)
 {
-    // several rows per sequence (more rows than sequences): the kernel whose workgroups share K rows through LDS
-    const bool shared = total_tokens > batch;
+    // eight or more rows per sequence on average: the kernel whose workgroups share K rows through LDS. (Its workgroups
+    // take 1024 positions; with fewer rows per sequence most of them would span sequences and run the per-row code over
+    // ranges four times as long as the per-row kernel's, on a quarter of its waves.)
+    const bool shared = total_tokens >= 8 * static_cast<uint64_t>(batch);
     const dim3 grid(ceil_div(total_tokens, kWavesPerWg), ceil_div(max_num_block * block_size, kRange), 1);
     const dim3 grid_sh(ceil_div(total_tokens, kShWaves), ceil_div(max_num_block * block_size, kShRange), 1);
     const size_t lds_sh = static_cast<size_t>(kShStages) * kShStage * 256 + kShWaves * kShRange * 2 + kShWaves * 4;
