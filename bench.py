@@ -461,11 +461,36 @@ def bench_indexer(args, torch, rt):
     ms = _time_region(torch, step, args.steps)
     kbytes = sum(ctx) * D * 2
     gbs = kbytes / (ms * 1e-3) / 1e9
+
+    # the same operator's scores on a prefill chunk: 2048 rows of one sequence after 6144 cached positions (the rows of a
+    # workgroup share the sequence's K rows through LDS), reported beside the decode figure
+    p_rows, p_cached = 2048, 6144
+    p_maxblk = (p_rows + p_cached + bs - 1) // bs
+    pq = torch.randn(p_rows, nH, D, generator=g, device=dev).bfloat16()
+    pw = torch.randn(p_rows, D + nH, generator=g, device=dev).bfloat16()
+    pkc = torch.randn(p_maxblk + 1, bs, D, generator=g, device=dev).bfloat16()
+    ptab = torch.randperm(p_maxblk + 1, generator=g, device=dev)[:p_maxblk].int()
+    pscores = torch.zeros(p_rows, p_maxblk * bs, dtype=torch.bfloat16, device=dev)
+    pz = torch.zeros(1, dtype=torch.int32, device=dev)
+    plens = torch.full((1,), p_rows, dtype=torch.int32, device=dev)
+    pcl = torch.full((1,), p_cached, dtype=torch.int32, device=dev)
+
+    def pstep():
+        _C.indexer_scores(rt, pq, pkc, pw, pscores, pz, plens, pcl, ptab, nH, D, bs, 1, p_maxblk)
+
+    for _ in range(3):
+        pstep()
+    pms = _time_region(torch, pstep, 10)
+    pflops = 2.0 * p_rows * (p_rows + p_cached) * nH * D
     return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
             "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "idx DSA indexer_topk on the c4 decode batch", "batch": batch, "n_heads": nH, "head_dim": D,
                        "top_k": top_k, "ctx_total": int(sum(ctx)), "key_bytes_per_step": int(kbytes)},
+            "prefill_scores": {"workload": "indexer_scores, %d rows of one sequence after %d cached positions" % (p_rows, p_cached),
+                               "ms": round(pms, 4), "tflops": round(pflops / (pms * 1e-3) / 1e12, 1),
+                               "frac_of_mfma_peak": round(pflops / (pms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                               "kernel": "indexer_scores_shared_kernel"},
             "roofline": {"bound": "hbm", "kernel": "indexer_scores_kernel (+ indexer_select_kernel)", "achieved": round(gbs, 2),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
             "cpu_baseline": None}
