@@ -261,10 +261,24 @@ def bench_prefill(args, torch, rt):
                          w["cached_lens"], w["block_tables"], shape.n_heads, shape.n_kv_heads, shape.head_dim,
                          shape.block_size, w["batch"], w["max_num_block"])
 
-    for _ in range(max(1, args.warmup // 4)):
+    # a step is 2.2 ms: at least 3 warm-up steps and 10 timed ones whatever --steps says, so that the figure
+    # does not hang on the clock ramp after the previous configuration
+    warm = max(3, args.warmup // 4)
+    for _ in range(warm):
         step()
-    steps = max(3, args.steps // 5)
+    steps = max(10, args.steps // 5)
     ms = _time_region(torch, step, steps)
+    step_dist = _launch_dist(torch, step, 20)
+
+    def call(w):
+        return lambda: _C.attention(rt, w["qkv"], w["k_cache"], w["v_cache"], w["output"], w["query_start_loc"], w["lens"],
+                                    w["cached_lens"], w["block_tables"], shape.n_heads, shape.n_kv_heads, shape.head_dim,
+                                    shape.block_size, w["batch"], w["max_num_block"])
+    per_call = []
+    for w in chunks:
+        d = _launch_dist(torch, call(w), 20)
+        d["tflops_at_median"] = round(w["flops"] / (d["median"] * 1e-3) / 1e12, 1)
+        per_call.append(d)
     flops = sum(w["flops"] for w in chunks)
     tokens = sum(w["tokens"] for w in chunks)
     tf = flops / (ms * 1e-3) / 1e12
@@ -301,11 +315,11 @@ def bench_prefill(args, torch, rt):
                          (i, rl, reps, _cpu_info()),
                "max_abs_err_vs_gpu": float(err.max())}
     return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(tf, 2),
-            "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": max(1, args.warmup // 4), "ms_per_step": round(ms, 4),
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "c3 qwen2.5-7b chunked causal prefill", "total_lens": lens, "chunk": 2048,
                        "calls_per_step": len(chunks)},
-            "tokens_per_s": round(tokens / (ms * 1e-3), 1),
+            "tokens_per_s": round(tokens / (ms * 1e-3), 1), "step_ms_dist": step_dist, "chunk_call_ms_dist": per_call,
             "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                          **_traffic("c3"), "algorithmic_flops_per_step": int(flops)},
@@ -562,7 +576,11 @@ def main():
                 others[c] = {"error": "%s: %s" % (type(e).__name__, e)}
             torch.cuda.empty_cache()
         out["other_configs"] = others
+        failed = [c for c, o in others.items() if "error" in o]
+        out["other_configs_failed"] = failed
         print(json.dumps(out), flush=True)
+        if failed:
+            raise SystemExit(1)   # the headline line is out; a broken configuration still fails the run
         return
     todo = ["c2", "c1", "c5", "c3", "c4"] if args.config == "all" else [args.config]
     for c in todo:

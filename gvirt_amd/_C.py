@@ -118,10 +118,12 @@ class Runtime:
         """One scratch pool per Runtime, shared by every call on it: calls that use one Runtime from two
         streams at once race on it (the reference's Runtime is not re-entrant either,
         xlite/csrc/runtime.cpp:42). A pool that was handed out is never freed while the Runtime lives:
-        kernels still queued and captured graphs keep its address."""
+        kernels still queued and captured graphs keep its address. A pool that has to grow at least doubles, so
+        the retired pools together stay smaller than the live one."""
         nbytes = max(nbytes, 1 << 20)
         if self._pool is None or self._pool.numel() < nbytes:
             if self._pool is not None:
+                nbytes = max(nbytes, 2 * self._pool.numel())
                 if torch.cuda.is_current_stream_capturing():
                     raise RuntimeError("Runtime: the scratch pool must grow to %d bytes, which cannot happen while a "
                                        "graph is being captured; run the shape once before the capture or give "

@@ -37,7 +37,7 @@ class DecoderModel:
         if len(norms) != len(layers) + 1:
             raise RuntimeError("DecoderModel: one norm per layer and a final one")
         self.rt, self.layers, self.norms, self.embed, self.lm_head, self.rope = rt, list(layers), list(norms), embed, lm_head, rope
-        self.max_seq_len, self.norm_eps = max_seq_len, norm_eps
+        self.max_batch, self.max_seq_len, self.norm_eps = max_batch, max_seq_len, norm_eps
         cfg = layers[0].cfg
         self.block_size = cfg.block_size
         self.blocks_per_seq = (max_seq_len + cfg.block_size - 1) // cfg.block_size
@@ -51,11 +51,20 @@ class DecoderModel:
             self.caches = [(torch.zeros(nb, cfg.block_size, cfg.n_kv_heads, cfg.head_dim, dtype=dt, device=dev),
                             torch.zeros(nb, cfg.block_size, cfg.n_kv_heads, cfg.head_dim, dtype=dt, device=dev)) for _ in layers]
 
+    def check_batch(self, batch: int, longest: int) -> None:
+        """The caches hold `max_batch` sequences of `max_seq_len` positions: anything beyond would be written and
+        read outside them."""
+        if batch > self.max_batch:
+            raise RuntimeError("DecoderModel: batch of %d sequences exceeds max_batch=%d" % (batch, self.max_batch))
+        if longest > self.max_seq_len:
+            raise RuntimeError("DecoderModel: a sequence of %d positions exceeds max_seq_len=%d" % (longest, self.max_seq_len))
+
     def attn_meta(self, lens: Sequence[int], cached_lens: Sequence[int]) -> _C.ModelAttnMeta:
         """The step's host lists (xlite/tests/models/llama.py:640-651): sequence i uses blocks i * blocks_per_seq ..."""
         meta = _C.ModelAttnMeta()
         meta.lens = [int(x) for x in lens]
         meta.cached_lens = [int(x) for x in cached_lens]
+        self.check_batch(len(meta.lens), max((l + c for l, c in zip(meta.lens, meta.cached_lens)), default=0))
         meta.block_tables = [[i * self.blocks_per_seq + b for b in range((l + c + self.block_size - 1) // self.block_size)]
                              for i, (l, c) in enumerate(zip(meta.lens, meta.cached_lens))]
         return meta
@@ -91,38 +100,40 @@ class DecoderModel:
 
 def generate(model: DecoderModel, prompt_tokens: List[List[int]], max_new_tokens: int, eos_id: int,
              temperature: float = 0.0) -> Tuple[List[List[int]], int]:
-    """xlite/tests/generate.py:52-103 with greedy selection (temperature 0; sampling is outside this path)."""
+    """The rectangular loop of the reference's harness (xlite/tests/generate.py:52-103), greedy: the first call
+    feeds every sequence the shortest prompt's length, every later call one position of every sequence; where a
+    prompt still has a token for the position, that token stands and the model's choice is dropped. Sequences
+    keep stepping after their end token so that the batch stays rectangular; the answer of each is cut at its
+    first end token. Returns the new tokens per sequence and the number of model calls."""
     if temperature > 0:
         raise RuntimeError("generate: only greedy selection (temperature 0) is built")
-    prompt_lens = [len(t) for t in prompt_tokens]
-    if max(prompt_lens) > model.max_seq_len:
+    n = len(prompt_tokens)
+    longest = max(len(t) for t in prompt_tokens)
+    if longest > model.max_seq_len:
         raise RuntimeError("Prompt length exceeds model maximum sequence length (max_seq_len=%d)" % model.max_seq_len)
+    model.check_batch(n, longest)
+    horizon = min(model.max_seq_len, longest + max_new_tokens)
+    known = [[int(x) for x in t] for t in prompt_tokens]     # per sequence: the prompt, then what was chosen
+    ended = [False] * n
+    fed, calls = 0, 0
     dev = model.embed.device
-    total_len = min(model.max_seq_len, max_new_tokens + max(prompt_lens))
-    tokens_cpu = torch.full((len(prompt_tokens), total_len), -1, dtype=torch.int32)
-    for i, t in enumerate(prompt_tokens):
-        tokens_cpu[i, : len(t)] = torch.tensor(t, dtype=torch.int32)
-    prompt_mask = (tokens_cpu != -1).to(dev)
-    tokens = tokens_cpu.to(dev)
-    finished = torch.zeros(len(prompt_tokens), dtype=torch.bool, device=dev)
-    prev_pos, step = 0, 0
-    for cur_pos in range(min(prompt_lens), total_len):
-        logits = model.forward(tokens[:, prev_pos:cur_pos], prev_pos)
-        next_token = logits.argmax(dim=-1).to(torch.int32)
-        next_token = torch.where(prompt_mask[:, cur_pos], tokens[:, cur_pos], next_token)
-        tokens[:, cur_pos] = next_token
-        finished |= torch.logical_and(~prompt_mask[:, cur_pos], next_token == eos_id)
-        prev_pos = cur_pos
-        step += 1
-        if bool(finished.all()):
+    for pos in range(min(len(t) for t in known), horizon):
+        # every sequence holds at least `pos` tokens here: the columns fed .. pos - 1 of the token matrix
+        window = torch.tensor([k[fed:pos] for k in known], dtype=torch.int32, device=dev)
+        choice = model.forward(window, fed).argmax(dim=-1).tolist()
+        calls += 1
+        for i, k in enumerate(known):
+            if len(k) == pos:          # the prompt is used up: the model's token is the sequence's next one
+                k.append(int(choice[i]))
+                ended[i] = ended[i] or k[-1] == eos_id
+        fed = pos
+        if all(ended):
             break
-    out = []
-    for i, toks in enumerate(tokens.tolist()):
-        toks = toks[prompt_lens[i]: prompt_lens[i] + max_new_tokens]
-        if eos_id in toks:
-            toks = toks[: toks.index(eos_id)]
-        out.append(toks)
-    return out, step
+    answers = []
+    for k, t in zip(known, prompt_tokens):
+        new = k[len(t): len(t) + max_new_tokens]
+        answers.append(new[: new.index(eos_id)] if eos_id in new else new)
+    return answers, calls
 
 
 def generate_ragged(model: DecoderModel, prompt_tokens: List[List[int]], max_new_tokens: int, eos_id: int) -> Tuple[List[List[int]], int]:

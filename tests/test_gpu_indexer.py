@@ -99,7 +99,7 @@ def test_indexer_scores_prefill_rows_share_key_rows(rt, nH, bs, dtype):
     LDS, 1024 positions per workgroup in stages of 64. Three sequences whose row counts leave whole workgroups, a
     workgroup across a sequence boundary and a partial last one; ranges that end inside a stage, at its end and after
     one position of the next; blocks of 8 positions and of one (more than 64 table entries per range: the per-row code
-    serves those, as it does 128 heads). The bits must not depend on the block permutation."""
+    serves those); 128 heads take the shared-K code too. The bits must not depend on the block permutation."""
     c = indexer_case(43, [40, 9, 23], [2500, 1015, 0], nH, bs=bs, dtype=dtype)
     got = run_scores(rt, c)
     check_scores(c, got, oracle_scores(c))
