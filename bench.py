@@ -12,8 +12,10 @@ kernel (the decode attention kernel) against the 8 TB/s HBM peak; `cpu_baseline`
 oracle on a bounded sample of the same workload on the host cores.
 
 With no `--config` the same line also carries `other_configs`: configurations 1, 3, 4 and 5 measured in
-the same run, each with its own value, roofline and CPU baseline. `--config c1|c2|c3|c4|c5|idx` prints the
-line of that workload alone; `all` prints one line per configuration (the first is configuration 2).
+the same run, each with its own value, roofline and CPU baseline, and beside configuration 4 the whole `mla_v2`
+operator (`c4_mla_v2`), the attention over the indexer's position lists (`c4_dsa`) and the indexer itself (`idx`).
+`--config c1|c2|c3|c4|c5|idx` prints the line(s) of that workload alone; `all` prints one line per
+configuration (the first is configuration 2).
 
 Cache residency: configurations 2, 3 and 5 stream far more than the 256 MB of last-level cache per step.
 Configuration 4 (233 MB of latent cache) rotates over four distinct cache sets (932 MB) so that no step finds
@@ -426,7 +428,10 @@ def bench_mla(args, torch, rt):
                          (len(sample), len(ctx), sample, reps, _cpu_info()),
                "max_abs_err_vs_gpu": float(err.max())}
     floor_ms = max(w["kv_bytes"] / (HBM_PEAK_GBS * 1e9), w["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12)) * 1e3
-    return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
+    extra = {"c4_mla_v2": _bench_mla_v2(args, torch, rt, s, ctx, sets, wuk, wuv, q_nope, steps),
+             "c4_dsa": _bench_mla_dsa(args, torch, rt, s, ctx, sets, steps)}
+    return {"extra_legs": extra,
+            "metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
             "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, n_sets), "ms_per_step": round(ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "c4 deepseek-r1 MLA absorbed decode", "batch": 32, "n_heads": 128, "ctx_total": int(sum(ctx)),
@@ -440,6 +445,166 @@ def bench_mla(args, torch, rt):
                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), **_traffic("c4"),
                          "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
             "cpu_baseline": cpu}
+
+
+def _line(value, unit, steps, warmup, ms, dtype="bf16"):
+    return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": value, "unit": unit,
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic"}
+
+
+def _time_oracle(fn, budget_s=15.0, max_reps=3):
+    reps, t = 0, 0.0
+    while reps < max_reps and t < budget_s:
+        t1 = time.perf_counter()
+        fn()
+        t += time.perf_counter() - t1
+        reps += 1
+    return t / reps, reps
+
+
+def _bench_mla_v2(args, torch, rt, s, ctx, sets, wuk, wuv, q_nope, steps):
+    """The operator the reference exposes (xlite/csrc/_C.cpp:1234-1301): W_UK absorb einsum + absorbed attention +
+    W_UV einsum in one call, on the configuration-4 batch; cache sets and weight sets used in turn."""
+    from gvirt_amd import _C
+    B, H, C, N, V, R = len(ctx), s.n_heads, s.kv_lora_rank, s.nope_head_dim, s.v_head_dim, s.rope_head_dim
+    out = torch.empty(B, H * V, dtype=torch.bfloat16, device="cuda:0")
+    none = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+    turn = [0]
+
+    def call(x, ku, kv):
+        _C.mla_v2(rt, q_nope, x["qr"], x["k_cache"], x["pe_cache"], ku, kv, out, x["query_start_loc"], x["lens"],
+                  x["cached_lens"], x["block_tables"], H, R, N, V, C, s.block_size, x["batch"], x["max_num_blocks"], s.scale,
+                  none, 0)
+
+    def step():
+        i = turn[0]
+        call(sets[i % len(sets)], wuk[i % len(wuk)], wuv[i % len(wuv)])
+        turn[0] += 1
+
+    for _ in range(max(args.warmup, len(sets))):
+        step()
+    ms = _time_region(torch, step, steps)
+    w = sets[0]
+    wbytes = 2 * H * N * C * 2
+    alg = w["kv_bytes"] + wbytes + q_nope.numel() * 2 + w["qr"].numel() * 2 + out.numel() * 2
+    gbs = alg / (ms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        from oracle import xlite_oracle as O
+        ncpu = _cpu_threads(torch)
+        call(w, wuk[0], wuv[0])
+        torch.cuda.synchronize()
+        sample = [0, len(ctx) // 2]
+        c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in w.items()}
+        mb = w["max_num_blocks"]
+        sub = lambda t: torch.stack([t[i] for i in sample])
+        sub_tables = torch.cat([c["block_tables"].view(len(ctx), mb)[i] for i in sample])
+        qn, ku, kv = q_nope.cpu(), wuk[0].cpu(), wuv[0].cpu()
+
+        def run_oracle():
+            return O.mla_v2_ref(sub(qn), sub(c["qr"]), c["k_cache"], c["pe_cache"], ku, kv,
+                                torch.arange(len(sample), dtype=torch.int32), torch.ones(len(sample), dtype=torch.int32),
+                                sub(c["cached_lens"]), sub_tables, H, R, N, V, C, s.block_size, len(sample), mb, s.scale)
+        ref = run_oracle()
+        got = sub(out.float().cpu()).reshape(ref.shape)
+        err = float((got - ref).abs().max())
+        if err > 2e-2:
+            raise SystemExit("parity check failed in bench (mla_v2): max abs err %g" % err)
+        t_cpu, reps = _time_oracle(run_oracle)
+        sample_bytes = sum(ctx[i] for i in sample) * (C + R) * 2 + wbytes
+        cpu = {"value": round(sample_bytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": ncpu, "kind": "port",
+               "sample": "%d of %d sequences (indices %s) with both weight tensors, %d timed runs of the PyTorch oracle, %s" %
+                         (len(sample), len(ctx), sample, reps, _cpu_info()), "max_abs_err_vs_gpu": err}
+    o = _line(round(gbs, 2), "GB/s", steps, max(args.warmup, len(sets)), ms)
+    o.update({"config": {"workload": "c4_mla_v2: the mla_v2 operator (absorb einsum + attention + W_UV einsum) on the c4 batch",
+                         "batch": B, "n_heads": H, "ctx_total": int(sum(ctx)), "weight_bytes": int(wbytes),
+                         "cache_residency": "%d cache sets and %d weight sets used in turn" % (len(sets), len(wuk))},
+              "tokens_per_s": round(B / (ms * 1e-3), 1),
+              "roofline": {"bound": "hbm", "kernel": "einsum_htd_kernel + mla_decode_kernel + merge_mla_kernel + einsum_kernel",
+                           "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                           "traffic": None, "algorithmic_bytes_per_launch": int(alg)},
+              "cpu_baseline": cpu})
+    return o
+
+
+def _bench_mla_dsa(args, torch, rt, s, ctx, sets, steps):
+    """DeepSeek sparse attention on the configuration-4 batch: the indexer's lists of 2048 positions per row
+    (indexer_topk on random index queries and keys, run once per cache set, untimed) consumed by mla_attention."""
+    from gvirt_amd import workloads as W
+    from gvirt_amd import _C
+    dev = "cuda:0"
+    B, H, C, R, bs, top_k, iH, iD = len(ctx), s.n_heads, s.kv_lora_rank, s.rope_head_dim, s.block_size, 2048, 64, 128
+    g = torch.Generator(device=dev).manual_seed(W.SEED_BASE + 46)
+    lists = []
+    for x in sets:
+        NB, mb = x["k_cache"].shape[0], x["max_num_blocks"]
+        iq = torch.randn(B, iH, iD, generator=g, device=dev).bfloat16()
+        iw = torch.randn(B, iD + iH, generator=g, device=dev).bfloat16()
+        ik = torch.randn(NB, bs, iD, generator=g, device=dev).bfloat16()
+        l = torch.full((B, top_k), -1, dtype=torch.int32, device=dev)
+        _C.indexer_topk(rt, iq, ik, iw, torch.arange(mb * bs, dtype=torch.int32, device=dev), l, x["query_start_loc"],
+                        x["lens"], x["cached_lens"], x["block_tables"], iH, iD, bs, B, mb, top_k)
+        lists.append(l)
+        del iq, iw, ik
+    torch.cuda.synchronize()
+    turn = [0]
+
+    def call(x, l):
+        _C.mla_attention(rt, x["q_absorb"], x["qr"], x["k_cache"], x["pe_cache"], x["o_absorb"], x["query_start_loc"],
+                         x["lens"], x["cached_lens"], x["block_tables"], H, R, C, bs, x["batch"], x["max_num_blocks"],
+                         s.scale, l, top_k)
+
+    def step():
+        i = turn[0] % len(sets)
+        call(sets[i], lists[i])
+        turn[0] += 1
+
+    for _ in range(max(args.warmup, len(sets))):
+        step()
+    ms = _time_region(torch, step, steps)
+    n_pos = sum(min(c, top_k) for c in ctx)
+    alg = n_pos * (C + R) * 2 + B * H * (C + R) * 2 + B * H * C * 2 + B * top_k * 4
+    gbs = alg / (ms * 1e-3) / 1e9
+    flops = n_pos * H * (2 * (C + R) + 2 * C)
+    cpu = None
+    if not args.no_cpu:
+        from oracle import xlite_oracle as O
+        ncpu = _cpu_threads(torch)
+        w, l = sets[0], lists[0]
+        call(w, l)
+        torch.cuda.synchronize()
+        sample = [0, len(ctx) // 2]
+        c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in w.items()}
+        mb = w["max_num_blocks"]
+        sub = lambda t: torch.stack([t[i] for i in sample])
+        sub_tables = torch.cat([c["block_tables"].view(len(ctx), mb)[i] for i in sample])
+        sub_lists = sub(l.cpu()).clamp(min=0)
+
+        def run_oracle():
+            return O.mla_attention_ref(sub(c["q_absorb"]), sub(c["qr"]), c["k_cache"], c["pe_cache"],
+                                       torch.arange(len(sample), dtype=torch.int32), torch.ones(len(sample), dtype=torch.int32),
+                                       sub(c["cached_lens"]), sub_tables, H, R, C, bs, len(sample), mb, s.scale, sub_lists, top_k)
+        ref = run_oracle()
+        got = sub(w["o_absorb"].float().cpu()).reshape(ref.shape)
+        err = float((got - ref).abs().max())
+        if err > 2e-2:
+            raise SystemExit("parity check failed in bench (DSA): max abs err %g" % err)
+        t_cpu, reps = _time_oracle(run_oracle)
+        cpu = {"value": round(len(sample) * top_k * (C + R) * 2 / t_cpu / 1e9, 3), "unit": "GB/s", "cores": ncpu, "kind": "port",
+               "sample": "%d of %d rows (indices %s) over their lists, %d timed runs of the PyTorch oracle, %s" %
+                         (len(sample), len(ctx), sample, reps, _cpu_info()), "max_abs_err_vs_gpu": err}
+    o = _line(round(gbs, 2), "GB/s", steps, max(args.warmup, len(sets)), ms)
+    o.update({"config": {"workload": "c4_dsa: mla_attention over top-k position lists (2048 per row, from indexer_topk) on the c4 batch",
+                         "batch": B, "n_heads": H, "top_k": top_k, "positions_per_step": int(n_pos),
+                         "cache_residency": "%d cache sets used in turn" % len(sets)},
+              "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "tokens_per_s": round(B / (ms * 1e-3), 1),
+              "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<lists> (+ merge_mla_kernel)", "achieved": round(gbs, 2),
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                           "algorithmic_bytes_per_launch": int(alg),
+                           "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
+              "cpu_baseline": cpu})
+    return o
 
 
 def bench_indexer(args, torch, rt):
@@ -496,6 +661,35 @@ def bench_indexer(args, torch, rt):
         pstep()
     pms = _time_region(torch, pstep, 10)
     pflops = 2.0 * p_rows * (p_rows + p_cached) * nH * D
+    cpu = None
+    if not args.no_cpu:
+        # the oracle on two rows of the decode batch: its lists against the operator's (the reference test's 3 % bound)
+        from oracle import xlite_oracle as O
+        ncpu = _cpu_threads(torch)
+        step()
+        torch.cuda.synchronize()
+        sample = [0, batch // 2]
+        sub = lambda t: torch.stack([t[i] for i in sample])
+        tb = torch.cat([tables.view(batch, maxblk)[i] for i in sample]).cpu()
+        qc, wc, kcc, clc = sub(q.cpu()), sub(wgt.cpu()), kc.cpu(), sub(clens.cpu())
+
+        def run_oracle():
+            sc = O.indexer_scores_ref(qc, kcc, wc, torch.arange(len(sample), dtype=torch.int32),
+                                      torch.ones(len(sample), dtype=torch.int32), clc, tb, nH, D, bs, len(sample), maxblk)
+            return O.indexer_topk_ref(sc, top_k)
+        want = run_oracle()
+        got = sub(out.cpu())
+        worst = 0.0
+        for j, i in enumerate(sample):
+            row = got[j, :min(top_k, ctx[i])].tolist()
+            worst = max(worst, len(set(want[j][0]) - set(row)) / max(1, len(row)))
+        if worst > 0.03:
+            raise SystemExit("parity check failed in bench (indexer): %.1f %% of the oracle's list missing" % (100 * worst))
+        t_cpu, reps = _time_oracle(run_oracle)
+        cpu = {"value": round(sum(ctx[i] for i in sample) * D * 2 / t_cpu / 1e9, 3), "unit": "GB/s", "cores": ncpu, "kind": "port",
+               "sample": "%d of %d rows (indices %s), %d timed runs of the PyTorch oracle (scores + selection), %s" %
+                         (len(sample), batch, sample, reps, _cpu_info()),
+               "list_fraction_missing_vs_gpu": round(worst, 5)}
     return {"metric": "decode attn KV-read GB/s (% of HBM peak) + prefill TFLOP/s, 1 MI355X", "value": round(gbs, 2),
             "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -506,8 +700,9 @@ def bench_indexer(args, torch, rt):
                                "frac_of_mfma_peak": round(pflops / (pms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                "kernel": "indexer_scores_shared_kernel"},
             "roofline": {"bound": "hbm", "kernel": "indexer_scores_kernel (+ indexer_select_kernel)", "achieved": round(gbs, 2),
-                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
-            "cpu_baseline": None}
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "algorithmic_bytes_per_launch": int(kbytes)},
+            "cpu_baseline": cpu}
 
 
 def main():
@@ -566,10 +761,13 @@ def main():
         # the headline line (configuration 2) carrying the other configurations measured in the same run
         out = run_config("c2")
         others = {}
-        for c in ("c1", "c3", "c4", "c5"):
+        drop = ("metric", "n_gpus", "higher_is_better", "scaling", "vs_baseline", "data")
+        for c in ("c1", "c3", "c4", "c5", "idx"):
             try:
                 o = run_config(c)
-                for k in ("metric", "n_gpus", "higher_is_better", "scaling", "vs_baseline", "data"):
+                for name, leg in (o.pop("extra_legs", None) or {}).items():   # c4: the whole mla_v2 operator, the DSA lists
+                    others[name] = {k: v for k, v in leg.items() if k not in drop}
+                for k in drop:
                     o.pop(k, None)
                 others[c] = o
             except (Exception, SystemExit) as e:   # the headline line is printed whatever happens to the others
@@ -582,9 +780,13 @@ def main():
         if failed:
             raise SystemExit(1)   # the headline line is out; a broken configuration still fails the run
         return
-    todo = ["c2", "c1", "c5", "c3", "c4"] if args.config == "all" else [args.config]
+    todo = ["c2", "c1", "c5", "c3", "c4", "idx"] if args.config == "all" else [args.config]
     for c in todo:
-        print(json.dumps(run_config(c)), flush=True)
+        o = run_config(c)
+        legs = o.pop("extra_legs", None) or {}
+        print(json.dumps(o), flush=True)
+        for leg in legs.values():
+            print(json.dumps(leg), flush=True)
         torch.cuda.empty_cache()
 
 
