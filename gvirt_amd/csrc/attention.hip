@@ -23,7 +23,7 @@ size_t workspace_bytes_16(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv
                           uint32_t block_size, uint32_t batch, uint32_t max_num_block)
 {
     const uint32_t max_ctx = max_num_block * block_size;
-    if (is_decode_batch(total_tokens, batch)) {
+    if (is_decode_batch(total_tokens, batch) && decode_supported(head_dim)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
             return decode_mfma_workspace_bytes(batch, n_heads, head_dim, block_size, max_num_block);
         }
@@ -139,13 +139,14 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
     }
     if (kv_dtype != XLITE_HIP_KV_SAME &&
         !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
-        XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");
+        XL_REQUIRE(decode_supported(head_dim), "quantised KV caches: head_dim must be 64 or 128");
         if (const int rc = launch_kv_dequant(s, &a)) {   // from here on: 16-bit caches in the workspace
             return rc;
         }
     }
-    if (is_decode_batch(total_tokens, batch)) {
-        XL_REQUIRE(decode_supported(head_dim), "head_dim must be 64 or 128");
+    // head_dim 256 (the reference kernel is generic over headSize, xlite/csrc/kernels/attention.h:39-74, and ships
+    // such models): the generic matrix-core kernel serves decode and prefill batches alike
+    if (is_decode_batch(total_tokens, batch) && decode_supported(head_dim)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
             return launch_decode_mfma(s, a);
         }
@@ -172,7 +173,7 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
         XL_LAUNCH_CHECK();
         return XLITE_HIP_OK;
     }
-    XL_REQUIRE(mfma_gqa_supported(head_dim), "head_dim must be 64 or 128");
+    XL_REQUIRE(mfma_gqa_supported(head_dim), "head_dim must be 64, 128 or 256");
     if (prefill_mfma_supported(a)) {
         return launch_prefill_mfma(s, a);
     }

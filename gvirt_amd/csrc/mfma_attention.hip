@@ -387,7 +387,7 @@ void fill_common(MfmaParams &p, const PartialBuffers &pb)
 
 }  // namespace
 
-bool mfma_gqa_supported(uint32_t head_dim) { return head_dim == 64 || head_dim == 128; }
+bool mfma_gqa_supported(uint32_t head_dim) { return head_dim == 64 || head_dim == 128 || head_dim == 256; }
 
 size_t mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t dv, uint32_t splits)
 {
@@ -461,7 +461,10 @@ int launch_mfma_gqa(hipStream_t stream, const AttentionArgs &a)
     dim3 grid(max_splits, m_tiles, a.n_kv_heads);
     const bool bf = a.dtype == XLITE_HIP_BF16;
     int rc;
-    if (a.head_dim == 128) {
+    if (a.head_dim == 256) {
+        rc = bf ? launch_kernel<BF16, 256, 0, 256, BN, true>(stream, p, grid)
+                : launch_kernel<FP16, 256, 0, 256, BN, true>(stream, p, grid);
+    } else if (a.head_dim == 128) {
         rc = bf ? launch_kernel<BF16, 128, 0, 128, BN, true>(stream, p, grid)
                 : launch_kernel<FP16, 128, 0, 128, BN, true>(stream, p, grid);
     } else {

@@ -82,6 +82,8 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  * block_tables [batch * max_num_block] int32
  * Row r of sequence i attends to cache positions 0 .. cached_lens[i] + r.
  * No softmax scale is applied here (q arrives pre-scaled).
+ * head_dim 64, 128 or 256 (the reference kernel is generic over headSize,
+ * xlite/csrc/kernels/attention.h:39-74; 256 is its Qwen3.5 shape); quantised caches: 64 or 128.
  *
  * workspace   device scratch of at least xlite_hip_attention_workspace_bytes()
  *             (or ..._bytes_kv() for a quantised cache; split-KV partial results;

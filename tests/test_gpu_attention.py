@@ -67,7 +67,9 @@ def test_config1_qwen2_05b_decode(rt):
 # model shapes of xlite/tests/kernels/attention.py:28-39
 MODELS = [(1, 1, 64, torch.float16), (1, 1, 64, torch.bfloat16), (1, 1, 128, torch.bfloat16), (14, 2, 64, torch.bfloat16),
           (5, 1, 128, torch.bfloat16), (8, 1, 128, torch.bfloat16), (4, 1, 128, torch.bfloat16), (32, 32, 128, torch.float16),
-          (20, 20, 128, torch.float16), (32, 8, 128, torch.bfloat16)]
+          (20, 20, 128, torch.float16), (32, 8, 128, torch.bfloat16),
+          # head_dim 256: the Qwen3.5 shape of xlite/tests/models/qwen3_5.py:67-71 (8 / 2 heads), and a 16-bit float one
+          (8, 2, 256, torch.bfloat16), (4, 4, 256, torch.float16)]
 # decode workloads of the same file (:50-59), contexts bounded to what the CPU oracle does in seconds
 DECODE_WORK = [([0], [1]), ([1800], [1]), ([8, 13, 65, 11, 5], [1] * 5), ([4000] * 2, [1] * 2), ([16000, 127], [1] * 2),
                ([127, 128, 129, 255, 256, 257], [1] * 6)]
@@ -390,7 +392,8 @@ PREFILL_WORK = [([0], [30]), ([0], [77]), ([0], [1800]), ([128], [1800]), ([0] *
 
 
 @pytest.mark.parametrize("model", [(1, 1, 64, torch.float16), (1, 1, 128, torch.bfloat16), (14, 2, 64, torch.bfloat16),
-                                   (5, 1, 128, torch.bfloat16), (8, 1, 128, torch.bfloat16), (28, 4, 128, torch.bfloat16)])
+                                   (5, 1, 128, torch.bfloat16), (8, 1, 128, torch.bfloat16), (28, 4, 128, torch.bfloat16),
+                                   (8, 2, 256, torch.bfloat16), (4, 4, 256, torch.float16)])
 @pytest.mark.parametrize("work", PREFILL_WORK)
 def test_prefill_model_grid(rt, model, work):
     """Prefill / chunked-prefill workloads of xlite/tests/kernels/attention.py:42-60 (bounded)."""
@@ -553,3 +556,23 @@ def test_decode_batches_beyond_one_launch_of_the_split(rt, model, batch):
     w = compact_case(91, lens, clens, nH, nKV, d, bs, dtype)
     assert w["k_cache"].numel() * 2 < 2 << 30
     check(run_attention(rt, w), oracle_attention(w))
+
+
+@pytest.mark.parametrize("bs", [16, 128, 48])
+def test_head_dim_256_split_decode_and_chunked_prefill(rt, bs):
+    """head_dim 256 (xlite/tests/models/qwen3_5.py:67, served by the reference's generic kernel,
+    xlite/csrc/kernels/attention.h:39-74): long decode contexts whose KV range is split across workgroups, a chunked
+    prefill behind a long cached context, sequences without rows, other block sizes."""
+    w = generic_case(81, [1] * 5, [9000, 0, 255, 256, 4097], 8, 2, 256, bs, torch.bfloat16, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+    w = generic_case(82, [200, 0, 1, 33], [5000, 10, 700, 0], 8, 2, 256, bs, torch.bfloat16, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
+def test_head_dim_256_quantised_cache_is_refused(rt):
+    w = generic_case(83, [1], [100], 8, 2, 256, 128, torch.bfloat16)
+    kq, ks = O.quantize_kv_int8(w["k_cache"].float())
+    vq, vs = O.quantize_kv_int8(w["v_cache"].float())
+    w.update(k_cache=kq, v_cache=vq, k_scale=ks, v_scale=vs)
+    with pytest.raises(RuntimeError, match="head_dim must be 64 or 128"):
+        run_attention(rt, w)

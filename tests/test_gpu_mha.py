@@ -14,12 +14,14 @@ def _cosin(rot, max_pos, dtype):
     return torch.cat([fr.cos(), fr.sin()], -1).to(dtype)
 
 
-@pytest.mark.parametrize("qk_norm", [False, True])
-def test_mha_layer_prefill_then_decode_steps(rt, qk_norm):
+@pytest.mark.parametrize("qk_norm,head_dim,rot_dim", [(False, 128, 128), (True, 128, 128), (True, 256, 64)])
+def test_mha_layer_prefill_then_decode_steps(rt, qk_norm, head_dim, rot_dim):
+    """The last case is the Qwen3.5 attention shape (xlite/tests/models/qwen3_5.py:67-71: 8 / 2 heads of 256 with
+    qk-norm, a rotary span of a quarter of the head)."""
     from gvirt_amd.mha import MhaConfig, MhaLayer, prepare_attn
     g = torch.Generator().manual_seed(77)
     dt = torch.bfloat16
-    cfg = MhaConfig(hidden=256, n_heads=8, n_kv_heads=2, head_dim=128, rot_dim=128, block_size=16, qk_norm=qk_norm)
+    cfg = MhaConfig(hidden=256, n_heads=8, n_kv_heads=2, head_dim=head_dim, rot_dim=rot_dim, block_size=16, qk_norm=qk_norm)
     cols = (cfg.n_heads + 2 * cfg.n_kv_heads) * cfg.head_dim
     wqkv = (torch.randn(cfg.hidden, cols, generator=g) * cfg.hidden ** -0.5).to(dt)
     wo = (torch.randn(cfg.n_heads * cfg.head_dim, cfg.hidden, generator=g) * (cfg.n_heads * cfg.head_dim) ** -0.5).to(dt)
