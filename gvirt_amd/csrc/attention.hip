@@ -67,6 +67,8 @@ bool quantised_direct(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_hea
 
 }  // namespace
 
+static int run_16bit(hipStream_t s, AttentionArgs &a);
+
 extern "C" size_t xlite_hip_attention_workspace_bytes_kv(uint32_t total_tokens, uint32_t n_heads,
                                                          uint32_t n_kv_heads, uint32_t head_dim,
                                                          uint32_t block_size, uint32_t batch,
@@ -82,6 +84,7 @@ extern "C" size_t xlite_hip_attention_workspace_bytes_kv(uint32_t total_tokens, 
     if (kv_dtype != XLITE_HIP_KV_SAME &&
         !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
         need += kv_dequant_bytes(n_kv_heads, head_dim, block_size, batch, max_num_block);
+        need += kv_dequant_f16_io_bytes(total_tokens, n_heads, n_kv_heads, head_dim);   // bf16 models (the size does not know)
     }
     return need;
 }
@@ -140,10 +143,37 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
     if (kv_dtype != XLITE_HIP_KV_SAME &&
         !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
         XL_REQUIRE(decode_supported(head_dim), "quantised KV caches: head_dim must be 64 or 128");
-        if (const int rc = launch_kv_dequant(s, &a)) {   // from here on: 16-bit caches in the workspace
+        if (const int rc = launch_kv_dequant(s, &a)) {   // from here on: fp16 caches in the workspace
             return rc;
         }
+        if (dtype == XLITE_HIP_BF16) {
+            // a bf16 model: this batch runs in fp16 over the fp16 copy. The streaming prefill kernel converts the
+            // query rows as it loads them and stores bf16; the other kernels get converted queries and an fp16
+            // result buffer in the workspace, converted back afterwards
+            AttentionArgs f = a;
+            f.dtype = XLITE_HIP_FP16;
+            if (!is_decode_batch(total_tokens, batch) && prefill_mfma_supported(f)) {
+                f.io_bf16 = true;
+                return launch_prefill_mfma(s, f);
+            }
+            void *real_out = nullptr;
+            if (const int rc = launch_kv_dequant_f16_begin(s, &a, &real_out)) {
+                return rc;
+            }
+            if (const int rc = run_16bit(s, a)) {
+                return rc;
+            }
+            return launch_kv_dequant_f16_finish(s, a, real_out);
+        }
     }
+    return run_16bit(s, a);
+}
+
+// a batch over 16-bit caches (or a decode batch of the streaming kernels' shapes over a quantised one)
+static int run_16bit(hipStream_t s, AttentionArgs &a)
+{
+    const uint32_t total_tokens = a.total_tokens, n_heads = a.n_heads, n_kv_heads = a.n_kv_heads, head_dim = a.head_dim,
+                   block_size = a.block_size, batch = a.batch, max_num_block = a.max_num_block;
     // head_dim 256 (the reference kernel is generic over headSize, xlite/csrc/kernels/attention.h:39-74, and ships
     // such models): the generic matrix-core kernel serves decode and prefill batches alike
     if (is_decode_batch(total_tokens, batch) && decode_supported(head_dim)) {

@@ -23,6 +23,9 @@ struct AttentionArgs {
     // a batch served by two kernels: kOnlySingle = only the sequences with exactly one query row (the decode
     // kernels), kSkipSingle = all the others (the prefill kernel, the dequantising copy)
     int rows_mode;
+    // a bf16 model over the fp16 copy of a quantised cache, on a kernel that converts at its edges: dtype says
+    // FP16 (the products), qkv and output are bf16
+    bool io_bf16;
 };
 enum { kAllRows = 0, kOnlySingle = 1, kSkipSingle = 2 };
 
@@ -127,6 +130,10 @@ size_t prefill_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uin
 // kv_dequant.hip: the 16-bit copy of a quantised cache's visible blocks, at the front of the workspace
 size_t kv_dequant_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size, uint32_t batch, uint32_t max_num_block);
 int launch_kv_dequant(hipStream_t stream, AttentionArgs *a);
+// bf16 models run over the fp16 copy in fp16: converted queries and an fp16 result buffer in the workspace
+size_t kv_dequant_f16_io_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim);
+int launch_kv_dequant_f16_begin(hipStream_t stream, AttentionArgs *a, void **real_out);
+int launch_kv_dequant_f16_finish(hipStream_t stream, const AttentionArgs &a, void *real_out);
 
 // mla_topk.hip
 size_t mla_topk_scratch_bytes(uint32_t total_tokens, uint32_t kv_lora_rank, uint32_t rope_head_dim, uint32_t top_k);

@@ -3,11 +3,19 @@
 // paged cache in the workspace, addressed by a block table of its own, and the 16-bit kernels run on that.
 // The copy reads one byte and writes two per cached element, which a prefill's matrix work dwarfs; decode
 // batches of the common shapes never come here (decode_mfma.hip reads the bytes directly).
+// The copy is always fp16: a dequantised value (7 or 4 significant bits times an fp32 scale) then carries a
+// rounding of 2^-11 instead of the 2^-8 of bf16, which unscaled queries would amplify. bf16 models run these
+// batches in fp16: the queries are converted into the workspace, the 16-bit kernels compute and store fp16, and
+// the result rows are converted back (values beyond the fp16 range saturate at +-65504).
+#include <algorithm>
+
 #include "attention_common.h"
 
 namespace xlite {
 
 namespace {
+
+__device__ __forceinline__ float clamp_f16(float x) { return fminf(fmaxf(x, -65504.f), 65504.f); }
 
 template <typename T, int KVF>
 __device__ __forceinline__ uint4 dequant8(const uint2 &raw, float scale)
@@ -32,6 +40,10 @@ __device__ __forceinline__ uint4 dequant8(const uint2 &raw, float scale)
             }
             x[j] = f * scale;
         }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        x[j] = clamp_f16(x[j]);
     }
     return make_uint4(T::pack(x[0], x[1]), T::pack(x[2], x[3]), T::pack(x[4], x[5]), T::pack(x[6], x[7]));
 }
@@ -60,20 +72,53 @@ dequant_blocks_kernel(const unsigned char *__restrict__ k_cache, const unsigned 
     }
     const uint32_t rows_here = min(block_size, static_cast<uint32_t>(visible) - j * block_size);   // positions of the block
     const uint64_t phys = static_cast<uint32_t>(block_tables[out_block]);
-    const uint32_t cpr = head_dim / 8;                               // 8-element chunks per (position, kv head) row
+    const uint32_t cpr = head_dim / 16;                              // 16-element chunks per (position, kv head) row
     const uint64_t chunks = static_cast<uint64_t>(rows_here) * n_kv_heads * cpr;
     const unsigned char *src = (is_v ? v_cache : k_cache) + phys * block_size * n_kv_heads * head_dim;
     const float *sc = (is_v ? v_scale : k_scale) + phys * block_size * n_kv_heads;
     uint16_t *dst = (is_v ? v_out : k_out) + out_block * block_size * n_kv_heads * head_dim;
     for (uint64_t c = threadIdx.x; c < chunks; c += blockDim.x) {
-        const uint2 raw = *reinterpret_cast<const uint2 *>(src + c * 8);
-        *reinterpret_cast<uint4 *>(dst + c * 8) = dequant8<T, KVF>(raw, sc[c / cpr]);
+        const uint4 raw = *reinterpret_cast<const uint4 *>(src + c * 16);
+        const float scale = sc[c / cpr];
+        *reinterpret_cast<uint4 *>(dst + c * 16) = dequant8<T, KVF>(make_uint2(raw.x, raw.y), scale);
+        *reinterpret_cast<uint4 *>(dst + c * 16 + 8) = dequant8<T, KVF>(make_uint2(raw.z, raw.w), scale);
     }
     // the rest of a partly visible block: zeros (the 16-bit kernels may load whole tiles and give the positions
     // past the end probability zero, which stale workspace bits that read as NaN would turn into NaN)
     const uint64_t all_chunks = static_cast<uint64_t>(block_size) * n_kv_heads * cpr;
     for (uint64_t c = chunks + threadIdx.x; c < all_chunks; c += blockDim.x) {
-        *reinterpret_cast<uint4 *>(dst + c * 8) = make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4 *>(dst + c * 16) = make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4 *>(dst + c * 16 + 8) = make_uint4(0, 0, 0, 0);
+    }
+}
+
+// q | k | v rows of a bf16 model as fp16 (the whole fused row: the kernels address q inside it)
+__global__ void __launch_bounds__(256)
+rows_bf16_to_f16_kernel(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, uint64_t n_oct)
+{
+    auto one = [](uint32_t w) { return FP16::pack(clamp_f16(BF16::lo(w)), clamp_f16(BF16::hi(w))); };
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < n_oct; i += gridDim.x * 256ull) {
+        const uint4 w = reinterpret_cast<const uint4 *>(src)[i];
+        reinterpret_cast<uint4 *>(dst)[i] = make_uint4(one(w.x), one(w.y), one(w.z), one(w.w));
+    }
+}
+
+// result rows back to bf16, sequence by sequence (x = row chunk, y = sequence); with skip_single the rows of
+// sequences with exactly one query row belong to another kernel, which wrote them in the output's own type
+__global__ void __launch_bounds__(256)
+rows_f16_to_bf16_kernel(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, const int32_t *__restrict__ query_start_loc,
+                        const int32_t *__restrict__ lens, uint32_t row_oct, uint32_t skip_single)
+{
+    const uint32_t i = blockIdx.y;
+    const int32_t n = lens[i];
+    if (n <= 0 || (skip_single && n == 1)) {
+        return;
+    }
+    auto one = [](uint32_t w) { return BF16::pack(FP16::lo(w), FP16::hi(w)); };
+    const uint64_t first = static_cast<uint64_t>(query_start_loc[i]) * row_oct, count = static_cast<uint64_t>(n) * row_oct;
+    for (uint64_t j = blockIdx.x * 256ull + threadIdx.x; j < count; j += gridDim.x * 256ull) {
+        const uint4 w = reinterpret_cast<const uint4 *>(src)[first + j];
+        reinterpret_cast<uint4 *>(dst)[first + j] = make_uint4(one(w.x), one(w.y), one(w.z), one(w.w));
     }
 }
 
@@ -105,7 +150,7 @@ size_t kv_dequant_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_s
 // identity-like table, the rest of the workspace.
 int launch_kv_dequant(hipStream_t stream, AttentionArgs *a)
 {
-    XL_REQUIRE(a->head_dim % 8 == 0, "head_dim must be a multiple of 8");
+    XL_REQUIRE(a->head_dim % 16 == 0, "head_dim must be a multiple of 16");
     const DequantLayout l = dequant_layout(a->n_kv_heads, a->head_dim, a->block_size, a->batch, a->max_num_block);
     if (a->workspace == nullptr || a->workspace_bytes < l.total) {
         return fail(XLITE_HIP_ENOSPC, __func__,
@@ -127,11 +172,7 @@ int launch_kv_dequant(hipStream_t stream, AttentionArgs *a)
     };
     using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
     using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;
-    if (a->dtype == XLITE_HIP_BF16) {
-        a->kv_dtype == XLITE_HIP_KV_INT8 ? launch(BF16{}, I8{}) : launch(BF16{}, F8{});
-    } else {
-        a->kv_dtype == XLITE_HIP_KV_INT8 ? launch(FP16{}, I8{}) : launch(FP16{}, F8{});
-    }
+    a->kv_dtype == XLITE_HIP_KV_INT8 ? launch(FP16{}, I8{}) : launch(FP16{}, F8{});
     XL_LAUNCH_CHECK();
     a->k_cache = k_out;
     a->v_cache = v_out;
@@ -141,6 +182,53 @@ int launch_kv_dequant(hipStream_t stream, AttentionArgs *a)
     a->v_scale = nullptr;
     a->workspace = ws + l.total;
     a->workspace_bytes -= l.total;
+    return XLITE_HIP_OK;
+}
+
+// bf16 models over the fp16 copy: fp16 queries and an fp16 result buffer behind the copy
+size_t kv_dequant_f16_io_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim)
+{
+    const size_t q = (static_cast<size_t>(total_tokens) * (n_heads + 2 * n_kv_heads) * head_dim * 2 + 255) / 256 * 256;
+    const size_t o = (static_cast<size_t>(total_tokens) * n_heads * head_dim * 2 + 255) / 256 * 256;
+    return q + o;
+}
+
+// Rewrites `a` of a bf16 model to an fp16 problem: qkv converted into the workspace, output redirected to an fp16
+// buffer there; *real_out keeps the caller's output for kv_dequant_f16_finish.
+int launch_kv_dequant_f16_begin(hipStream_t stream, AttentionArgs *a, void **real_out)
+{
+    const size_t row = static_cast<size_t>(a->n_heads + 2 * a->n_kv_heads) * a->head_dim;
+    const size_t q_bytes = (static_cast<size_t>(a->total_tokens) * row * 2 + 255) / 256 * 256;
+    const size_t o_bytes = (static_cast<size_t>(a->total_tokens) * a->n_heads * a->head_dim * 2 + 255) / 256 * 256;
+    if (a->workspace == nullptr || a->workspace_bytes < q_bytes + o_bytes) {
+        return fail(XLITE_HIP_ENOSPC, __func__, "workspace too small for the fp16 queries and results of a bf16 batch over a "
+                                                "quantised cache: need " + std::to_string(q_bytes + o_bytes) + " more bytes");
+    }
+    char *ws = static_cast<char *>(a->workspace);
+    const uint64_t octs = static_cast<uint64_t>(a->total_tokens) * row / 8;   // head_dim is a multiple of 16
+    const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>((octs + 255) / 256, 4096));
+    rows_bf16_to_f16_kernel<<<blocks, 256, 0, stream>>>(static_cast<const uint16_t *>(a->qkv), reinterpret_cast<uint16_t *>(ws), octs);
+    XL_LAUNCH_CHECK();
+    *real_out = a->output;
+    a->qkv = ws;
+    a->output = ws + q_bytes;
+    a->dtype = XLITE_HIP_FP16;
+    a->workspace = ws + q_bytes + o_bytes;
+    a->workspace_bytes -= q_bytes + o_bytes;
+    return XLITE_HIP_OK;
+}
+
+int launch_kv_dequant_f16_finish(hipStream_t stream, const AttentionArgs &a, void *real_out)
+{
+    XL_REQUIRE(a.batch <= 65535, "more than 65535 sequences over a quantised cache outside the decode kernels");
+    const uint32_t row_pairs = a.n_heads * a.head_dim / 8;
+    // enough workgroups per sequence for the longest chunk a batch of this size can hold
+    const uint64_t per_seq = static_cast<uint64_t>(a.total_tokens) * row_pairs;
+    const uint32_t bx = static_cast<uint32_t>(std::min<uint64_t>((per_seq + 255) / 256, 256));
+    rows_f16_to_bf16_kernel<<<dim3(bx, a.batch, 1), 256, 0, stream>>>(static_cast<const uint16_t *>(a.output),
+                                                                      static_cast<uint16_t *>(real_out), a.query_start_loc,
+                                                                      a.lens, row_pairs, a.rows_mode == kSkipSingle ? 1u : 0u);
+    XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
 }
 

@@ -20,6 +20,8 @@
 //
 // Replaces attention.h / flash_attention.h for batches with multi-token queries
 // (xlite/csrc/kernels/attention.h:308-492, causal rule softmax_attn_aiv.h:739-741).
+#include <type_traits>
+
 #include "attention_common.h"
 
 namespace xlite {
@@ -116,7 +118,23 @@ __device__ __forceinline__ void dma_wait()
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-template <typename T, int D>
+// eight 16-bit values of storage type FROM as type TO
+template <typename FROM, typename TO>
+__device__ __forceinline__ uint4 convert8(const uint4 &x)
+{
+    if constexpr (std::is_same<FROM, TO>::value) {
+        return x;
+    } else {
+        auto one = [](uint32_t w) {
+            return TO::pack(fminf(fmaxf(FROM::lo(w), -65504.f), 65504.f), fminf(fmaxf(FROM::hi(w), -65504.f), 65504.f));
+        };
+        return make_uint4(one(x.x), one(x.y), one(x.z), one(x.w));
+    }
+}
+
+// T: the type of the caches and of the products; TIO: the type of the query rows and of the output (the same, or
+// bf16 over fp16 caches: a bf16 model over the fp16 copy of a quantised cache)
+template <typename T, int D, typename TIO = T>
 __global__ void __launch_bounds__(kThreads, 1)
 prefill_kernel(const PrefillParams p)
 {
@@ -252,7 +270,7 @@ prefill_kernel(const PrefillParams p)
         const uint16_t *src = p.q + static_cast<uint64_t>(tok) * p.q_tok_stride + static_cast<uint64_t>(head) * D;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            qreg[ks] = m_valid ? *reinterpret_cast<const uint4 *>(src + ks * 16 + half * 8) : make_uint4(0, 0, 0, 0);
+            qreg[ks] = m_valid ? convert8<TIO, T>(*reinterpret_cast<const uint4 *>(src + ks * 16 + half * 8)) : make_uint4(0, 0, 0, 0);
         }
         // the block-table entries of this workgroup's range go to LDS while the query loads are in flight
         for (uint32_t i = __umulhi(first_tile * BN, p.block_magic) + threadIdx.x;
@@ -538,8 +556,8 @@ prefill_kernel(const PrefillParams p)
 #pragma unroll
             for (int kg = 0; kg < 4; kg++) {
                 uint2 o;
-                o.x = T::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
-                o.y = T::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
+                o.x = TIO::pack(O[dt][kg * 4] * inv, O[dt][kg * 4 + 1] * inv);
+                o.y = TIO::pack(O[dt][kg * 4 + 2] * inv, O[dt][kg * 4 + 3] * inv);
                 *reinterpret_cast<uint2 *>(mine + col * PITCH + (dt * 32 + kg * 8 + half * 4) * 2) = o;
             }
         }
@@ -681,7 +699,10 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
                        (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
     const bool bf = a.dtype == XLITE_HIP_BF16;
     XL_REQUIRE(lds <= kLdsLimit, "block table too long for the prefill kernel");
-    const void *kernel = a.head_dim == 128
+    XL_REQUIRE(!a.io_bf16 || a.dtype == XLITE_HIP_FP16, "bf16 rows over fp16 caches: the products are fp16");
+    const void *kernel = a.io_bf16 ? (a.head_dim == 128 ? reinterpret_cast<const void *>(prefill_kernel<FP16, 128, BF16>)
+                                                        : reinterpret_cast<const void *>(prefill_kernel<FP16, 64, BF16>))
+                         : a.head_dim == 128
                              ? (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 128>)
                                    : reinterpret_cast<const void *>(prefill_kernel<FP16, 128>))
                              : (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 64>)
@@ -698,7 +719,13 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
         n_wg = a.n_kv_heads * p.n_mtiles;
     }
     dim3 grid(n_wg, splits, 1);
-    if (a.head_dim == 128) {
+    if (a.io_bf16) {
+        if (a.head_dim == 128) {
+            prefill_kernel<FP16, 128, BF16><<<grid, kThreads, lds, stream>>>(p);
+        } else {
+            prefill_kernel<FP16, 64, BF16><<<grid, kThreads, lds, stream>>>(p);
+        }
+    } else if (a.head_dim == 128) {
         if (bf) {
             prefill_kernel<BF16, 128><<<grid, kThreads, lds, stream>>>(p);
         } else {
@@ -713,7 +740,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     if (splits == 1) {
         return XLITE_HIP_OK;
     }
-    return launch_merge(stream, a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, splits);
+    return launch_merge(stream, a.io_bf16 ? XLITE_HIP_BF16 : a.dtype, a.output, pb, a.total_tokens, a.n_heads, a.head_dim, splits);
 }
 
 }  // namespace xlite
