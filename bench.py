@@ -18,6 +18,10 @@ configuration 3 over an int8 cache (`c3_int8`).
 `--config c1|c2|c3|c3_int8|c4|c5|idx` prints the line(s) of that workload alone; `all` prints one line per
 configuration (the first is configuration 2).
 
+Before its warm-up steps every configuration runs its step, untimed, for 80 ms of GPU time (`device_spin_up_ms`):
+the part's clocks take tens of milliseconds of sustained load to settle, and each timed region follows an idle
+GPU (data set-up, the previous configuration's CPU baseline).
+
 Cache residency: configurations 2, 3 and 5 stream far more than the 256 MB of last-level cache per step.
 Configuration 4 (233 MB of latent cache) rotates over four distinct cache sets (932 MB) so that no step finds
 its cache resident; configuration 1 (0.8 MB) is timed step by step with a 1 GiB fill between the steps.
@@ -62,6 +66,25 @@ def _time_region(torch, fn, iters):
     b.record()
     torch.cuda.synchronize()
     return a.elapsed_time(b) / iters
+
+
+SPIN_UP_MS = 80.0
+
+
+def _spin_up(torch, fn, min_ms=SPIN_UP_MS):
+    """Untimed: calls `fn` until `min_ms` of GPU time have passed. The part is power-managed and takes tens of
+    milliseconds of sustained load to settle its clocks (the MLA decode batch: 0.106 ms per call over the first 52
+    calls after an idle second, 0.088 ms from about the 300th on); every configuration's timed region follows the CPU
+    baseline of the one before, during which the GPU sits idle."""
+    a, b = _events(torch)
+    done = 0.0
+    while done < min_ms:
+        a.record()
+        for _ in range(8):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        done += a.elapsed_time(b)
 
 
 def _launch_dist(torch, fn, launches=100):
@@ -136,6 +159,9 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
             rope()
         attn()
 
+    _spin_up(torch, step)
+    if r is not None:
+        r["inout"].copy_(pristine)   # (rope_and_cache rotates its rows in place)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -230,7 +256,8 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
         "config": {"workload": name, "batch": B, "n_heads": s.n_heads, "n_kv_heads": s.n_kv_heads,
                    "head_dim": s.head_dim, "block_size": s.block_size, "ctx_total": int(sum(ctx)),
                    "ctx_max": int(max(ctx)), "kv_bytes_per_step": int(kv_bytes),
-                   "launch": "graph replay" if args.graph else "eager", "cache_residency": residency},
+                   "launch": "graph replay" if args.graph else "eager", "cache_residency": residency,
+                   "device_spin_up_ms": SPIN_UP_MS},
         "pct_of_hbm_peak": round(100.0 * kv_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "kernel_ms": {"attention": round(ms_kernel, 4), "rope_and_cache": round(ms_rope, 4)},
@@ -276,6 +303,7 @@ def bench_prefill(args, torch, rt, int8=False):
     # a step is 2.2 ms: at least 3 warm-up steps and 10 timed ones whatever --steps says, so that the figure
     # does not hang on the clock ramp after the previous configuration
     warm = max(3, args.warmup // 4)
+    _spin_up(torch, step)
     for _ in range(warm):
         step()
     steps = max(10, args.steps // 5)
@@ -364,6 +392,7 @@ def bench_mla(args, torch, rt):
         run(sets[turn[0] % n_sets])
         turn[0] += 1
 
+    _spin_up(torch, step)
     for _ in range(max(args.warmup, n_sets)):
         step()
     steps = ((max(args.steps, n_sets) + n_sets - 1) // n_sets) * n_sets   # every set equally often
@@ -392,8 +421,7 @@ def bench_mla(args, torch, rt):
         et[0] += 1
 
     for f in (absorb, unabsorb):
-        for _ in range(3):
-            f()
+        _spin_up(torch, f, 20.0)
     ms_abs = _time_region(torch, absorb, 32)
     ms_unabs = _time_region(torch, unabsorb, 32)
     wbytes = H * N * C * 2
@@ -496,6 +524,7 @@ def _bench_mla_v2(args, torch, rt, s, ctx, sets, wuk, wuv, q_nope, steps):
         call(sets[i % len(sets)], wuk[i % len(wuk)], wuv[i % len(wuv)])
         turn[0] += 1
 
+    _spin_up(torch, step)
     for _ in range(max(args.warmup, len(sets))):
         step()
     ms = _time_region(torch, step, steps)
@@ -574,6 +603,7 @@ def _bench_mla_dsa(args, torch, rt, s, ctx, sets, steps):
         call(sets[i], lists[i])
         turn[0] += 1
 
+    _spin_up(torch, step)
     for _ in range(max(args.warmup, len(sets))):
         step()
     ms = _time_region(torch, step, steps)
@@ -649,6 +679,7 @@ def bench_indexer(args, torch, rt):
     def step():
         _C.indexer_topk(rt, q, kc, wgt, idx, out, qsl, lens, clens, tables, nH, D, bs, batch, maxblk, top_k)
 
+    _spin_up(torch, step)
     for _ in range(args.warmup):
         step()
     ms = _time_region(torch, step, args.steps)
@@ -671,8 +702,7 @@ def bench_indexer(args, torch, rt):
     def pstep():
         _C.indexer_scores(rt, pq, pkc, pw, pscores, pz, plens, pcl, ptab, nH, D, bs, 1, p_maxblk)
 
-    for _ in range(3):
-        pstep()
+    _spin_up(torch, pstep)
     pms = _time_region(torch, pstep, 10)
     pflops = 2.0 * p_rows * (p_rows + p_cached) * nH * D
     cpu = None

@@ -536,6 +536,10 @@ mla_decode_kernel(const MlaDecodeParams p)
     __shared__ uint32_t scan_ws[kWaves];
     __shared__ uint32_t found[4];
     const uint32_t B = p.batch, T = p.total_rows;
+    // Workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own; consecutive chunks are parts of
+    // one row and read the same 147 KB of queries, so chunk numbers follow the XCD first: XCD x takes the chunks
+    // x G / 8 .. (x + 1) G / 8 - 1, and a row's query block is fetched from memory once, not once per chunk.
+    const uint32_t wg = gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
     // the sequence that owns query row t (query_start_loc is a prefix sum), or B. A batch of one row per
     // sequence answers with one round of loads.
     auto seq_of = [&](uint32_t t) {
@@ -616,7 +620,7 @@ mla_decode_kernel(const MlaDecodeParams p)
             }
         }
         if (fits) {
-            const uint32_t c = blockIdx.x;
+            const uint32_t c = wg;
             if (c >= n_chunks) {
                 return;
             }
@@ -649,7 +653,7 @@ mla_decode_kernel(const MlaDecodeParams p)
         // no bound within reach (rows far longer than the staging allows): the general split below
     }
 
-    for (uint32_t c = blockIdx.x;; c += gridDim.x) {
+    for (uint32_t c = wg;; c += gridDim.x) {
         // block-wide prefix sums of the rows' step counts (redone for every chunk: nothing of it stays in
         // registers while a segment runs)
         const uint32_t per = ceil_div(T, kNT);
