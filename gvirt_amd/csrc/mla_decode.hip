@@ -170,6 +170,13 @@ mla_decode_kernel(const MlaDecodeParams p)
                 qreg[KS_C + ks] = qq[4 * ks];
             }
         };
+        // The block-table entries of the segment are requested before the query rows (memory operations finish in
+        // order: behind the 147 KB of queries the first copies would start five microseconds later) ...
+        const uint32_t nblk_seg = dense || listed ? 0 : (t1 - 1) / p.block_size - blk0 + 1;
+        uint32_t tbl_first = 0;
+        if (threadIdx.x < nblk_seg) {
+            tbl_first = static_cast<uint32_t>(table[blk0 + threadIdx.x]);
+        }
         load_q(0);
         if (listed) {
             // cache row of every list entry of the segment (tbl_lds[i] for entry t0 + i) and, per step, the mask
@@ -196,8 +203,11 @@ mla_decode_kernel(const MlaDecodeParams p)
             }
         } else if (!dense) {
             // block-table entries of the tile (lookups in the loop then cost an LDS read only)
-            const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
-            for (uint32_t i = threadIdx.x; i < nblk; i += kNT) {
+            // ... and stored here, with the query loads still in flight (segments of more than 512 blocks: the rest)
+            if (threadIdx.x < nblk_seg) {
+                tbl_lds[threadIdx.x] = tbl_first;
+            }
+            for (uint32_t i = threadIdx.x + kNT; i < nblk_seg; i += kNT) {
                 tbl_lds[i] = static_cast<uint32_t>(table[blk0 + i]);
             }
         }
@@ -447,17 +457,20 @@ mla_decode_kernel(const MlaDecodeParams p)
             // the wait counts are exact.
             const uint32_t last = n_steps - 1;
             __syncthreads();   // the previous pass has left the stages
-#pragma unroll
-            for (int i = 0; i < kDepth; i++) {
-                issue(min(static_cast<uint32_t>(i), last));
-            }
-            // The query loads were issued before these copies and complete before them (memory operations finish
-            // in order); their latency overlaps the copies'. They must have landed before the loop: a wait for
-            // them inside it would also wait for the cache copies in flight. The wait the compiler places here
-            // counts the copies too, so it errs on the late side.
+            issue(0);
+            // The query loads were issued before this copy and complete before it (memory operations finish in
+            // order); their latency overlaps the copy's. They must have landed before the loop: a wait for them
+            // inside it would also wait for the cache copies in flight. The wait the compiler places here counts
+            // the copies too (it does not know of them), so only the first step's are issued ahead of it: every
+            // workgroup of the launch starts at once, and with three steps of each in the burst the first products
+            // waited for all of it (27 MB across the chip) instead of a third.
 #pragma unroll
             for (int ks = 0; ks < KS_C + KS_R; ks++) {
                 asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+            }
+#pragma unroll
+            for (int i = 1; i < kDepth; i++) {
+                issue(min(static_cast<uint32_t>(i), last));
             }
             f32x4_t S[2];
             for (uint32_t it = 0; it < n_steps; it++) {
@@ -588,8 +601,12 @@ mla_decode_kernel(const MlaDecodeParams p)
     if (T <= 64) {
         uint32_t my_seq = B, my_causal = 0, my_limit = 0, my_n = 0;
         if (lane < T) {
-            my_seq = seq_of(lane);
-            my_causal = row_causal(lane, my_seq);
+            // a decode batch has row t in sequence t: that sequence's cached length is fetched in the same round of
+            // loads as the answer to "which sequence" (one memory round trip instead of two)
+            const uint32_t guess = lane < B ? static_cast<uint32_t>(p.cached_lens[lane]) : 0u;
+            const bool own = lane < B && p.query_start_loc[lane] == static_cast<int32_t>(lane) && p.lens[lane] == 1;
+            my_seq = own ? lane : seq_of(lane);
+            my_causal = own && !dense ? guess + 1 : row_causal(lane, my_seq);
             my_limit = LISTS && my_causal > p.top_k ? p.top_k : my_causal;
             my_n = ceil_div(my_limit, static_cast<uint32_t>(kStep));
             if (my_n == 0 && blockIdx.x == 0 && wave == 0) {
