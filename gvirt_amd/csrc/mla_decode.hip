@@ -1,15 +1,21 @@
 // DeepSeek-style absorbed MLA decode on the matrix cores, split along the KV axis.
 //
-// One latent "kv head" is shared by all query heads, so the heads are the MFMA columns: a workgroup of eight
-// wavefronts (two per SIMD, 256 registers each, all of them ordinary vector registers) covers up to 128
-// heads, 16 per wave. A row's positions are walked in steps of 32:
+// One latent "kv head" is shared by all query heads. A workgroup of eight wavefronts (two per SIMD, 256 registers
+// each, all of them ordinary vector registers) covers up to 128 heads; a row's positions are walked in steps of 32:
 //   S^T[pos][head]  = [kc | pe][pos][:] . [q_absorb | qr][head][:]   2 x 18 v_mfma_f32_16x16x32_bf16
-//   O^T[c][head]   += kc^T[c][pos] . P^T[pos][head]                   32 x v_mfma_f32_16x16x32_bf16
-// A lane holds Q of one head for a quarter of every 32-element k-step (72 registers) and 128 O^T
-// accumulators. The cache never passes through registers: every wave copies its share of a step straight
-// from global memory into LDS (global_load_lds_dwordx4, 1 KiB of consecutive cache bytes per instruction)
-// into a ring of four 36 KiB stages, three steps in flight while the fourth is consumed, one barrier per
-// step. K rows are read from LDS as MFMA A operands with ds_read_b128; the latent is read again,
+//   O^T[c][head]   += kc^T[c][pos] . P^T[pos][head]                   16 x v_mfma_f32_32x32x16_bf16
+// The two products split the work differently. Scores by heads: wave w owns heads 16 w .. 16 w + 15 (Q in 72
+// registers per lane, the online softmax state of its heads). The second product by latent columns: wave w owns
+// columns 64 w .. 64 w + 63 of O^T for ALL heads (128 accumulators per lane): it reads only its own eighth of the
+// transposed latent from LDS, once for the 128 heads, and takes the probabilities of the other waves' heads from
+// LDS, where every wave leaves the 1 KiB of its heads after the softmax (with the factor by which the reference
+// maximum moved). Per step that is 16 + 16 LDS operand reads and products of 32 x 32 heads instead of 64 reads and
+// 32 products per wave. The probabilities of step i are consumed one step later (behind the barrier of step i + 1,
+// which the copies need anyway), so there is still one barrier per step.
+// The cache never passes through registers: every wave copies its share of a step straight from global memory
+// into LDS (global_load_lds_dwordx4, 1 KiB of consecutive cache bytes per instruction) into a ring of three 36 KiB
+// stages (the step whose scores are being formed, the one before it whose second product is running, the one after
+// it in flight). K rows are read from LDS as MFMA A operands with ds_read_b128; the latent is read again,
 // transposed, with ds_read_b64_tr_b16, so the same LDS bytes serve both products. The 16-byte chunks of a
 // row are XOR-swizzled (by choosing which global chunk a lane copies) so that both read shapes are
 // bank-conflict free.
@@ -31,38 +37,38 @@ constexpr float kRescaleSlack = 8.0f;
 constexpr int kWaves = 8;
 constexpr int kNT = kWaves * 64;
 constexpr int kStep = 32;
-constexpr int kStages = 4;
-constexpr int kDepth = 3;                // steps whose copies are in flight
+constexpr int kStages = 3;
 constexpr int kAhead = 4;               // operand fetches in flight ahead of the matrix instruction using them
-constexpr int VB = 4;                   // transposed-operand buffers: the fetches run three tiles ahead of the products
 constexpr int C = 512;                 // kv_lora_rank
 constexpr int R = 64;                  // rope_head_dim
 constexpr int KS_C = C / 32;           // k-steps over the latent part
 constexpr int KS_R = R / 32;           // k-steps over the rotary part
-constexpr int DT = C / 16;             // 16-row tiles of O^T
+constexpr int kHeads = 16 * kWaves;    // heads of one pass
+constexpr int HG = kHeads / 32;        // 32-head groups of the second product
+constexpr int WC = C / kWaves;         // latent columns a wave owns in the second product
+constexpr int CT = WC / 32;            // its 32-column tiles
 constexpr int KC_ROWB = C * 2;         // 1024: LDS bytes of a latent row
 constexpr int PE_ROWB = R * 2;         // 128
 constexpr int KC_BYTES = kStep * KC_ROWB;             // 32 KiB
 constexpr int STAGE_BYTES = KC_BYTES + kStep * PE_ROWB;  // 36 KiB: latent rows, then rotary rows
 constexpr int PE_WAVES = kStep * PE_ROWB / 1024;      // waves that also copy 1 KiB of rotary rows
-constexpr int TR_ROWB = C * 2 + 16;    // row pitch of the output transposition
+constexpr int P_ROWB = kStep * 2;      // a head's probabilities of one step
+constexpr int P_BYTES = kHeads * P_ROWB;   // 8 KiB: two such buffers, used in turn
+constexpr int F_BYTES = kHeads * 4;    // one fp32 per head: two buffers of rescale factors, one of final normalisers
+constexpr int TR_ROWB = WC * 2 + 16;   // row pitch of the output transposition (a head's 64 columns of one wave)
 constexpr uint32_t kTblCap = 3000;     // block-table entries of a segment staged in LDS
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 
 // XOR patterns for the 16-byte chunk index inside a row.
-// Latent rows (1024 bytes, every row starts at bank 0): low four chunk bits. The hardware serves a ds_read_b128
-// in four passes of 16 lanes, and a pass is not 16 consecutive lanes: lanes 0-3, 12-15, 20-23 and 24-27 go together,
-// then 4-11, 16-19 and 28-31 (the upper half of the wave likewise). With lane = 16 j + row that is rows 0-3 and 12-15
-// of one 16-byte column group next to rows 4-11 of its neighbour, so the rows 0-3 and 12-15 must own complete pairs
-// of slots (2k, 2k + 1): measured with the pattern ((row & 7) << 1) | (row >> 3), which gives 16 consecutive lanes
-// 16 different slots, every K read took 8 cycles instead of 4. The 8 rows that one transposing pass (32 lanes)
-// touches get 8 different 32-byte groups.
-__device__ __forceinline__ uint32_t swz_kc(uint32_t row)
-{
-    const uint32_t hi = (row >> 3) & 1;
-    return (((row & 7) ^ (hi << 2)) << 1) | hi;
-}
+// Latent rows (1024 bytes, every row starts at bank 0): the pattern is even (a chunk pair stays a pair). The
+// hardware serves a ds_read_b128 in four passes of 16 lanes, and a pass is not 16 consecutive lanes: lanes 0-3, 12-15,
+// 20-23 and 24-27 go together, then 4-11, 16-19 and 28-31 (the upper half of the wave likewise). With lane = 16 j + row
+// (j picks one of four consecutive chunks) a pass is rows 0-3 and 12-15 of one chunk next to rows 4-11 of its odd
+// neighbour: half the pattern must be a bijection onto 0..7 on either row set. The transposing reads of the second
+// product touch four consecutive rows 4 t .. 4 t + 3 per pass (32 lanes, 64 bytes of each row): their patterns differ
+// in the two upper bits, so they land in four different 64-byte groups.
+__device__ __forceinline__ uint32_t swz_kc(uint32_t row) { return ((row & 3) << 2) | (((row >> 2) & 1) << 1); }
 // Rotary rows (128 bytes, two per bank window): low three chunk bits; rows of equal parity differ.
 __device__ __forceinline__ uint32_t swz_pe(uint32_t row) { return (row >> 1) & 7; }
 
@@ -97,12 +103,14 @@ __device__ __forceinline__ void dma_wait()
 
 // LISTS: rows may come with position lists (p.top_k != 0); a separate instantiation, so that the plain kernel
 // keeps its register allocation.
-template <bool LISTS>
+template <bool LISTS, int HGN>
 __global__ void __launch_bounds__(kNT)
 mla_decode_kernel(const MlaDecodeParams p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE_BYTES);
+    unsigned char *p_lds = smem + kStages * STAGE_BYTES;                        // probabilities: 2 x [head][32 positions]
+    float *f_lds = reinterpret_cast<float *>(p_lds + 2 * P_BYTES);              // 2 x rescale factors, then normalisers
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(p_lds + 2 * P_BYTES + 3 * F_BYTES);
     uint32_t *mask_lds = tbl_lds + kTblCap;   // kTblCap / kStep + 2 words: valid positions of a listed row's steps
     const uint32_t smem_addr = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
         static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
@@ -116,25 +124,31 @@ mla_decode_kernel(const MlaDecodeParams p)
     // ---- per-lane address roles, recomputed from the lane index at every step (a dozen vector
     // instructions) instead of living in registers for the whole kernel.
     // Copy roles: wave w moves latent rows 4w .. 4w+3 (lane = chunk slot; a slot holds chunk
-    // slot ^ pattern(row), and the pattern of row 4w + i is that of row 4w XOR 2i) and, for w < 4, rotary
+    // slot ^ pattern(row), and the pattern of row 4w + i is (i << 2) | ((w & 1) << 1)) and, for w < 4, rotary
     // rows 8w .. 8w+7 (lane / 8 = row, lane % 8 = chunk slot).
-    // Read roles: K rows as the A operand (row = position 16 mt + col, chunk 4 ks + gi); transposed latent:
-    // the 16-lane group gi covers positions 4 gi .. 4 gi + 3 (+16 for the second read); lane 4 j' + q points
-    // at elements [4 q, +4) of position 4 gi + j' inside the tile's 16 columns.
-    uint32_t kc_voff, pe_voff, pe_row, kx, px, k_row, p_row, vr_off, gi4;
+    // Score product: K rows as the A operand (row = position 16 mt + col, chunk 4 ks + gi).
+    // Second product (32 x 32 x 16, lane = 32 half + n): n is a latent column of the tile (A) and a head of the
+    // group (B, D), `half` picks 8 of a k-step's 16 positions. Transposed latent: the 16-lane group (half, cg)
+    // covers positions 8 half .. + 3 (+4 for the second read) of a k-step and columns 16 cg .. + 15 of the tile;
+    // lane 4 j' + q of the group points at elements [4 q, +4) of position 8 half + j'.
+    uint32_t kc_voff, pe_voff, pe_row, kx, px, k_row, p_row, gi4, vt0, vt1, pr_off;
     auto set_roles = [&](uint32_t ln) {
         const uint32_t c4 = ln & 15, g = ln >> 4;
         gi4 = g * 4;
-        kc_voff = ((ln & ~15u) | ((ln & 15u) ^ swz_kc(4 * wave))) << 4;   // (row 4 wave + i: this ^ (i << 5))
+        kc_voff = ((ln & ~15u) | ((ln & 15u) ^ swz_kc(4 * wave))) << 4;   // (row 4 wave + i: this ^ (i << 6))
         pe_row = (wave & (PE_WAVES - 1)) * 8 + (ln >> 3);
         pe_voff = ((ln & 7u) ^ swz_pe(pe_row)) << 4;
         kx = (g ^ swz_kc(c4)) << 4;
         px = (g ^ swz_pe(c4)) << 4;
         k_row = c4 * KC_ROWB;
         p_row = KC_BYTES + c4 * PE_ROWB;
-        const uint32_t jp = (ln & 15) >> 2, q = ln & 3;
-        const uint32_t pos = 4 * g + jp;
-        vr_off = pos * KC_ROWB + (((q >> 1) ^ swz_kc(pos)) << 4) + ((q & 1) << 3);
+        const uint32_t hf = ln >> 5, cg = (ln >> 4) & 1, jp = (ln & 15) >> 2, q = ln & 3, n = ln & 31;
+        // the wave's columns start at chunk 8 w; tile ct adds 4 chunks (XOR of bit 6 of the byte offset)
+        const uint32_t chunk = 8 * (wave & 1) + 2 * cg + (q >> 1);
+        vt0 = (8 * hf + jp) * KC_ROWB + (wave >> 1) * 256 + ((chunk ^ ((jp << 2) | 0u)) << 4) + ((q & 1) << 3);
+        vt1 = (8 * hf + 4 + jp) * KC_ROWB + (wave >> 1) * 256 + ((chunk ^ ((jp << 2) | 2u)) << 4) + ((q & 1) << 3);
+        // probabilities of head n of a 32-head group: 16 bytes = the 8 positions of this half of a k-step
+        pr_off = n * P_ROWB + ((hf ^ ((n >> 2) & 3)) << 4);
     };
     set_roles(lane);
 
@@ -215,22 +229,23 @@ mla_decode_kernel(const MlaDecodeParams p)
 
         // passes over groups of 128 heads
         for (uint32_t h0 = 0; h0 < p.n_heads; h0 += 16 * kWaves) {
-            const uint32_t hw = h0 + wave * 16;
-            const uint32_t head = hw + col;
-            const bool h_ok = head < p.n_heads;
-
             if (h0 != 0) {
                 load_q(h0);
             }
-            f32x4_t O[DT];
+            // O^T of the wave's 64 columns for all heads of the pass: tile (ct, hg) is columns 32 ct .. + 31 by heads
+            // 32 hg .. + 31; lane = 32 half + n holds head n, register v column 8 (v / 4) + 4 half + v % 4 of the tile
+            f32x16_t O[CT][HG];
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
+            for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    O[dt][k] = 0.f;
+                for (int hg = 0; hg < HG; hg++) {
+#pragma unroll
+                    for (int k = 0; k < 16; k++) {
+                        O[ct][hg][k] = 0.f;
+                    }
                 }
             }
-            float m_run = -INFINITY, l_run = 0.f;
+            float m_run = -INFINITY, l_run = 0.f;   // of the lane's own head (the score side)
 
             // ---- cache copies of one step: scalars first, then four or five 1 KiB copies per wave ---------
             struct StepCopy {
@@ -267,7 +282,7 @@ mla_decode_kernel(const MlaDecodeParams p)
 #pragma unroll
                     for (uint32_t i = 0; i < 4; i++) {
                         const uint64_t phys = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row_of[i])));
-                        dma_1k(stage + (r0 + i) * KC_ROWB, kc_voff ^ (i << 5),
+                        dma_1k(stage + (r0 + i) * KC_ROWB, kc_voff ^ (i << 6),
                                reinterpret_cast<const char *>(p.k_cache) + phys * KC_ROWB);
                     }
                     if (wave < PE_WAVES) {
@@ -279,8 +294,8 @@ mla_decode_kernel(const MlaDecodeParams p)
                 }
                 const StepCopy c = plan(step);
                 if (c.last_pos == kStep - 1) {
-                    dma_4x1k(c.stage + r0 * KC_ROWB, kc_voff, kc_voff ^ (1u << 5), kc_voff ^ (2u << 5),
-                             kc_voff ^ (3u << 5), c.kb + r0 * KC_ROWB);
+                    dma_4x1k(c.stage + r0 * KC_ROWB, kc_voff, kc_voff ^ (1u << 6), kc_voff ^ (2u << 6),
+                             kc_voff ^ (3u << 6), c.kb + r0 * KC_ROWB);
                     if (wave < PE_WAVES) {
                         dma_1k(c.stage + KC_BYTES + wave * 1024, pe_row * PE_ROWB + pe_voff, c.pb);
                     }
@@ -288,7 +303,7 @@ mla_decode_kernel(const MlaDecodeParams p)
 #pragma unroll
                     for (uint32_t i = 0; i < 4; i++) {
                         const uint32_t src = min(r0 + i, c.last_pos);   // uniform
-                        dma_1k(c.stage + (r0 + i) * KC_ROWB, kc_voff ^ (i << 5), c.kb + src * KC_ROWB);
+                        dma_1k(c.stage + (r0 + i) * KC_ROWB, kc_voff ^ (i << 6), c.kb + src * KC_ROWB);
                     }
                     if (wave < PE_WAVES) {
                         const uint32_t prow = min(pe_row, c.last_pos);
@@ -333,35 +348,18 @@ mla_decode_kernel(const MlaDecodeParams p)
                 }
             };
 
-            // ---- online softmax of one step, then O^T += kc^T . P^T. Register k of score tile mt holds
-            // position t + 16 mt + 4 gi + k. The reference maximum only moves when the step maximum exceeds
-            // it by more than 2^8: probabilities then stay below 2^8 (the same relative precision in bf16, and
-            // the normaliser shares the reference), and the accumulators are rescaled rarely.
-            auto softmax_pv = [&](uint32_t step, f32x4_t (&S)[2]) {
+            // ---- online softmax of one step. Register k of score tile mt holds position t + 16 mt + 4 gi + k. The
+            // reference maximum only moves when the step maximum exceeds it by more than 2^8: probabilities then
+            // stay below 2^8 (the same relative precision in bf16, and the normaliser shares the reference), and the
+            // accumulators are rescaled rarely. The probabilities of the lane's head go to LDS, [head][position] in
+            // 16-bit, 16-byte chunk c of head h in slot c ^ ((h >> 2) & 3) (the reads of the second product, 32 heads
+            // a pass, then touch every bank once), and with them the factor by which the head's reference moved.
+            auto softmax = [&](uint32_t step, f32x4_t (&S)[2]) {
                 const uint32_t t = t0 + step * kStep;
-                const uint32_t soff = (step % kStages) * STAGE_BYTES;
                 const uint32_t lane_pos = t + gi4;
                 float mx = -INFINITY;
-                // the first transposed operands of the second product do not depend on the softmax: in flight during it
-                typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
-                uint32_t xv[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    xv[j] = soff + (vr_off ^ (j << 5));
-                }
-                auto rd_v = [&](int dt, int rd) {
-                    unsigned char *ptr = smem + xv[dt & 7] + ((dt >> 3) << 8) + rd * 16 * KC_ROWB;
-                    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)ptr));
-                };
-                uint2 v[VB][2];
-#pragma unroll
-                for (int d = 0; d < VB - 1; d++) {
-                    v[d][0] = rd_v(d, 0);
-                    v[d][1] = rd_v(d, 1);
-                }
-                __builtin_amdgcn_sched_barrier(0);
                 // the softmax runs at a raised wave priority: its vector instructions go ahead of the products of
-                // the SIMD's other wave (1-2 % on the step; raising it around the products instead gains nothing)
+                // the SIMD's other wave
                 __builtin_amdgcn_s_setprio(2);
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++) {
@@ -405,7 +403,8 @@ mla_decode_kernel(const MlaDecodeParams p)
                 }
                 const float m_new = mx > m_run + kRescaleSlack ? mx : m_run;
                 const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-                const float alpha = fast_exp2(m_run - m_safe);
+                // (nothing accumulated yet: no rescale)
+                const float alpha = m_run == -INFINITY ? 1.0f : fast_exp2(m_run - m_safe);
                 m_run = m_new;
                 uint32_t pw[4];
                 float psum = 0.f;
@@ -420,57 +419,106 @@ mla_decode_kernel(const MlaDecodeParams p)
                     }
                 }
                 l_run = l_run * alpha + psum;
+                // positions 16 mt + 4 gi .. + 3 of head 16 wave + col: chunk 2 mt + gi / 2, its half gi % 2
+                {
+                    uint32_t ln;
+                    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+                    const uint32_t h = wave * 16 + (ln & 15), g = ln >> 4;
+                    unsigned char *row = p_lds + (step & 1) * P_BYTES + h * P_ROWB + ((g & 1) << 3);
+                    const uint32_t f = (h >> 2) & 3;
+                    *reinterpret_cast<uint2 *>(row + (((g >> 1) ^ f) << 4)) = make_uint2(pw[0], pw[1]);
+                    *reinterpret_cast<uint2 *>(row + (((2 + (g >> 1)) ^ f) << 4)) = make_uint2(pw[2], pw[3]);
+                    if (g == 0) {
+                        f_lds[(step & 1) * kHeads + h] = alpha;
+                    }
+                }
+                __builtin_amdgcn_s_setprio(0);
+            };
 
-                if (__any(alpha != 1.0f)) {
-                    // all 256 registers of the wave are ordinary vector registers here (no accumulation
-                    // registers), so the rescale is a plain multiply
+            // ---- O^T += kc^T . P^T of step `step`, whose probabilities every wave left in LDS before the barrier
+            // this call follows: the wave's two 32-column tiles by four 32-head groups, two k-steps of 16 positions.
+            // Four transposed latent operands (two reads each) and eight probability operands per step.
+            auto pv = [&](uint32_t step) {
+                const uint32_t soff = (step % kStages) * STAGE_BYTES;
+                const unsigned char *pbuf = p_lds + (step & 1) * P_BYTES;
+                typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+                // the heads' rescale factors (rarely other than 1)
+                {
+                    float al[HG];
+                    bool any = false;
 #pragma unroll
-                    for (int dt = 0; dt < DT; dt++) {
+                    for (int hg = 0; hg < HGN; hg++) {
+                        al[hg] = f_lds[(step & 1) * kHeads + hg * 32 + (pr_off / P_ROWB)];
+                        any = any || al[hg] != 1.0f;
+                    }
+                    if (__any(any)) {
 #pragma unroll
-                        for (int k = 0; k < 4; k++) {
-                            O[dt][k] *= alpha;
+                        for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+                            for (int hg = 0; hg < HGN; hg++) {
+#pragma unroll
+                                for (int k = 0; k < 16; k++) {
+                                    O[ct][hg][k] *= al[hg];
+                                }
+                            }
                         }
                     }
                 }
-
-                // 32 tiles of 16 latent columns, one k-step of 32 positions in the order (16 mt + 4 gi + k),
-                // which is the order the lane's own probabilities already have
-                const uint4 pb = make_uint4(pw[0], pw[1], pw[2], pw[3]);
-                __builtin_amdgcn_s_setprio(0);
-                __builtin_amdgcn_sched_barrier(0);
+                auto rd_v = [&](int ks2, int ct) {
+                    const unsigned char *base = smem + soff + ks2 * 16 * KC_ROWB;
+                    const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + (vt0 ^ (ct << 6)))));
+                    const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + (vt1 ^ (ct << 6)))));
+                    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+                };
+                auto rd_p = [&](int ks2, int hg) {
+                    return *reinterpret_cast<const uint4 *>(pbuf + hg * 32 * P_ROWB + (pr_off ^ (ks2 << 5)));
+                };
+                // (operands of one k-step at a time: 24 registers; the SIMD's other wave covers their latency)
 #pragma unroll
-                for (int dt = 0; dt < DT; dt++) {
-                    if (dt + VB - 1 < DT) {
-                        v[(dt + VB - 1) % VB][0] = rd_v(dt + VB - 1, 0);
-                        v[(dt + VB - 1) % VB][1] = rd_v(dt + VB - 1, 1);
+                for (int ks2 = 0; ks2 < 2; ks2++) {
+                    uint4 va[CT], pb[HG];
+#pragma unroll
+                    for (int ct = 0; ct < CT; ct++) {
+                        va[ct] = rd_v(ks2, ct);
                     }
-                    const uint2 *x = v[dt % VB];
-                    O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8_t, make_uint4(x[0].x, x[0].y, x[1].x, x[1].y)),
-                        __builtin_bit_cast(bf16x8_t, pb), O[dt], 0, 0, 0);
+#pragma unroll
+                    for (int hg = 0; hg < HG; hg++) {
+                        pb[hg] = rd_p(ks2, hg);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+                        for (int hg = 0; hg < HG; hg++) {
+                            // (head groups beyond the model's heads hold nothing: HGN = 1 for models of at most 32 heads,
+                            // which run a quarter of the products)
+                            if (hg < HGN) {
+                                O[ct][hg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[ct]),
+                                                                                   __builtin_bit_cast(bf16x8_t, pb[hg]),
+                                                                                   O[ct][hg], 0, 0, 0);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
                 }
             };
 
-            // ---- pipeline: copies run kDepth steps ahead of the step being consumed. Every copy is
-            // unconditional (steps past the end copy the last step again, same bytes to the same place), so
-            // the wait counts are exact.
+            // ---- pipeline. Iteration `it` follows a barrier behind which step it's copies (issued one iteration
+            // earlier) have landed for everybody, every wave has left the probabilities of step it - 1 in LDS and
+            // nobody reads the stage of step it - 2 any more: it issues the copies of step it + 1 into that stage,
+            // forms the scores of step it, runs their softmax and then the second product of step it - 1. Every copy
+            // is unconditional (steps past the end copy the last step again, same bytes to the same place), so the
+            // wait counts are exact.
             const uint32_t last = n_steps - 1;
             __syncthreads();   // the previous pass has left the stages
             issue(0);
             // The query loads were issued before this copy and complete before it (memory operations finish in
             // order); their latency overlaps the copy's. They must have landed before the loop: a wait for them
             // inside it would also wait for the cache copies in flight. The wait the compiler places here counts
-            // the copies too (it does not know of them), so only the first step's are issued ahead of it: every
-            // workgroup of the launch starts at once, and with three steps of each in the burst the first products
-            // waited for all of it (27 MB across the chip) instead of a third.
+            // the copies too (it does not know of them).
 #pragma unroll
             for (int ks = 0; ks < KS_C + KS_R; ks++) {
                 asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
-            }
-#pragma unroll
-            for (int i = 1; i < kDepth; i++) {
-                issue(min(static_cast<uint32_t>(i), last));
             }
             f32x4_t S[2];
             for (uint32_t it = 0; it < n_steps; it++) {
@@ -481,52 +529,87 @@ mla_decode_kernel(const MlaDecodeParams p)
                     asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
                     set_roles(ln);
                 }
-                // this wave's share of step `it` has landed ...
-                if (wave < PE_WAVES) {
-                    dma_wait<(kDepth - 1) * 5>();
-                } else {
-                    dma_wait<(kDepth - 1) * 4>();
-                }
-                __syncthreads();            // ... and everybody else's; the stage issued into below is free
+                dma_wait<0>();              // this wave's share of step `it` has landed ...
+                __syncthreads();            // ... and everybody else's; see above
                 uint4 a[kAhead];
                 qk_fetch(it, a);
                 __builtin_amdgcn_sched_barrier(0);
-                issue(min(it + kDepth, last));
+                issue(min(it + 1, last));
                 qk(it, S, a);
-                softmax_pv(it, S);
+                softmax(it, S);
+                if (it > 0) {
+                    pv(it - 1);
+                }
             }
             dma_wait<0>();
-            __syncthreads();   // nothing in flight, nobody reading: the ring can be reused
+            __syncthreads();   // the last step's probabilities are in LDS
+            {
+                uint32_t ln;
+                asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+                set_roles(ln);
+            }
+            pv(last);
 
-            // ---- results: O^T lane layout is column = head, register k of tile dt = latent
-            // 16 dt + 4 gi + k. Normalised, rounded and transposed through a wave-private LDS region so that
-            // every store instruction writes one head's contiguous 1 KiB row.
+            // ---- results. The normaliser of a head lives with the wave that formed its scores: it goes through LDS
+            // to the eight waves that hold the head's columns.
+            // (lane roles from the hardware once more: nothing derived from threadIdx stays live across the loop,
+            // where its register would be spilled and reloaded every step)
+            uint32_t ln_e;
+            asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln_e));
+            const uint32_t col_e = ln_e & 15, gi_e = ln_e >> 4;
             float l_tot = l_run + __shfl_xor(l_run, 16);
             l_tot += __shfl_xor(l_tot, 32);
-            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-            unsigned char *my_tr = smem + wave * (16 * TR_ROWB);
-            const uint32_t heads_here = min(16u, p.n_heads > hw ? p.n_heads - hw : 0u);
-            const uint64_t rh0 = static_cast<uint64_t>(tok) * p.n_heads + hw;
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-                uint2 o;
-                o.x = BF16::pack(O[dt][0] * inv, O[dt][1] * inv);
-                o.y = BF16::pack(O[dt][2] * inv, O[dt][3] * inv);
-                *reinterpret_cast<uint2 *>(my_tr + col * TR_ROWB + dt * 32 + gi * 8) = o;
+            const float inv_own = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            const uint32_t head = h0 + wave * 16 + col_e;
+            const bool h_ok = head < p.n_heads;
+            if (gi_e == 0) {
+                f_lds[2 * kHeads + wave * 16 + col_e] = inv_own;
             }
-            // wave-private region: the LDS counter wait the compiler inserts is all the ordering needed
-            for (uint32_t hr = 0; hr < heads_here; hr++) {
-                const uint4 x = *reinterpret_cast<const uint4 *>(my_tr + hr * TR_ROWB + lane * 16);
-                uint16_t *dst = single ? p.out + (rh0 + hr) * C
-                                       : reinterpret_cast<uint16_t *>(p.part_acc) +
-                                             (static_cast<uint64_t>(pslot) * p.n_heads + hw + hr) * C;
-                *reinterpret_cast<uint4 *>(dst + lane * 8) = x;
-            }
-            if (h_ok && gi == 0 && !single) {
+            if (h_ok && gi_e == 0 && !single) {
                 *reinterpret_cast<float2 *>(p.part_ml + (static_cast<uint64_t>(pslot) * p.n_heads + head) * 2) =
                     make_float2(m_run, l_tot);
             }
-            if (step_a == 0 && h0 == 0 && threadIdx.x == 0) {
+            __syncthreads();   // normalisers visible; every wave is past its last product: the stages are free
+            // O^T lane layout: lane = 32 half + n holds head 32 hg + n, register v of tile (ct, hg) = column
+            // 64 wave + 32 ct + 8 (v / 4) + 4 half + v % 4. Normalised, rounded and transposed through a wave-private
+            // LDS region (64 heads x 64 columns at a time) so that a store instruction writes 128 contiguous bytes of
+            // each of eight heads' rows.
+            {
+                const uint32_t n = ln_e & 31, hf = ln_e >> 5;
+                unsigned char *my_tr = smem + wave * (64 * TR_ROWB);
+                uint16_t *dst_base = single ? p.out + static_cast<uint64_t>(tok) * p.n_heads * C
+                                            : reinterpret_cast<uint16_t *>(p.part_acc) + static_cast<uint64_t>(pslot) * p.n_heads * C;
+#pragma unroll
+                for (int half_pass = 0; half_pass < (HGN + 1) / 2; half_pass++) {
+#pragma unroll
+                    for (int hh = 0; hh < (HGN < 2 ? HGN : 2); hh++) {
+                        const int hg = 2 * half_pass + hh;
+                        const float inv = f_lds[2 * kHeads + hg * 32 + n];
+#pragma unroll
+                        for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+                            for (int g4 = 0; g4 < 4; g4++) {
+                                uint2 o;
+                                o.x = BF16::pack(O[ct][hg][4 * g4 + 0] * inv, O[ct][hg][4 * g4 + 1] * inv);
+                                o.y = BF16::pack(O[ct][hg][4 * g4 + 2] * inv, O[ct][hg][4 * g4 + 3] * inv);
+                                *reinterpret_cast<uint2 *>(my_tr + (hh * 32 + n) * TR_ROWB + (32 * ct + 8 * g4 + 4 * hf) * 2) = o;
+                            }
+                        }
+                    }
+                    // wave-private region: the LDS counter wait the compiler inserts is all the ordering needed.
+                    // Lane l stores 16 bytes: head 8 i + l / 8 of the 64, chunk l % 8 of its 128 bytes.
+#pragma unroll
+                    for (int i = 0; i < (HGN < 2 ? 4 : 8); i++) {
+                        const uint32_t hl = 8 * i + (ln_e >> 3);
+                        const uint32_t hd = h0 + 64 * half_pass + hl;
+                        const uint4 x = *reinterpret_cast<const uint4 *>(my_tr + hl * TR_ROWB + (ln_e & 7) * 16);
+                        if (hd < p.n_heads) {
+                            *reinterpret_cast<uint4 *>(dst_base + static_cast<uint64_t>(hd) * C + wave * WC + (ln_e & 7) * 8) = x;
+                        }
+                    }
+                }
+            }
+            if (step_a == 0 && h0 == 0 && wave == 0 && ln_e == 0) {
                 reinterpret_cast<int4 *>(p.part_meta)[tok] = meta;
             }
         }
@@ -867,17 +950,29 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
     p.top_k = a.top_k;
     XL_REQUIRE(a.top_k == 0 || a.topk_indices != nullptr, "top_k > 0 needs topk_indices");
 
-    const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + (kTblCap + kTblCap / kStep + 2) * sizeof(uint32_t);
+    const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + 2 * P_BYTES + 3 * F_BYTES +
+                       (kTblCap + kTblCap / kStep + 2) * sizeof(uint32_t);
     // the kernel also has a few words of static LDS: ask for exactly the dynamic part
     const bool lists = a.top_k != 0;
-    if (const int rc = ensure_dynamic_lds(lists ? reinterpret_cast<const void *>(mla_decode_kernel<true>)
-                                                : reinterpret_cast<const void *>(mla_decode_kernel<false>), lds)) {
+    const bool few = a.n_heads <= 32;
+    const void *kernel = lists ? (few ? reinterpret_cast<const void *>(mla_decode_kernel<true, 1>)
+                                      : reinterpret_cast<const void *>(mla_decode_kernel<true, 4>))
+                               : (few ? reinterpret_cast<const void *>(mla_decode_kernel<false, 1>)
+                                      : reinterpret_cast<const void *>(mla_decode_kernel<false, 4>));
+    if (const int rc = ensure_dynamic_lds(kernel, lds)) {
         return rc;
     }
+    const dim3 grid(pl.n_workgroups, 1, 1);
     if (lists) {
-        mla_decode_kernel<true><<<dim3(pl.n_workgroups, 1, 1), kNT, lds, stream>>>(p);
+        if (few) {
+            mla_decode_kernel<true, 1><<<grid, kNT, lds, stream>>>(p);
+        } else {
+            mla_decode_kernel<true, 4><<<grid, kNT, lds, stream>>>(p);
+        }
+    } else if (few) {
+        mla_decode_kernel<false, 1><<<grid, kNT, lds, stream>>>(p);
     } else {
-        mla_decode_kernel<false><<<dim3(pl.n_workgroups, 1, 1), kNT, lds, stream>>>(p);
+        mla_decode_kernel<false, 4><<<grid, kNT, lds, stream>>>(p);
     }
     XL_LAUNCH_CHECK();
     // rows that ended up in a single segment were stored directly
