@@ -156,8 +156,12 @@ def bench_gqa_decode(args, torch, rt, name, shape, ctx, seed, int8=False, with_r
 
     def step():
         if r is not None:
-            rope()
-        attn()
+            # the pair as one call into the library (same kernels as rope() then attn())
+            _C.decode_step(rt, r["inout"], w["k_cache"], w["v_cache"], w["output"], r["position"], r["cosin"],
+                           r["slot_mapping"], w["query_start_loc"], w["lens"], w["cached_lens"], w["block_tables"],
+                           s.n_heads, s.n_kv_heads, s.head_dim, s.head_dim, s.block_size, B, w["max_num_block"])
+        else:
+            attn()
 
     _spin_up(torch, step)
     if r is not None:

@@ -95,6 +95,7 @@ class Runtime:
         self.aiv_num = self.num_cu
         self._pool: Optional[torch.Tensor] = None
         self._retired: List[torch.Tensor] = []
+        self._step_plans: dict = {}   # decode_step: argument combinations already checked
         self.init_tensor_pool(size)
 
     # -- reference API ---------------------------------------------------------------------
@@ -258,6 +259,57 @@ def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
         rt.stream(), _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(output), _ptr(query_start_loc), _ptr(lens),
         _ptr(cached_lens), _ptr(block_tables), T, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
         dt, kv, _ptr(k_scale), _ptr(v_scale), _ptr(ws), ws.numel()))
+    rt.finish()
+
+
+def decode_step(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, output: torch.Tensor,
+                position: torch.Tensor, cosin: torch.Tensor, slot_mapping: torch.Tensor,
+                query_start_loc: torch.Tensor, lens: torch.Tensor, cached_lens: torch.Tensor,
+                block_tables: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, rot_dim: int,
+                block_size: int, batch: int, max_num_block: int, is_neox: bool = True, mrope_mask_h: int = 0,
+                mrope_mask_w: int = 0) -> None:
+    """`rope_and_cache` followed by `attention` over the same rows and caches, as a layer of the reference's model
+    loop runs them (xlite/csrc/model.cpp:544-571), through one call into the library. The argument checks of the
+    two run once per combination of shapes, dtypes and devices: a serving loop repeats the same combination step
+    after step, and for a small batch the checks cost more than the kernels. 16-bit caches."""
+    tensors = (qkv, k_cache, v_cache, output, position, cosin, slot_mapping, query_start_loc, lens, cached_lens,
+               block_tables)
+    key = (tuple((t.shape, t.dtype, t.device, t.is_contiguous()) for t in tensors), n_heads, n_kv_heads, head_dim,
+           rot_dim, block_size, batch, max_num_block, is_neox, mrope_mask_h, mrope_mask_w)
+    plan = rt._step_plans.get(key)
+    if plan is None:
+        if not is_neox:
+            raise RuntimeError("rope_and_cache: unsupported rope type gptj")
+        for n, t in (("qkv", qkv), ("k_cache", k_cache), ("v_cache", v_cache), ("output", output), ("cosin", cosin)):
+            _dev(n, t)
+        _dev("position", position, torch.int64)
+        for n, t in (("slot_mapping", slot_mapping), ("query_start_loc", query_start_loc), ("lens", lens),
+                     ("cached_lens", cached_lens), ("block_tables", block_tables)):
+            _dev(n, t, torch.int32)
+        dt = _act_dtype("decode_step", qkv, k_cache, v_cache, cosin, output)
+        T = qkv.shape[0]
+        _req(n_kv_heads > 0 and n_heads % n_kv_heads == 0, "decode_step: n_heads must be a multiple of n_kv_heads")
+        _req(qkv.numel() == T * (n_heads + 2 * n_kv_heads) * head_dim, "decode_step: qkv shape mismatch")
+        _req(output.numel() == T * n_heads * head_dim, "decode_step: output shape mismatch")
+        _req(k_cache.shape == v_cache.shape, "decode_step: cache shapes differ")
+        _req(k_cache.numel() % (block_size * n_kv_heads * head_dim) == 0, "decode_step: cache shape mismatch")
+        mrope = bool(mrope_mask_h or mrope_mask_w)
+        _req(position.numel() == (3 * T if mrope else T), "decode_step: position shape mismatch")
+        _req(slot_mapping.numel() >= T, "decode_step: slot_mapping too short")
+        _req(cosin.shape[-1] == rot_dim, "decode_step: cosin row must hold rot_dim values")
+        _req(min(query_start_loc.numel(), lens.numel(), cached_lens.numel()) >= batch,
+             "decode_step: metadata shorter than batch")
+        _req(block_tables.numel() >= batch * max_num_block, "decode_step: block_tables shorter than batch * max_num_block")
+        need = rt._lib.xlite_hip_attention_workspace_bytes(T, n_heads, n_kv_heads, head_dim, block_size, batch,
+                                                           max_num_block)
+        plan = rt._step_plans[key] = (T, dt, need)
+    T, dt, need = plan
+    ws = rt.workspace(need)
+    _lib.check(rt._lib.xlite_hip_decode_step(
+        rt.stream(), qkv.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), position.data_ptr(),
+        cosin.data_ptr(), slot_mapping.data_ptr(), query_start_loc.data_ptr(), lens.data_ptr(), cached_lens.data_ptr(),
+        block_tables.data_ptr(), T, n_heads, n_kv_heads, head_dim, rot_dim, block_size, batch, max_num_block, 1,
+        mrope_mask_h, mrope_mask_w, dt, ws.data_ptr(), ws.numel()))
     rt.finish()
 
 

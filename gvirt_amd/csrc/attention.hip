@@ -210,6 +210,26 @@ static int run_16bit(hipStream_t s, AttentionArgs &a)
     return launch_mfma_gqa(s, a);
 }
 
+extern "C" int xlite_hip_decode_step(void *stream, void *qkv, void *k_cache, void *v_cache, void *output,
+                                     const int64_t *position, const void *cosin, const int32_t *slot_mapping,
+                                     const int32_t *query_start_loc, const int32_t *lens,
+                                     const int32_t *cached_lens, const int32_t *block_tables,
+                                     uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                                     uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, uint32_t batch,
+                                     uint32_t max_num_block, int is_neox, uint64_t mrope_mask_h,
+                                     uint64_t mrope_mask_w, int dtype, void *workspace, size_t workspace_bytes)
+{
+    // the two calls of a layer's attention block, enqueued back to back on the caller's stream
+    if (const int rc = xlite_hip_rope_and_cache(stream, qkv, k_cache, v_cache, position, cosin, slot_mapping, total_tokens,
+                                                n_heads, n_kv_heads, head_dim, rot_dim, block_size, is_neox, mrope_mask_h,
+                                                mrope_mask_w, dtype)) {
+        return rc;
+    }
+    return xlite_hip_attention(stream, qkv, k_cache, v_cache, output, query_start_loc, lens, cached_lens, block_tables,
+                               total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block, dtype,
+                               XLITE_HIP_KV_SAME, nullptr, nullptr, workspace, workspace_bytes);
+}
+
 extern "C" size_t xlite_hip_mla_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
                                                 uint32_t kv_lora_rank, uint32_t rope_head_dim,
                                                 uint32_t block_size, uint32_t batch,

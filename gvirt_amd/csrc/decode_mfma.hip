@@ -260,8 +260,22 @@ struct DecodeSplit {
             *limit = static_cast<uint32_t>(lim > 1 ? lim : 1);
             return ceil_div(*limit, static_cast<uint32_t>(kStep));
         }
-        const uint32_t s = seq_of_row(u);
-        const int32_t lim = p.cached_lens[s] + (static_cast<int32_t>(u) - p.query_start_loc[s]) + 1;
+        // A decode batch (one row per sequence) answers at once, and its cached length is requested together with
+        // the two loads that say so: one trip to memory instead of two.
+        int32_t lim;
+        uint32_t s = u;
+        if (u < p.batch) {
+            const int32_t start = p.query_start_loc[u], ql = p.lens[u], cached = p.cached_lens[u];
+            if (start == static_cast<int32_t>(u) && ql == 1) {
+                lim = cached + 1;
+            } else {
+                s = seq_of_row(u);
+                lim = p.cached_lens[s] + (static_cast<int32_t>(u) - p.query_start_loc[s]) + 1;
+            }
+        } else {
+            s = seq_of_row(u);
+            lim = p.cached_lens[s] + (static_cast<int32_t>(u) - p.query_start_loc[s]) + 1;
+        }
         *limit = static_cast<uint32_t>(lim > 1 ? lim : 1);
         *seq = s;
         *tok = u;
@@ -492,6 +506,19 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         const uint32_t ta = min(t1, t0 + my_sub * sub_len);   // this wave's range
         const uint32_t tb = min(t1, ta + sub_len);
         const uint32_t blk0 = t0 / p.block_size;
+        // ---- Q^T as the B operand: column = head, 8 consecutive elements per k group. The first pass's rows are
+        // requested ahead of the block-table entries: one trip to memory for the two.
+        uint4 qreg[KS];
+        auto request_q = [&](uint32_t kv0) {
+            const uint32_t kvh = kv0 + my_kvl;
+            const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride + static_cast<uint64_t>(kvh * p.group + col) * D;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                qreg[ks] = (kvh < p.n_kv_heads && col < g_valid) ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8)
+                                                                 : make_uint4(0, 0, 0, 0);
+            }
+        };
+        request_q(0);
         {
             const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
             for (uint32_t i = threadIdx.x; i < nblk; i += NT) {
@@ -509,14 +536,12 @@ decode_mfma_kernel(const DecodeMfmaParams p)
             const bool kv_ok = kvh < p.n_kv_heads;
             const uint32_t head0 = kvh * p.group;
 
-            // ---- Q^T as the B operand: column = head, 8 consecutive elements per k group ----------
-            uint4 qreg[KS];
             {
-                const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride + static_cast<uint64_t>(head0 + col) * D;
+                if (kv0 != 0) {
+                    request_q(kv0);
+                }
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    qreg[ks] = (kv_ok && col < g_valid) ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8)
-                                                        : make_uint4(0, 0, 0, 0);
                     if constexpr (KV8 && !std::is_same<T, TM>::value) {   // bf16 activations: q as fp16
                         uint32_t *w = reinterpret_cast<uint32_t *>(&qreg[ks]);
 #pragma unroll

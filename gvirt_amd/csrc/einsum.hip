@@ -98,10 +98,11 @@ constexpr int kSlabCols = 64;                 // output columns of a workgroup
 constexpr int kSlabPitch = kSlabCols * 2 + 32;   // LDS bytes of a weight row: 128 + 32 keeps the transposing reads off each other's banks
 constexpr int kSlabRowsMax = 64;              // weight rows (k) a wave holds at a time
 
-// ONCE: one row tile (m <= 32), so every weight byte is used once in the launch and is fetched with the non-temporal
-// hint (the W_UV projection of a 32-token decode batch: 12.1 -> 7.4 us; with several row tiles the tiles share the
-// weight lines through L2 and the loads stay plain).
-template <typename T, bool ONCE>
+// A workgroup covers RT row tiles of 32 rows (1 or 2), so that a decode batch of up to 64 rows reads every weight byte
+// once. ONCE: the workgroup's rows are all there are (m <= 32 RT), so every weight byte is used once in the launch and
+// is fetched with the non-temporal hint (the W_UV projection of a 32-token decode batch: 12.1 -> 7.4 us; with several
+// workgroups per weight slab they share the weight lines through L2 and the loads stay plain).
+template <typename T, bool ONCE, int RT>
 __global__ void __launch_bounds__(256)
 einsum_htd_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__ w, uint16_t *__restrict__ mhd,
                   uint32_t m, uint32_t h, uint32_t t, uint32_t d, uint32_t t_stride)
@@ -110,11 +111,16 @@ einsum_htd_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t col = lane & 31, half = lane >> 5;
     const uint32_t head = blockIdx.z;
-    const uint32_t m0 = blockIdx.y * 32;
+    const uint32_t m0 = blockIdx.y * (32 * RT);
     const uint32_t n0 = blockIdx.x * kSlabCols;
-    const uint32_t row = m0 + col;
-    const bool row_ok = row < m;
-    const uint16_t *a_ptr = mht + (static_cast<uint64_t>(row_ok ? row : 0) * h + head) * t_stride;
+    bool row_ok[RT];
+    const uint16_t *a_ptr[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        const uint32_t row = m0 + 32 * rt + col;
+        row_ok[rt] = row < m;
+        a_ptr[rt] = mht + (static_cast<uint64_t>(row_ok[rt] ? row : 0) * h + head) * t_stride;
+    }
     const uint16_t *w_head = w + static_cast<uint64_t>(head) * t * d + n0;
     unsigned char *mine = slab + wave * (kSlabRowsMax * kSlabPitch);
 
@@ -122,12 +128,15 @@ einsum_htd_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__
     const uint32_t steps = t / 16, per = ceil_div(steps, 4u);
     const uint32_t k_lo = min(steps, wave * per) * 16, k_hi = min(steps, (wave + 1) * per) * 16;
 
-    f32x16_t acc[2];
+    f32x16_t acc[RT][2];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int rt = 0; rt < RT; rt++) {
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
-            acc[j][k] = 0.f;
+        for (int j = 0; j < 2; j++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                acc[rt][j][k] = 0.f;
+            }
         }
     }
     // transposing read role: the 16-lane group g serves columns 16 (g % 2) .. + 15 of a 32-column tile and the
@@ -162,35 +171,43 @@ einsum_htd_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__
         // wave-private region: the LDS counter wait the compiler inserts between the writes and the reads is all
         // the ordering needed
         for (uint32_t k0 = 0; k0 < rows; k0 += 16) {
-            uint4 a = make_uint4(0, 0, 0, 0);
-            if (row_ok) {
-                a = *reinterpret_cast<const uint4 *>(a_ptr + kb + k0 + half * 8);
+            uint4 a[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                a[rt] = make_uint4(0, 0, 0, 0);
+                if (row_ok[rt]) {
+                    a[rt] = *reinterpret_cast<const uint4 *>(a_ptr[rt] + kb + k0 + half * 8);
+                }
             }
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 unsigned char *src = mine + k0 * kSlabPitch + tr_off + j * 64;
                 const uint2 b0 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)src));
                 const uint2 b1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(src + 4 * kSlabPitch)));
-                acc[j] = Mma<T>::run(a, make_uint4(b0.x, b0.y, b1.x, b1.y), acc[j]);
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++) {
+                    acc[rt][j] = Mma<T>::run(a[rt], make_uint4(b0.x, b0.y, b1.x, b1.y), acc[rt][j]);
+                }
             }
         }
     }
-    // the four partial tiles meet in LDS (the slabs are done with): [wave][32 rows][64 columns] fp32
-    __syncthreads();
+    // the four partial tiles meet in LDS (the slabs are done with), one row tile at a time: [wave][32 rows][64 columns] fp32
     float *part = reinterpret_cast<float *>(slab);
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int rt = 0; rt < RT; rt++) {
+        __syncthreads();
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
-            const uint32_t r = (k / 4) * 8 + half * 4 + (k % 4);
-            part[(wave * 32 + r) * kSlabCols + j * 32 + col] = acc[j][k];
+        for (int j = 0; j < 2; j++) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                const uint32_t r = (k / 4) * 8 + half * 4 + (k % 4);
+                part[(wave * 32 + r) * kSlabCols + j * 32 + col] = acc[rt][j][k];
+            }
         }
-    }
-    __syncthreads();
-    // thread = (row, 8 columns): sums the four partials and stores 16 bytes
-    {
+        __syncthreads();
+        // thread = (row, 8 columns): sums the four partials and stores 16 bytes
         const uint32_t r = threadIdx.x >> 3, c8 = (threadIdx.x & 7) * 8;
-        if (m0 + r < m) {
+        if (m0 + 32 * rt + r < m) {
             float sum[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -208,7 +225,7 @@ einsum_htd_kernel(const uint16_t *__restrict__ mht, const uint16_t *__restrict__
             o.y = T::pack(sum[2], sum[3]);
             o.z = T::pack(sum[4], sum[5]);
             o.w = T::pack(sum[6], sum[7]);
-            *reinterpret_cast<uint4 *>(mhd + (static_cast<uint64_t>(m0 + r) * h + head) * d + n0 + c8) = o;
+            *reinterpret_cast<uint4 *>(mhd + (static_cast<uint64_t>(m0 + 32 * rt + r) * h + head) * d + n0 + c8) = o;
         }
     }
 }
@@ -241,20 +258,26 @@ extern "C" int xlite_hip_einsum_mht_mhd(void *stream, const void *mht, const voi
     uint16_t *c = static_cast<uint16_t *>(mhd);
     if (!w_is_hdt && d % kSlabCols == 0) {
         // [h,t,d] weights: the LDS-transposing kernel
-        dim3 g2(d / kSlabCols, ceil_div(m, 32), h);
-        const bool once = m <= 32;
+        // (more than 32 rows: two row tiles per workgroup, so a decode batch of up to 64 rows streams the weights once)
+        const uint32_t rt = m > 32 ? 2 : 1;
+        dim3 g2(d / kSlabCols, ceil_div(m, 32 * rt), h);
+        const bool once = m <= 32 * rt;
+        auto launch = [&](auto tag) {
+            using T = decltype(tag);
+            if (rt == 2) {
+                if (once) {
+                    einsum_htd_kernel<T, true, 2><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
+                } else {
+                    einsum_htd_kernel<T, false, 2><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
+                }
+            } else {
+                einsum_htd_kernel<T, true, 1><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
+            }
+        };
         if (dtype == XLITE_HIP_BF16) {
-            if (once) {
-                einsum_htd_kernel<BF16, true><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
-            } else {
-                einsum_htd_kernel<BF16, false><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
-            }
+            launch(BF16{});
         } else {
-            if (once) {
-                einsum_htd_kernel<FP16, true><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
-            } else {
-                einsum_htd_kernel<FP16, false><<<g2, 256, 0, s>>>(a, b, c, m, h, t, d, t_stride);
-            }
+            launch(FP16{});
         }
         XL_LAUNCH_CHECK();
         return XLITE_HIP_OK;

@@ -112,6 +112,24 @@ int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, cons
                         const float *v_scale, void *workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------------------------------
+ * decode_step — the attention block of one layer as the reference's model loop runs it
+ * (xlite/csrc/model.cpp:544-571: XliteOpRopeCache, then XliteOpAttention or
+ * XliteOpFlashAttention over the same qkv rows and caches), enqueued from one call:
+ * xlite_hip_rope_and_cache followed by xlite_hip_attention with the arguments of the
+ * two (16-bit caches), same results bit for bit. For serving loops whose small batches
+ * are bound by the cost of a call, not of the kernels. Any batch the two accept, not
+ * only decode rows.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_decode_step(void *stream, void *qkv, void *k_cache, void *v_cache, void *output,
+                          const int64_t *position, const void *cosin, const int32_t *slot_mapping,
+                          const int32_t *query_start_loc, const int32_t *lens,
+                          const int32_t *cached_lens, const int32_t *block_tables,
+                          uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                          uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, uint32_t batch,
+                          uint32_t max_num_block, int is_neox, uint64_t mrope_mask_h,
+                          uint64_t mrope_mask_w, int dtype, void *workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
  * mla_attention — replaces XliteOpMLAV2 / XliteOpFlashMLAV2
  * (xlite/csrc/op.cpp:995-1058) + kernels mla_v2.h / flash_mla_v2.h: the absorbed
  * MLA attention between the two einsums of the mla_v2 operator.
