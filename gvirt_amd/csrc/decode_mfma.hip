@@ -510,12 +510,15 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         // requested ahead of the block-table entries: one trip to memory for the two.
         uint4 qreg[KS];
         auto request_q = [&](uint32_t kv0) {
-            const uint32_t kvh = kv0 + my_kvl;
-            const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride + static_cast<uint64_t>(kvh * p.group + col) * D;
+            // Every lane loads: columns past the group's heads (and waves past the last kv head) repeat the last valid
+            // head, and their results are never stored. (A load under a per-lane condition is compiled into a branch
+            // with a wait of its own: one trip to memory per load instead of one for all.)
+            const uint32_t kvh = min(kv0 + my_kvl, p.n_kv_heads - 1);
+            const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
+                                   static_cast<uint64_t>(kvh * p.group + min(col, g_valid - 1)) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
-                qreg[ks] = (kvh < p.n_kv_heads && col < g_valid) ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8)
-                                                                 : make_uint4(0, 0, 0, 0);
+                qreg[ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8);
             }
         };
         request_q(0);
@@ -953,11 +956,13 @@ decode_dma_kernel(const DecodeMfmaParams p)
         // the query rows of the first pass travel together with the block-table entries
         uint4 qreg[KS];
         auto load_q = [&](uint32_t kv0) {
+            // (every lane loads: columns past the group's heads repeat its last head and are never stored; a load under
+            // a per-lane condition is compiled into a branch with a wait of its own, one trip to memory per load)
             const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
-                                   static_cast<uint64_t>((kv0 + kvl) * p.group + col) * D;
+                                   static_cast<uint64_t>((kv0 + kvl) * p.group + min(col, g_valid - 1)) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
-                qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8) : make_uint4(0, 0, 0, 0);
+                qreg[ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8);
             }
         };
         load_q(0);
@@ -1332,12 +1337,12 @@ decode_dma8_kernel(const DecodeMfmaParams p)
         // [16 (j + 4r) + 8h, + 8) of the head
         uint4 qreg[4];
         auto load_q = [&](uint32_t kv0) {
+            // (every lane loads: columns past the group's heads repeat its last head and are never stored)
             const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
-                                   static_cast<uint64_t>((kv0 + kvl) * p.group + col) * D;
+                                   static_cast<uint64_t>((kv0 + kvl) * p.group + min(col, g_valid - 1)) * D;
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                qreg[ks] = col < g_valid ? *reinterpret_cast<const uint4 *>(qrow + 16 * (jq + 4 * (ks >> 1)) + 8 * (ks & 1))
-                                         : make_uint4(0, 0, 0, 0);
+                qreg[ks] = *reinterpret_cast<const uint4 *>(qrow + 16 * (jq + 4 * (ks >> 1)) + 8 * (ks & 1));
             }
         };
         auto q_to_fp16 = [&]() {

@@ -265,27 +265,7 @@ prefill_kernel(const PrefillParams p)
     // tiles wholly below every row's limit need no mask; first tile that does (uniform per wave)
     const uint32_t wave_min_vis = static_cast<uint32_t>(clen) + min(m_first + wave * 32, m_rows - 1) / G + 1;
 
-    uint4 qreg[KS];
-    {
-        const uint16_t *src = p.q + static_cast<uint64_t>(tok) * p.q_tok_stride + static_cast<uint64_t>(head) * D;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            qreg[ks] = m_valid ? convert8<TIO, T>(*reinterpret_cast<const uint4 *>(src + ks * 16 + half * 8)) : make_uint4(0, 0, 0, 0);
-        }
-        // the block-table entries of this workgroup's range go to LDS while the query loads are in flight
-        for (uint32_t i = __umulhi(first_tile * BN, p.block_magic) + threadIdx.x;
-             i <= __umulhi(min(n_tiles * BN, range_end) - 1, p.block_magic); i += kThreads) {
-            tbl_lds[i] = static_cast<uint32_t>(table[i]);
-        }
-        __syncthreads();
-        // complete these loads before any copy is issued: memory operations finish in order, and their
-        // first use is inside the streaming loop
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
-        }
-    }
-
+    uint4 qreg[KS];   // the lane's query row as the B operand of the first product; loaded by the set-up below
     f32x16_t O[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; dt++) {
@@ -498,9 +478,38 @@ prefill_kernel(const PrefillParams p)
     // fetches the next tile's first K operands. Every copy is unconditional (tiles past the end copy the last
     // tile again into a stage nobody reads any more), so the wait counts are exact.
     const uint32_t last = n_tiles - 1;
+    // Set-up in two trips to memory: the block-table entries of this workgroup's range are requested first and the
+    // query rows right behind them; the entries go to LDS as soon as they are there (the wait leaves the query
+    // loads in flight), the first three tiles' copies are issued, and only then are the query rows awaited
+    // (memory operations finish in order: that wait covers the copies too, which were going to be awaited anyway).
+    {
+        const uint32_t i_lo = __umulhi(first_tile * BN, p.block_magic);
+        const uint32_t i_hi = __umulhi(min(n_tiles * BN, range_end) - 1, p.block_magic);
+        const uint32_t i_mine = i_lo + threadIdx.x;
+        const uint32_t entry = i_mine <= i_hi ? static_cast<uint32_t>(table[i_mine]) : 0u;
+        const uint16_t *src = p.q + static_cast<uint64_t>(tok) * p.q_tok_stride + static_cast<uint64_t>(head) * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            // (every lane loads: rows past the tile's end point at the sequence's first row and are cleared below; a
+            // load under a condition is compiled into a branch with a wait of its own, eight trips to memory in a row)
+            qreg[ks] = *reinterpret_cast<const uint4 *>(src + ks * 16 + half * 8);
+        }
+        if (i_mine <= i_hi) {
+            tbl_lds[i_mine] = entry;
+        }
+        for (uint32_t i = i_mine + kThreads; i <= i_hi; i += kThreads) {   // (ranges of more than 512 blocks)
+            tbl_lds[i] = static_cast<uint32_t>(table[i]);
+        }
+        __syncthreads();
+    }
     issue(first_tile);
     issue(min(first_tile + 1, last));
     issue(min(first_tile + 2, last));
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+        qreg[ks] = m_valid ? convert8<TIO, T>(qreg[ks]) : make_uint4(0, 0, 0, 0);
+    }
     dma_wait<2 * PER_WAVE>();
     __syncthreads();
     fetch_k((first_tile % kStages) * STAGE, 0);
