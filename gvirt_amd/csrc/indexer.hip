@@ -69,6 +69,15 @@ struct Mma<FP16> {
 __device__ __forceinline__ bool find_row(uint32_t t, const int32_t *query_start_loc, const int32_t *lens,
                                          const int32_t *cached_lens, uint32_t batch, uint32_t *seq, uint32_t *total)
 {
+    if (t < batch) {
+        // a decode batch (one row per sequence) answers with one round of loads: row t is sequence t
+        const int32_t s = query_start_loc[t], l = lens[t], c = cached_lens[t];
+        if (s == static_cast<int32_t>(t) && l == 1) {
+            *seq = t;
+            *total = static_cast<uint32_t>(c + 1);
+            return true;
+        }
+    }
     uint32_t lo = 0, hi = batch;   // first index in [lo, hi) whose start is beyond t
     while (lo < hi) {
         const uint32_t mid = (lo + hi) / 2;
@@ -93,8 +102,8 @@ __device__ __forceinline__ bool find_row(uint32_t t, const int32_t *query_start_
 
 // Scores of query row t (of sequence `seq`, `total` candidate positions) for the positions [p0, p1), by one wave,
 // K rows straight from the cache. NT = n_heads / 16, head_dim = 128.
-template <typename T, int NT>
-__device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
+template <typename T, int NT, bool TBL_IN_REG>
+__device__ __forceinline__ void indexer_row_range_impl(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
                                                   const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
                                                   const int32_t *__restrict__ block_tables, uint32_t t, uint32_t seq,
                                                   uint32_t total, uint32_t p0, uint32_t p1, uint32_t block_size,
@@ -104,6 +113,16 @@ __device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q
     constexpr int KS = D / 32;
     constexpr int H = NT * 16;
     const uint32_t col = lane & 15, kg = lane >> 4;
+
+    // the block-table entries of the range sit in the lanes of one register (lane i: block p0 / bs + i), so that
+    // a K load does not wait for a table load first; ranges of more than 64 blocks look the table up directly.
+    // Requested ahead of the query rows: the first K loads wait for these entries only, and travel with the queries.
+    const int32_t *table = block_tables + static_cast<uint64_t>(seq) * max_num_block;
+    const uint32_t blk0 = p0 / block_size;
+    const uint32_t nblk = (p1 - 1) / block_size - blk0 + 1;
+    // (TBL_IN_REG is a template parameter, not a run-time choice inside load_k: a load that may or may not be issued
+    // is awaited at the join, and that wait covers every K load in flight)
+    const int32_t tbl_reg = table[blk0 + min(lane, nblk - 1)];   // (every lane loads: no branch, no wait of its own)
 
     // A operands: Q of head 16 nt + col, dims 32 ks + 8 kg .. +8; weights of heads 16 nt + 4 kg .. +4 in the
     // lanes of row 0 only
@@ -117,26 +136,18 @@ __device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q
         for (int ks = 0; ks < KS; ks++) {
             qa[nt][ks] = *reinterpret_cast<const uint4 *>(qrow + (16 * nt + col) * D + 32 * ks + 8 * kg);
         }
-        uint2 w = make_uint2(0u, 0u);
-        if (col == 0) {
-            const uint16_t *wp = wrow + 16 * nt + 4 * kg;   // 2-byte aligned only: the row pitch may be odd pairs
-            w.x = static_cast<uint32_t>(wp[0]) | (static_cast<uint32_t>(wp[1]) << 16);
-            w.y = static_cast<uint32_t>(wp[2]) | (static_cast<uint32_t>(wp[3]) << 16);
-        }
-        wa[nt] = w;
+        // (every row of the operand carries the weights: only row 0 of the product is read, and a load under a
+        // per-lane condition is compiled into a branch with a wait of its own, which here would also wait for every
+        // query load before it)
+        const uint16_t *wp = wrow + 16 * nt + 4 * kg;   // 2-byte aligned only: the row pitch may be odd pairs
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2], w3 = wp[3];
+        wa[nt] = make_uint2(w0 | (w1 << 16), w2 | (w3 << 16));
     }
 
-    // the block-table entries of the range sit in the lanes of one register (lane i: block p0 / bs + i), so that
-    // a K load does not wait for a table load first; ranges of more than 64 blocks look the table up directly
-    const int32_t *table = block_tables + static_cast<uint64_t>(seq) * max_num_block;
-    const uint32_t blk0 = p0 / block_size;
-    const uint32_t nblk = (p1 - 1) / block_size - blk0 + 1;
-    const bool tbl_in_reg = nblk <= 64;
-    const int32_t tbl_reg = tbl_in_reg && lane < nblk ? table[blk0 + lane] : 0;
     auto load_k = [&](uint32_t pos0, uint4 (&kb)[KS]) {
         const uint32_t pos = min(pos0 + col, total - 1);   // positions past the end repeat the last one
         const uint32_t blk = pos / block_size;
-        const uint32_t phys = static_cast<uint32_t>(tbl_in_reg ? __shfl(tbl_reg, static_cast<int>(min(blk - blk0, 63u)))
+        const uint32_t phys = static_cast<uint32_t>(TBL_IN_REG ? __shfl(tbl_reg, static_cast<int>(min(blk - blk0, 63u)))
                                                                : table[blk]);
         const uint16_t *row = k_cache + (static_cast<uint64_t>(phys) * block_size + pos % block_size) * D + 8 * kg;
 #pragma unroll
@@ -144,16 +155,19 @@ __device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q
             kb[ks] = *reinterpret_cast<const uint4 *>(row + 32 * ks);
         }
     };
-    constexpr int kPre = 3;   // K tiles in registers: two are in flight while one is consumed
+    constexpr int kPre = 5;   // K tiles in registers: four are in flight while one is consumed (16 KiB per wave: with
+                              // four waves on a compute unit, what its share of the memory system's latency needs)
     uint4 kb[kPre][KS];
-    load_k(p0, kb[0]);
-    if (p0 + 16 < p1) {
-        load_k(p0 + 16, kb[1]);
+#pragma unroll
+    for (int i = 0; i < kPre - 1; i++) {
+        if (p0 + 16 * i < p1) {
+            load_k(p0 + 16 * i, kb[i]);
+        }
     }
     uint16_t *out = scores + static_cast<uint64_t>(t) * ld_scores;
     auto tile = [&](uint32_t pos0, const uint4 (&kt)[KS], uint4 (&knext)[KS]) {
-        if (pos0 + 32 < p1) {
-            load_k(pos0 + 32, knext);
+        if (pos0 + 16 * (kPre - 1) < p1) {
+            load_k(pos0 + 16 * (kPre - 1), knext);
         }
         f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -172,15 +186,30 @@ __device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q
             out[pos0 + col] = T::from_f32(acc[0]);
         }
     };
-    // the ring of three register tiles, unrolled so that every index is a constant
-    for (uint32_t pos0 = p0; pos0 < p1; pos0 += 48) {
-        tile(pos0, kb[0], kb[2]);
-        if (pos0 + 16 < p1) {
-            tile(pos0 + 16, kb[1], kb[0]);
+    // the ring of register tiles, unrolled so that every index is a constant
+    for (uint32_t pos0 = p0; pos0 < p1; pos0 += 16 * kPre) {
+#pragma unroll
+        for (int i = 0; i < kPre; i++) {
+            if (pos0 + 16 * i < p1) {
+                tile(pos0 + 16 * i, kb[i], kb[(i + kPre - 1) % kPre]);
+            }
         }
-        if (pos0 + 32 < p1) {
-            tile(pos0 + 32, kb[2], kb[1]);
-        }
+    }
+}
+
+template <typename T, int NT>
+__device__ __forceinline__ void indexer_row_range(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache,
+                                                  const uint16_t *__restrict__ weight, uint16_t *__restrict__ scores,
+                                                  const int32_t *__restrict__ block_tables, uint32_t t, uint32_t seq,
+                                                  uint32_t total, uint32_t p0, uint32_t p1, uint32_t block_size,
+                                                  uint32_t max_num_block, uint32_t ld_scores, uint32_t lane)
+{
+    if ((p1 - 1) / block_size - p0 / block_size + 1 <= 64) {   // the same in every lane
+        indexer_row_range_impl<T, NT, true>(q, k_cache, weight, scores, block_tables, t, seq, total, p0, p1, block_size,
+                                            max_num_block, ld_scores, lane);
+    } else {
+        indexer_row_range_impl<T, NT, false>(q, k_cache, weight, scores, block_tables, t, seq, total, p0, p1, block_size,
+                                             max_num_block, ld_scores, lane);
     }
 }
 
