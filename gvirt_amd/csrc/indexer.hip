@@ -436,6 +436,11 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
                       uint32_t batch, uint32_t top_k, uint32_t ld_scores)
 {
     __shared__ uint32_t hist[256];
+    // 32 private copies of the histogram, copy c of bin b at [b][c]: a wave's lanes count into the copies of their
+    // lane index modulo 32, which lie in 32 different banks. (Scores of one row share their sign and most of their
+    // exponent: counted into one histogram, the high bytes of a wave's 64 keys fall into a handful of bins, and
+    // atomic additions to one address are carried out one lane at a time.)
+    __shared__ __attribute__((aligned(16))) uint32_t hist_priv[256 * 32];
     __shared__ uint32_t wave_cnt[2][kSelThreads / 64];
     __shared__ __attribute__((aligned(16))) uint16_t staged[kSelStage];
     __shared__ uint32_t sel[4];
@@ -461,15 +466,17 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
     // (the first pass's barrier orders these stores before any read)
     uint32_t prefix = 0, above = 0;   // keys whose high byte equals `prefix` are the candidates of pass 2
     for (int pass = 0; pass < 2; pass++) {
-        if (threadIdx.x < 256) {
-            hist[threadIdx.x] = 0;
+#pragma unroll
+        for (int i = 0; i < 256 * 32 / (kSelThreads * 4); i++) {
+            reinterpret_cast<uint4 *>(hist_priv)[threadIdx.x + i * kSelThreads] = make_uint4(0u, 0u, 0u, 0u);
         }
         __syncthreads();
+        const uint32_t my_copy = threadIdx.x & 31u;
         auto count = [&](uint32_t key) {
             if (pass == 0) {
-                atomicAdd(&hist[key >> 8], 1u);
+                atomicAdd(&hist_priv[(key >> 8) * 32 + my_copy], 1u);
             } else if ((key >> 8) == prefix) {
-                atomicAdd(&hist[key & 0xffu], 1u);
+                atomicAdd(&hist_priv[(key & 0xffu) * 32 + my_copy], 1u);
             }
         };
         for (uint32_t j = threadIdx.x * 8; j < n8; j += kSelThreads * 8) {
@@ -483,6 +490,19 @@ indexer_select_kernel(const uint16_t *__restrict__ scores, const int32_t *__rest
         }
         for (uint32_t j = n8 + threadIdx.x; j < n; j += kSelThreads) {
             count(order_key(row[j]));
+        }
+        __syncthreads();
+        {
+            // the bins' totals: thread = (bin, quarter of its copies)
+            const uint32_t b = threadIdx.x >> 2, part = threadIdx.x & 3u;
+            const uint4 x = *reinterpret_cast<const uint4 *>(hist_priv + b * 32 + part * 8);
+            const uint4 y = *reinterpret_cast<const uint4 *>(hist_priv + b * 32 + part * 8 + 4);
+            uint32_t sum = x.x + x.y + x.z + x.w + y.x + y.y + y.z + y.w;
+            sum += __shfl_xor(sum, 1);
+            sum += __shfl_xor(sum, 2);
+            if (part == 0) {
+                hist[b] = sum;
+            }
         }
         __syncthreads();
         // the bin that holds the k-th key, counted from the top: a suffix sum over the 256 bins by one wave
