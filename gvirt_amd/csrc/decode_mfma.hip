@@ -244,7 +244,7 @@ struct DecodeSplit {
     {
         u += p.unit0;   // units are numbered inside the launch's slice
         if (p.only_single) {
-            const int32_t ql = p.lens[u], start = p.query_start_loc[u];
+            const int32_t ql = p.lens[u], start = p.query_start_loc[u], cached = p.cached_lens[u];   // one trip for the three
             *seq = u;
             *tok = static_cast<uint32_t>(start);
             if (ql != 1) {
@@ -256,7 +256,7 @@ struct DecodeSplit {
                 *limit = 0;
                 return 0;
             }
-            const int32_t lim = p.cached_lens[u] + 1;
+            const int32_t lim = cached + 1;
             *limit = static_cast<uint32_t>(lim > 1 ? lim : 1);
             return ceil_div(*limit, static_cast<uint32_t>(kStep));
         }

@@ -686,8 +686,12 @@ mla_decode_kernel(const MlaDecodeParams p)
         if (lane < T) {
             // a decode batch has row t in sequence t: that sequence's cached length is fetched in the same round of
             // loads as the answer to "which sequence" (one memory round trip instead of two)
-            const uint32_t guess = lane < B ? static_cast<uint32_t>(p.cached_lens[lane]) : 0u;
-            const bool own = lane < B && p.query_start_loc[lane] == static_cast<int32_t>(lane) && p.lens[lane] == 1;
+            // (three unconditional loads from a clamped index: written as a chain of && the compiler issues and
+            // awaits them one after the other)
+            const uint32_t li = min(lane, B - 1);
+            const int32_t g_cached = p.cached_lens[li], g_start = p.query_start_loc[li], g_len = p.lens[li];
+            const uint32_t guess = static_cast<uint32_t>(g_cached);
+            const bool own = (lane < B) & (g_start == static_cast<int32_t>(lane)) & (g_len == 1);
             my_seq = own ? lane : seq_of(lane);
             my_causal = own && !dense ? guess + 1 : row_causal(lane, my_seq);
             my_limit = LISTS && my_causal > p.top_k ? p.top_k : my_causal;
