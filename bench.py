@@ -37,6 +37,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE runs of this
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
+PEAK_CLOCK_GHZ = 2.4   # the engine clock the published MI355X matrix peaks are quoted at
 MEASURED_TRAFFIC_BYTES = {"c2": 1080257123, "c3": 335345883, "c4": 306642776, "c5": 1623782068}
 # where each constant comes from: the committed counter summary whose "HBM traffic per launch" line holds it
 TRAFFIC_SOURCE = {"c2": "profiles/decode_dma_kernel_c2_llama3_8b_b64_ctx4096.md",
@@ -53,6 +54,32 @@ def _traffic(key):
 
 def _events(torch):
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def _clock_under_load(torch, rt, fn, iters=200):
+    """Shader clock in GHz over `iters` back-to-back calls of `fn`, from the stamps workgroup 0 of the streaming MLA and
+    prefill kernels leaves when a probe buffer is set (xlite_hip_set_clock_probe): shader-clock ticks over 100 MHz
+    wall-clock ticks of the last launch."""
+    import ctypes
+    buf = torch.zeros(4, dtype=torch.int64, device="cuda:0")
+    rt._lib.xlite_hip_set_clock_probe(ctypes.c_void_p(buf.data_ptr()))
+    try:
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+    finally:
+        rt._lib.xlite_hip_set_clock_probe(None)
+    c0, w0, c1, w1 = [int(x) for x in buf.tolist()]
+    return round((c1 - c0) / ((w1 - w0) * 10.0), 3) if w1 > w0 else None
+
+
+def _clock_fields(clock_ghz, tflops):
+    """The measured clock next to the one the published matrix peak assumes, and the matrix rate against the peak
+    scaled to the measured clock (the published 2.5 PFLOP/s is 256 compute units at 2.4 GHz)."""
+    if not clock_ghz:
+        return {"shader_clock_ghz_under_load": None}
+    return {"shader_clock_ghz_under_load": clock_ghz, "peak_clock_ghz": PEAK_CLOCK_GHZ,
+            "mfma_frac_at_measured_clock": round(tflops / (MFMA_BF16_PEAK_TFLOPS * clock_ghz / PEAK_CLOCK_GHZ), 4)}
 
 
 def _time_region(torch, fn, iters):
@@ -370,7 +397,8 @@ def bench_prefill(args, torch, rt, int8=False):
             "roofline": {"bound": "mfma", "kernel": "dequant_blocks_kernel + prefill_kernel" if int8 else "prefill_kernel",
                          "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                         **(_traffic("c3") if not int8 else {"traffic": None}), "algorithmic_flops_per_step": int(flops)},
+                         **(_traffic("c3") if not int8 else {"traffic": None}), "algorithmic_flops_per_step": int(flops),
+                         **_clock_fields(_clock_under_load(torch, rt, step, iters=10), tf)},
             "cpu_baseline": cpu}
 
 
@@ -405,6 +433,7 @@ def bench_mla(args, torch, rt):
     gbs = w["kv_bytes"] / (ms * 1e-3) / 1e9
     tf = w["flops"] / (ms * 1e-3) / 1e12
     dist = _launch_dist(torch, step)
+    clock_ghz = _clock_under_load(torch, rt, step)
 
     # the two einsums of the mla_v2 operator around the attention (W_UK absorb, W_UV), reported separately
     g = torch.Generator(device="cuda:0").manual_seed(W.SEED_BASE + 44)
@@ -489,7 +518,8 @@ def bench_mla(args, torch, rt):
             "ms_per_step_one_resident_set": round(ms_resident, 4), "einsums": einsum,
             "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel (+ merge_mla_kernel)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), **_traffic("c4"),
-                         "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)},
+                         "frac_of_max_floor": round(floor_ms / ms, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                         **_clock_fields(clock_ghz, tf)},
             "cpu_baseline": cpu}
 
 

@@ -18,6 +18,7 @@ SIGNATURES = {
     "xlite_hip_attention_workspace_bytes": (_sz, [_u32] * 7),
     "xlite_hip_attention_workspace_bytes_kv": (_sz, [_u32] * 7 + [_i32]),
     "xlite_hip_attention": (_i32, [_vp] * 9 + [_u32] * 7 + [_i32, _i32, _vp, _vp, _vp, _sz]),
+    "xlite_hip_set_clock_probe": (_i32, [_vp]),
     "xlite_hip_decode_step": (_i32, [_vp] * 12 + [_u32] * 8 + [_i32, _u64, _u64, _i32, _vp, _sz]),
     "xlite_hip_attention_noalloc_scratch_bytes": (_sz, []),
     "xlite_hip_attention_noalloc": (_i32, [_vp] * 9 + [_u32] * 7 + [_i32, _i32, _vp, _vp]),

@@ -116,6 +116,7 @@ struct MlaDecodeParams {
     float scale_log2e;
     const int32_t *topk_indices;   // [total_rows][top_k] position lists (top_k == 0: none)
     uint32_t top_k;
+    unsigned long long *clock_probe;   // nullptr, or where workgroup 0 leaves its shader-clock and wall-clock stamps
 };
 bool mla_decode_supported(const MlaArgs &a);
 size_t mla_decode_workspace_bytes(const MlaArgs &a);

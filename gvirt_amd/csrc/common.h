@@ -16,6 +16,8 @@ void set_error(const std::string &msg);
 int fail(int code, const char *func, const std::string &msg);
 // allows `bytes` of dynamic LDS for `kernel` on the current device (once per kernel, device and size)
 int ensure_dynamic_lds(const void *kernel, size_t bytes);
+// device buffer of four 64-bit words set through xlite_hip_set_clock_probe, or nullptr (the usual case)
+unsigned long long *clock_probe();
 
 #define XL_REQUIRE(cond, msg)                                                      \
     do {                                                                           \

@@ -2,6 +2,7 @@
 #include <math.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <vector>
 
@@ -45,6 +46,16 @@ int fail(int code, const char *func, const std::string &msg)
 using namespace xlite;
 
 extern "C" const char *xlite_hip_last_error(void) { return g_last_error.c_str(); }
+
+static std::atomic<unsigned long long *> g_clock_probe{nullptr};
+namespace xlite {
+unsigned long long *clock_probe() { return g_clock_probe.load(std::memory_order_relaxed); }
+}  // namespace xlite
+extern "C" int xlite_hip_set_clock_probe(void *device_words)
+{
+    g_clock_probe.store(static_cast<unsigned long long *>(device_words), std::memory_order_relaxed);
+    return XLITE_HIP_OK;
+}
 
 extern "C" int xlite_hip_version(void) { return 1; }
 

@@ -116,6 +116,12 @@ mla_decode_kernel(const MlaDecodeParams p)
         static_cast<uint32_t>((size_t)((__attribute__((address_space(3))) unsigned char *)smem)))));
 
     const uint32_t lane = threadIdx.x & 63;
+    // Instrumentation, off unless a probe buffer was set: workgroup 0 leaves the shader clock counter and the 100 MHz
+    // wall clock at entry and after its last segment, whose ratio is the clock the kernel ran at.
+    if (p.clock_probe != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+        p.clock_probe[0] = clock64();
+        p.clock_probe[1] = wall_clock64();
+    }
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t col = lane & 15;    // head inside the wave's 16 (column of every product)
     const uint32_t gi = lane >> 4;     // which 8 of a k-step's 32 elements / which 4 rows of a result tile
@@ -614,6 +620,10 @@ mla_decode_kernel(const MlaDecodeParams p)
             }
         }
         __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
+        if (p.clock_probe != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+            p.clock_probe[2] = clock64();
+            p.clock_probe[3] = wall_clock64();
+        }
     };
 
     // ---- the work list. Every query row owns ceil(limit / 32) steps.
@@ -930,6 +940,7 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
     }
     char *ws = static_cast<char *>(a.workspace);
     MlaDecodeParams p{};
+    p.clock_probe = clock_probe();
     p.q_absorb = static_cast<const uint16_t *>(a.q_absorb);
     p.qr = static_cast<const uint16_t *>(a.qr);
     p.k_cache = static_cast<const uint16_t *>(a.k_cache);

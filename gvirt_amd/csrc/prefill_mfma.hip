@@ -84,6 +84,7 @@ struct PrefillParams {
     int32_t *part_cnt;         // [token][head] number of partials to merge (0: the value is final)
     float *part_acc;           // [token][head][max_splits][D]
     float *part_ml;            // [token][head][max_splits][2]: reference maximum (log2 domain), normaliser
+    unsigned long long *clock_probe;   // nullptr, or where workgroup 0 leaves its shader-clock and wall-clock stamps
 };
 
 // XOR pattern of the 16-byte chunk index of LDS row `row` (rows are 256 bytes = one bank window). The
@@ -230,6 +231,14 @@ prefill_kernel(const PrefillParams p)
     }
     if (qlen <= 0 || mt >= ceil_div(static_cast<uint32_t>(qlen) * G, static_cast<uint32_t>(kMTile))) {
         return;
+    }
+    // Instrumentation, off unless a probe buffer was set: the workgroup of the first sequence's first tile leaves the
+    // shader clock counter and the 100 MHz wall clock here and behind its tile loop, whose ratio is the clock the
+    // kernel ran at.
+    const bool probe = p.clock_probe != nullptr && seq == 0 && mt == 0 && kvh == 0 && blockIdx.y == 0 && threadIdx.x == 0;
+    if (probe) {
+        p.clock_probe[0] = clock64();
+        p.clock_probe[1] = wall_clock64();
     }
     const uint32_t m_rows = static_cast<uint32_t>(qlen) * G;
     const uint32_t m_first = mt * kMTile;
@@ -547,6 +556,10 @@ prefill_kernel(const PrefillParams p)
         }
     }
     dma_wait<0>();
+    if (probe) {
+        p.clock_probe[2] = clock64();
+        p.clock_probe[3] = wall_clock64();
+    }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     // O^T lane layout: column = M row, register k of tile dt = element 32 dt + 8 (k / 4) + 4 half + k % 4
@@ -673,6 +686,7 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
 {
     const uint32_t G = a.n_heads / a.n_kv_heads;
     PrefillParams p{};
+    p.clock_probe = clock_probe();
     p.q = static_cast<const uint16_t *>(a.qkv);
     p.k_cache = static_cast<const uint16_t *>(a.k_cache);
     p.v_cache = static_cast<const uint16_t *>(a.v_cache);

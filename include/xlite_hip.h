@@ -112,6 +112,18 @@ int xlite_hip_attention(void *stream, const void *qkv, const void *k_cache, cons
                         const float *v_scale, void *workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------------------------------
+ * Instrumentation (no counterpart in the reference). device_words: four 64-bit words in
+ * device memory, or NULL (off, the default). While set, workgroup 0 of every launch of the
+ * streaming MLA kernel and of the streaming prefill kernel stores
+ *   { shader clock counter at entry, 100 MHz wall clock at entry,
+ *     shader clock counter behind its loop, 100 MHz wall clock there }
+ * so that (w[2] - w[0]) / ((w[3] - w[1]) * 10 ns) is the clock the kernel ran at: the part is
+ * power-managed, and the matrix peak is quoted at a clock these kernels do not hold.
+ * Process-wide; the buffer must stay valid until the probe is set to NULL again.
+ * ---------------------------------------------------------------------- */
+int xlite_hip_set_clock_probe(void *device_words);
+
+/* ------------------------------------------------------------------------
  * decode_step — the attention block of one layer as the reference's model loop runs it
  * (xlite/csrc/model.cpp:544-571: XliteOpRopeCache, then XliteOpAttention or
  * XliteOpFlashAttention over the same qkv rows and caches), enqueued from one call:

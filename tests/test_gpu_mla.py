@@ -321,3 +321,24 @@ def test_mla_decode_at_the_longest_reference_context(rt):
     c = mla_case(36, [1, 1], [131071, 131071], 16)
     scale = 192 ** -0.5
     check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
+def test_clock_probe_reports_a_plausible_shader_clock_and_switches_off(rt):
+    """xlite_hip_set_clock_probe: while a buffer is set, workgroup 0 of the streaming MLA kernel leaves shader-clock
+    and 100 MHz wall-clock stamps; their ratio is a clock between 0.3 and 3 GHz; with the probe off nothing is written."""
+    import ctypes
+    c = mla_case(71, [1] * 4, [3000, 2000, 4000, 1000], 128)
+    buf = torch.zeros(4, dtype=torch.int64, device=DEV)
+    rt._lib.xlite_hip_set_clock_probe(ctypes.c_void_p(buf.data_ptr()))
+    try:
+        want = run_mla(rt, c, 192 ** -0.5)
+    finally:
+        rt._lib.xlite_hip_set_clock_probe(None)
+    c0, w0, c1, w1 = [int(x) for x in buf.tolist()]
+    assert w1 > w0 and c1 > c0
+    ghz = (c1 - c0) / ((w1 - w0) * 10.0)
+    assert 0.3 < ghz < 3.0, ghz
+    buf.zero_()
+    got = run_mla(rt, c, 192 ** -0.5)
+    assert torch.equal(got, want)
+    assert int(buf.abs().sum()) == 0
