@@ -16,20 +16,20 @@ union Vec16 {
 // (xlite/csrc/kernels/rope_and_cache.h:93-129): each product is rounded to the storage type, the difference /
 // sum is formed in fp32 and rounded again; the q scale is applied in fp32 and rounded once more (:576-586).
 template <typename T>
-__device__ __forceinline__ void rotate_chunk_pair(Vec16 &a, Vec16 &b, uint32_t e0, uint32_t half, uint32_t t,
+__device__ __forceinline__ void rotate_chunk_pair(Vec16 &a, Vec16 &b, uint32_t e0, uint32_t half, uint32_t t, int64_t pos_t,
                                                   uint32_t num_tokens, uint32_t rot_dim, const int64_t *position,
                                                   const uint16_t *cosin, uint64_t mask_h, uint64_t mask_w, bool is_q,
                                                   float q_scale)
 {
     Vec16 c, s;
     if ((mask_h | mask_w) == 0) {
-        const uint16_t *cs = cosin + static_cast<uint64_t>(position[t]) * rot_dim;
+        const uint16_t *cs = cosin + static_cast<uint64_t>(pos_t) * rot_dim;
         c.v = *reinterpret_cast<const uint4 *>(cs + e0);
         s.v = *reinterpret_cast<const uint4 *>(cs + half + e0);
     } else {
         // lane j of the rotary half takes its angle from the height / width position
         // when bit j of the matching mask is set, else from the temporal position
-        const uint16_t *cs_t = cosin + static_cast<uint64_t>(position[t]) * rot_dim;
+        const uint16_t *cs_t = cosin + static_cast<uint64_t>(pos_t) * rot_dim;
         const uint16_t *cs_h = cosin + static_cast<uint64_t>(position[num_tokens + t]) * rot_dim;
         const uint16_t *cs_w = cosin + static_cast<uint64_t>(position[2ull * num_tokens + t]) * rot_dim;
 #pragma unroll
@@ -95,9 +95,16 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
 
         const bool is_q = hs < n_heads;
         const bool is_k = !is_q && hs < n_heads + n_kv_heads;
+        // the token's position and slot are requested together with its row (every thread loads both: under a
+        // condition each would be a trip to memory of its own); only the cos / sin row waits for the position
+        const int64_t pos_t = position[t];
+        const uint32_t slot = static_cast<uint32_t>(slot_mapping[t]);
+        const uint32_t e_first = item < rot_pairs ? item * 8 : (item + rot_pairs) * 8;
+        Vec16 a, b;
+        a.v = *reinterpret_cast<const uint4 *>(row + e_first);
+        b.v = *reinterpret_cast<const uint4 *>(row + (item < rot_pairs ? e_first + half : e_first));
         uint16_t *cache_row = nullptr;
         if (!is_q && k_cache != nullptr) {   // no 16-bit caches: the caller quantises the rows afterwards
-            const uint32_t slot = static_cast<uint32_t>(slot_mapping[t]);
             const uint32_t kvh = is_k ? hs - n_heads : hs - n_heads - n_kv_heads;
             const uint64_t off =
                 ((static_cast<uint64_t>(slot / block_size) * block_size + slot % block_size) * n_kv_heads +
@@ -107,11 +114,8 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
 
         if (item < rot_pairs) {
             const uint32_t e0 = item * 8;  // first-half elements e0..e0+7, partners at +half
-            Vec16 a, b;
-            a.v = *reinterpret_cast<const uint4 *>(row + e0);
-            b.v = *reinterpret_cast<const uint4 *>(row + e0 + half);
             if (is_q || is_k) {
-                rotate_chunk_pair<T>(a, b, e0, half, t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
+                rotate_chunk_pair<T>(a, b, e0, half, t, pos_t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
                 *reinterpret_cast<uint4 *>(row + e0) = a.v;
                 *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
             }
@@ -121,8 +125,6 @@ rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cac
             }
         } else {
             const uint32_t e0 = (item + rot_pairs) * 8;  // beyond the rotary span
-            Vec16 a;
-            a.v = *reinterpret_cast<const uint4 *>(row + e0);
             if (is_q) {
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -514,6 +516,7 @@ rope_quant_cache_kernel(uint16_t *__restrict__ inout, unsigned char *__restrict_
         const bool active = lane < items_per_head;
         const bool rot = active && lane < rot_pairs;
         const uint32_t e0 = rot ? lane * 8 : (lane + rot_pairs) * 8;
+        const int64_t pos_t = position[t];   // requested with the row, not behind it
         Vec16 a, b;
         a.v = make_uint4(0, 0, 0, 0);
         b.v = make_uint4(0, 0, 0, 0);
@@ -523,7 +526,7 @@ rope_quant_cache_kernel(uint16_t *__restrict__ inout, unsigned char *__restrict_
                 b.v = *reinterpret_cast<const uint4 *>(row + e0 + half);
             }
             if (rot && (is_q || is_k)) {
-                rotate_chunk_pair<T>(a, b, e0, half, t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
+                rotate_chunk_pair<T>(a, b, e0, half, t, pos_t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
                 *reinterpret_cast<uint4 *>(row + e0) = a.v;
                 *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
             } else if (is_q) {
