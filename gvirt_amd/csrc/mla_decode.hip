@@ -322,21 +322,37 @@ mla_decode_kernel(const MlaDecodeParams p)
             // The two accumulation chains alternate; operands are fetched kAhead products ahead.
             // The first kAhead operands are fetched by `qk_fetch`, which the loop calls right behind the step's barrier:
             // their latency then overlaps the address arithmetic of the copies issued in between.
-            auto rd_k = [&](uint32_t soff, int i) {
-                const int ks = i >> 1, mt = i & 1;
-                return ks < KS_C
-                           ? *reinterpret_cast<const uint4 *>(smem + soff + k_row + (((ks & 3) << 6) ^ kx) + ((ks >> 2) << 8) + mt * 16 * KC_ROWB)
-                           : *reinterpret_cast<const uint4 *>(smem + soff + p_row + (((ks - KS_C) << 6) ^ px) + mt * 16 * PE_ROWB);
-            };
-            auto qk_fetch = [&](uint32_t step, uint4 (&a)[kAhead]) {
+            // The operand reads of a step go through six per-lane base offsets (the four XOR variants of the latent
+            // rows, the two of the rotary rows), formed once per step and made opaque to the compiler; everything else
+            // of a read's address is a constant that fits the instruction's offset field. (Left to itself the compiler
+            // forms biased bases and adds a negative constant per read: 35 vector additions per step.)
+            uint32_t kbase[4], pbase[2];
+            auto set_bases = [&](uint32_t step) {
                 const uint32_t soff = (step % kStages) * STAGE_BYTES;
 #pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    kbase[j] = soff + k_row + ((j << 6) ^ kx);
+                    asm volatile("" : "+v"(kbase[j]));
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    pbase[j] = soff + p_row + ((j << 6) ^ px);
+                    asm volatile("" : "+v"(pbase[j]));
+                }
+            };
+            auto rd_k = [&](int i) {
+                const int ks = i >> 1, mt = i & 1;
+                return ks < KS_C ? *reinterpret_cast<const uint4 *>(smem + kbase[ks & 3] + (((ks >> 2) << 8) + mt * 16 * KC_ROWB))
+                                 : *reinterpret_cast<const uint4 *>(smem + pbase[ks - KS_C] + mt * 16 * PE_ROWB);
+            };
+            auto qk_fetch = [&](uint32_t step, uint4 (&a)[kAhead]) {
+                set_bases(step);
+#pragma unroll
                 for (int i = 0; i < kAhead; i++) {
-                    a[i] = rd_k(soff, i);
+                    a[i] = rd_k(i);
                 }
             };
             auto qk = [&](uint32_t step, f32x4_t (&S)[2], uint4 (&a)[kAhead]) {
-                const uint32_t soff = (step % kStages) * STAGE_BYTES;
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
                     S[0][k] = 0.f;
@@ -348,7 +364,7 @@ mla_decode_kernel(const MlaDecodeParams p)
                                                                      __builtin_bit_cast(bf16x8_t, qreg[i >> 1]),
                                                                      S[i & 1], 0, 0, 0);
                     if (i + kAhead < 2 * (KS_C + KS_R)) {
-                        a[i % kAhead] = rd_k(soff, i + kAhead);
+                        a[i % kAhead] = rd_k(i + kAhead);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -446,7 +462,6 @@ mla_decode_kernel(const MlaDecodeParams p)
             // Four transposed latent operands (two reads each) and eight probability operands per step.
             auto pv = [&](uint32_t step) {
                 const uint32_t soff = (step % kStages) * STAGE_BYTES;
-                const unsigned char *pbuf = p_lds + (step & 1) * P_BYTES;
                 typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
                 // the heads' rescale factors (rarely other than 1)
                 {
@@ -470,14 +485,27 @@ mla_decode_kernel(const MlaDecodeParams p)
                         }
                     }
                 }
+                // (per-lane base offsets formed once per step and opaque to the compiler, the rest of an address a
+                // constant in the instruction's offset field: see the first product)
+                uint32_t vbase[2][CT], prbase[2];
+#pragma unroll
+                for (int ct = 0; ct < CT; ct++) {
+                    vbase[0][ct] = soff + (vt0 ^ (ct << 6));
+                    vbase[1][ct] = soff + (vt1 ^ (ct << 6));
+                    asm volatile("" : "+v"(vbase[0][ct]), "+v"(vbase[1][ct]));
+                }
+#pragma unroll
+                for (int ks2 = 0; ks2 < 2; ks2++) {
+                    prbase[ks2] = (step & 1) * P_BYTES + (pr_off ^ (ks2 << 5));
+                    asm volatile("" : "+v"(prbase[ks2]));
+                }
                 auto rd_v = [&](int ks2, int ct) {
-                    const unsigned char *base = smem + soff + ks2 * 16 * KC_ROWB;
-                    const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + (vt0 ^ (ct << 6)))));
-                    const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(base + (vt1 ^ (ct << 6)))));
+                    const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(smem + vbase[0][ct] + ks2 * 16 * KC_ROWB)));
+                    const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(smem + vbase[1][ct] + ks2 * 16 * KC_ROWB)));
                     return make_uint4(lo.x, lo.y, hi.x, hi.y);
                 };
                 auto rd_p = [&](int ks2, int hg) {
-                    return *reinterpret_cast<const uint4 *>(pbuf + hg * 32 * P_ROWB + (pr_off ^ (ks2 << 5)));
+                    return *reinterpret_cast<const uint4 *>(p_lds + prbase[ks2] + hg * 32 * P_ROWB);
                 };
                 // (operands of one k-step at a time: 24 registers; the SIMD's other wave covers their latency)
 #pragma unroll
