@@ -91,6 +91,7 @@ struct DecodeMfmaParams {
     uint32_t step_mult;    // steps (of 16 positions) the kernel takes at a time: chunks are multiples of it
     uint32_t block_magic;  // floor(2^32 / block_size) + 1: position / block_size == mulhi(position, magic) for positions
                            // below 2^32 / block_size; 0 when a table reaches further (then the kernels divide)
+    uint32_t whole_rows;   // 1: no split - workgroup i walks the whole range of the rows i, i + grid, ...: nothing to merge
 };
 
 // block and offset inside it of position t (a division by a run-time block size is some twenty instructions)
@@ -287,6 +288,10 @@ struct DecodeSplit {
     // second case: every thread of the workgroup calls it.
     __device__ __forceinline__ void scan()
     {
+        if (p.whole_rows) {   // (the rows are looked up one by one in for_each_segment)
+            total = 1;
+            return;
+        }
         if (in_lanes) {
             if (lane < R) {
                 ln_steps = steps_of(lane, &ln_limit, &ln_seq, &ln_tok, true);
@@ -389,6 +394,19 @@ struct DecodeSplit {
     template <typename F>
     __device__ __forceinline__ void for_each_segment(F &&segment) const
     {
+        if (p.whole_rows) {
+            // batches whose contexts are short by the width of their block tables: a row is one segment, stored
+            // directly, and there is no second launch to merge anything (a step of such a batch is bound by its
+            // launches, not by its bytes)
+            for (uint32_t row = blockIdx.x; row < R; row += gridDim.x) {
+                uint32_t limit, seq, tok;
+                const uint32_t n = steps_of(row, &limit, &seq, &tok, false);
+                if (n != 0) {
+                    segment(uni(seq), uni(tok), 0u, uni(limit), true, 0u, false, make_int4(0, 0, 0, 0));
+                }
+            }
+            return;
+        }
         for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
             const uint32_t start = c * chunk, end = min(total, start + chunk);
             uint32_t row = row_of_step(start), pos = start;
@@ -1798,6 +1816,16 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     // slice. (Sequences' rows lie anywhere among the batch's rows, so a batch served by two kernels is one slice.)
     const uint32_t units = p.only_single ? a.batch : a.total_tokens;
     XL_REQUIRE(!p.only_single || units <= kSplitSeqCap, "too many sequences for a batch served by two kernels");
+    // Contexts that are short by the width of the block tables (at most 16 steps per wave: the waves of a kv head
+    // share a row when there are fewer than 8 kv heads): no split, one workgroup per row, no merge launch. Such a
+    // step is bound by its launches: Qwen2-0.5B, 4 sequences of up to 512 positions, 12.7 us + 3.9 us of merge -> one
+    // kernel.
+    const uint32_t waves_per_kv = a.n_kv_heads >= kWaves ? 1u : kWaves / a.n_kv_heads;
+    const bool whole_rows = !p.only_single &&
+                            ceil_div(static_cast<uint64_t>(a.max_num_block) * a.block_size, static_cast<uint64_t>(kStep)) <=
+                                16ull * waves_per_kv &&
+                            a.max_num_block <= kSplitTblCap - 2;
+    p.whole_rows = whole_rows ? 1u : 0u;
     for (uint32_t u0 = 0; u0 < units; u0 += kSplitSeqCap) {
         p.unit0 = u0;
         p.n_units = min(kSplitSeqCap, units - u0);
@@ -1806,23 +1834,27 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
         p.block_magic = static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32)
                             ? static_cast<uint32_t>((1ull << 32) / a.block_size) + 1
                             : 0u;
+        const uint32_t gx = whole_rows ? min(grid_x, p.n_units) : grid_x;   // (whole rows: no workgroups without a row)
         if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             p.step_mult = a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1;
-            rc = bf ? launch_dma<BF16>(stream, p, grid_x) : launch_dma<FP16>(stream, p, grid_x);
+            rc = bf ? launch_dma<BF16>(stream, p, gx) : launch_dma<FP16>(stream, p, gx);
         } else if (decode_dma8_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             p.step_mult = 2 * (a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1);   // a wave takes 32 positions at a time
             if (a.kv_dtype == XLITE_HIP_KV_FP8) {
-                rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_FP8>(stream, p, grid_x) : launch_dma8<FP16, XLITE_HIP_KV_FP8>(stream, p, grid_x);
+                rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_FP8>(stream, p, gx) : launch_dma8<FP16, XLITE_HIP_KV_FP8>(stream, p, gx);
             } else {
-                rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_INT8>(stream, p, grid_x) : launch_dma8<FP16, XLITE_HIP_KV_INT8>(stream, p, grid_x);
+                rc = bf ? launch_dma8<BF16, XLITE_HIP_KV_INT8>(stream, p, gx) : launch_dma8<FP16, XLITE_HIP_KV_INT8>(stream, p, gx);
             }
         } else if (a.head_dim == 128) {
-            rc = bf ? launch_fmt<BF16, 128>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 128>(stream, p, grid_x, a.kv_dtype);
+            rc = bf ? launch_fmt<BF16, 128>(stream, p, gx, a.kv_dtype) : launch_fmt<FP16, 128>(stream, p, gx, a.kv_dtype);
         } else {
-            rc = bf ? launch_fmt<BF16, 64>(stream, p, grid_x, a.kv_dtype) : launch_fmt<FP16, 64>(stream, p, grid_x, a.kv_dtype);
+            rc = bf ? launch_fmt<BF16, 64>(stream, p, gx, a.kv_dtype) : launch_fmt<FP16, 64>(stream, p, gx, a.kv_dtype);
         }
         if (rc != XLITE_HIP_OK) {
             return rc;
+        }
+        if (whole_rows) {
+            continue;   // every row was stored directly
         }
         if (!p.only_single) {
             // the slice's rows are u0 .. u0 + n_units - 1
