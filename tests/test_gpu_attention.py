@@ -576,3 +576,30 @@ def test_head_dim_256_quantised_cache_is_refused(rt):
     w.update(k_cache=kq, v_cache=vq, k_scale=ks, v_scale=vs)
     with pytest.raises(RuntimeError, match="head_dim must be 64 or 128"):
         run_attention(rt, w)
+
+
+@pytest.mark.parametrize("model", [(14, 2, 64, torch.bfloat16), (32, 8, 128, torch.bfloat16), (28, 4, 128, torch.float16),
+                                   (32, 8, 128, "int8")])
+def test_short_block_tables_run_whole_rows_and_agree_with_the_split_path(rt, model):
+    """A decode batch whose block tables are narrow (at most 16 steps per wave) is served without a split and without
+    a merge launch; the same batch behind wider tables (same blocks, padding columns) takes the split path. Both
+    against the oracle, and against each other."""
+    nH, nKV, d, dtype = model
+    int8 = dtype == "int8"
+    ctx = [1, 15, 16, 17, 100, 128, 129, 200, 255, 256]
+    if nKV < 8:
+        ctx += [300, 511, 512]
+    w = generic_case(81, [1] * len(ctx), [c - 1 for c in ctx], nH, nKV, d, 16, torch.bfloat16 if int8 else dtype, rms=int8)
+    if int8:
+        w = quantised(w, torch.int8)
+    ref = oracle_attention(w)
+    narrow = run_attention(rt, w)
+    check(narrow, ref, 5e-2 if int8 else MAX_ABS, 5e-3 if int8 else MEAN_ABS)
+    wide = dict(w)
+    mb, pad = w["max_num_block"], 300   # 300 more columns: far beyond the whole-row bound
+    t = w["block_tables"].view(w["batch"], mb)
+    wide["block_tables"] = torch.cat([t, torch.zeros(w["batch"], pad, dtype=torch.int32)], dim=1).flatten().contiguous()
+    wide["max_num_block"] = mb + pad
+    split = run_attention(rt, wide)
+    check(split, ref, 5e-2 if int8 else MAX_ABS, 5e-3 if int8 else MEAN_ABS)
+    assert float((split - narrow).abs().max()) <= 1e-2
