@@ -206,6 +206,34 @@ prefill_kernel(const PrefillParams p)
         qlen = __builtin_amdgcn_readlane(my_len, static_cast<int>(seq));
         clen = __builtin_amdgcn_readlane(my_cached, static_cast<int>(seq));
         mt = tid - static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(fid), static_cast<int>(seq)));
+    } else if (__builtin_amdgcn_readfirstlane(p.batch <= 16 * kThreads ? 1 : 0)) {
+        // up to 8192 sequences: the whole workgroup counts the sequences that start at or before `tid`, every thread a
+        // few of them with independent loads - one trip to memory, where the bisection below is a chain of a dozen (a
+        // mixed batch of a thousand decode rows pays that chain in every one of its thousands of empty workgroups)
+        uint32_t mine = 0;
+        for (uint32_t i = threadIdx.x; i < p.batch; i += kThreads) {
+            mine += first_id(i) <= tid ? 1u : 0u;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            mine += __shfl_xor(mine, d);
+        }
+        uint32_t *cnt_lds = reinterpret_cast<uint32_t *>(smem);   // (the stages are not in use yet)
+        if (lane == 0) {
+            cnt_lds[wave] = mine;
+        }
+        __syncthreads();
+        uint32_t started = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) {
+            started += cnt_lds[w];
+        }
+        __syncthreads();   // the words are free again before anything else is written there
+        seq = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(started))) - 1;   // first_id(0) == 0: at least one
+        mt = tid - first_id(seq);
+        qlen = p.lens[seq];
+        clen = p.cached_lens[seq];
+        qstart = p.query_start_loc[seq];
     } else {
         uint32_t hi = p.batch;   // first_id(seq) <= tid < first_id(hi); first_id(0) == 0
         while (hi - seq > 1) {
