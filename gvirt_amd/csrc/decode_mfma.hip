@@ -91,7 +91,6 @@ struct DecodeMfmaParams {
     uint32_t step_mult;    // steps (of 16 positions) the kernel takes at a time: chunks are multiples of it
     uint32_t block_magic;  // floor(2^32 / block_size) + 1: position / block_size == mulhi(position, magic) for positions
                            // below 2^32 / block_size; 0 when a table reaches further (then the kernels divide)
-    uint32_t whole_rows;   // 1: no split - workgroup i walks the whole range of the rows i, i + grid, ...: nothing to merge
 };
 
 // block and offset inside it of position t (a division by a run-time block size is some twenty instructions)
@@ -204,6 +203,10 @@ __device__ __forceinline__ uint32_t uni(uint32_t x)
     return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(x)));
 }
 
+// WHOLE: no split - workgroup i walks the whole range of the rows i, i + grid, ...: nothing to merge (a template
+// parameter, so that each kernel has one call site for its segment body: a second copy of that body, or the extra live
+// values of a run-time choice, cost the streaming kernels 4 %)
+template <bool WHOLE = false>
 struct DecodeSplit {
     const DecodeMfmaParams &p;
     uint32_t *wave_tot, *pref;   // LDS: kWaves words, units + 1 words
@@ -288,7 +291,7 @@ struct DecodeSplit {
     // second case: every thread of the workgroup calls it.
     __device__ __forceinline__ void scan()
     {
-        if (p.whole_rows) {   // (the rows are looked up one by one in for_each_segment)
+        if constexpr (WHOLE) {   // (the rows are looked up one by one in for_each_segment)
             total = 1;
             return;
         }
@@ -394,7 +397,7 @@ struct DecodeSplit {
     template <typename F>
     __device__ __forceinline__ void for_each_segment(F &&segment) const
     {
-        if (p.whole_rows) {
+        if constexpr (WHOLE) {
             // batches whose contexts are short by the width of their block tables: a row is one segment, stored
             // directly, and there is no second launch to merge anything (a step of such a batch is bound by its
             // launches, not by its bytes)
@@ -405,33 +408,33 @@ struct DecodeSplit {
                     segment(uni(seq), uni(tok), 0u, uni(limit), true, 0u, false, make_int4(0, 0, 0, 0));
                 }
             }
-            return;
-        }
-        for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-            const uint32_t start = c * chunk, end = min(total, start + chunk);
-            uint32_t row = row_of_step(start), pos = start;
-            while (pos < end) {
-                uint32_t first, n, limit;
-                row_info(row, &first, &n, &limit);
-                if (n == 0) {   // a unit that takes no part (units without steps share their prefix with the next one)
+        } else {
+            for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+                const uint32_t start = c * chunk, end = min(total, start + chunk);
+                uint32_t row = row_of_step(start), pos = start;
+                while (pos < end) {
+                    uint32_t first, n, limit;
+                    row_info(row, &first, &n, &limit);
+                    if (n == 0) {   // a unit that takes no part (units without steps share their prefix with the next one)
+                        row++;
+                        continue;
+                    }
+                    const uint32_t a = pos - first, b = min(n, a + (end - pos));
+                    const bool whole = a == 0 && b == n;
+                    const bool first_seg = pos == start;
+                    const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
+                    const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
+                    segment(seq_of(row), tok_of(row), uni(a * kStep), uni(min(limit, b * kStep)), whole,
+                            uni(2 * c + (first_seg ? 0u : 1u)), a == 0, meta);
+                    pos += b - a;
                     row++;
-                    continue;
                 }
-                const uint32_t a = pos - first, b = min(n, a + (end - pos));
-                const bool whole = a == 0 && b == n;
-                const bool first_seg = pos == start;
-                const uint32_t n_slots = whole ? 0u : (first + n - 1) / chunk - c + 1;
-                const int4 meta = make_int4(static_cast<int>(n_slots), static_cast<int>(c), first_seg ? 1 : 0, 0);
-                segment(seq_of(row), tok_of(row), uni(a * kStep), uni(min(limit, b * kStep)), whole,
-                        uni(2 * c + (first_seg ? 0u : 1u)), a == 0, meta);
-                pos += b - a;
-                row++;
             }
         }
     }
 };
 
-template <typename T, int D, int KVF, bool MULTI_SUB>
+template <typename T, int D, int KVF, bool MULTI_SUB, bool WHOLE = false>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_mfma_kernel(const DecodeMfmaParams p)
 {
@@ -865,7 +868,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
     };
 
-    DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave, !(MULTI_SUB && D == 128));
+    DecodeSplit<WHOLE> split(p, tbl_lds + kSplitTblCap, lane, wave, !(MULTI_SUB && D == 128));
     split.scan();
     if (split.total == 0) {
         return;
@@ -959,7 +962,7 @@ decode_dma_kernel(const DecodeMfmaParams p)
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t row_bytes = p.n_kv_heads * HEADB;
 
-    DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
+    DecodeSplit<> split(p, tbl_lds + kSplitTblCap, lane, wave);
     split.scan();
     if (split.total == 0) {
         return;
@@ -1340,7 +1343,7 @@ decode_dma8_kernel(const DecodeMfmaParams p)
 
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
 
-    DecodeSplit split(p, tbl_lds + kSplitTblCap, lane, wave);
+    DecodeSplit<> split(p, tbl_lds + kSplitTblCap, lane, wave);
     split.scan();
     if (split.total == 0) {
         return;
@@ -1677,13 +1680,13 @@ int launch_dma8(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgr
     }
 }
 
-template <typename T, int D, int KVF, bool MULTI_SUB>
+template <typename T, int D, int KVF, bool MULTI_SUB, bool WHOLE = false>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
                        (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
-    auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB>;
+    auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB, WHOLE>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
             return rc;
@@ -1700,6 +1703,14 @@ int launch_one(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     return p.n_sub > 1 ? launch_inst<T, D, KVF, true>(stream, p, grid_x)
                        : launch_inst<T, D, KVF, false>(stream, p, grid_x);
+}
+
+// the whole-row instantiations (16-bit caches)
+template <typename T, int D>
+int launch_whole(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
+{
+    return p.n_sub > 1 ? launch_inst<T, D, XLITE_HIP_KV_SAME, true, true>(stream, p, grid_x)
+                       : launch_inst<T, D, XLITE_HIP_KV_SAME, false, true>(stream, p, grid_x);
 }
 
 template <typename T, int D>
@@ -1821,11 +1832,10 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     // step is bound by its launches: Qwen2-0.5B, 4 sequences of up to 512 positions, 12.7 us + 3.9 us of merge -> one
     // kernel.
     const uint32_t waves_per_kv = a.n_kv_heads >= kWaves ? 1u : kWaves / a.n_kv_heads;
-    const bool whole_rows = !p.only_single &&
+    const bool whole_rows = !p.only_single && a.kv_dtype == XLITE_HIP_KV_SAME &&
                             ceil_div(static_cast<uint64_t>(a.max_num_block) * a.block_size, static_cast<uint64_t>(kStep)) <=
                                 16ull * waves_per_kv &&
                             a.max_num_block <= kSplitTblCap - 2;
-    p.whole_rows = whole_rows ? 1u : 0u;
     for (uint32_t u0 = 0; u0 < units; u0 += kSplitSeqCap) {
         p.unit0 = u0;
         p.n_units = min(kSplitSeqCap, units - u0);
@@ -1835,7 +1845,10 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
                             ? static_cast<uint32_t>((1ull << 32) / a.block_size) + 1
                             : 0u;
         const uint32_t gx = whole_rows ? min(grid_x, p.n_units) : grid_x;   // (whole rows: no workgroups without a row)
-        if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
+        if (whole_rows) {   // (the register-staged kernel, whatever the shape: these contexts are a few steps long)
+            rc = a.head_dim == 128 ? (bf ? launch_whole<BF16, 128>(stream, p, gx) : launch_whole<FP16, 128>(stream, p, gx))
+                                   : (bf ? launch_whole<BF16, 64>(stream, p, gx) : launch_whole<FP16, 64>(stream, p, gx));
+        } else if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             p.step_mult = a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1;
             rc = bf ? launch_dma<BF16>(stream, p, gx) : launch_dma<FP16>(stream, p, gx);
         } else if (decode_dma8_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
