@@ -38,7 +38,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
 PEAK_CLOCK_GHZ = 2.4   # the engine clock the published MI355X matrix peaks are quoted at
-MEASURED_TRAFFIC_BYTES = {"c2": 1080257123, "c3": 335345883, "c4": 306642776, "c5": 1623782068}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080233421, "c3": 334714478, "c4": 274685113, "c5": 1623780115}
 # where each constant comes from: the committed counter summary whose "HBM traffic per launch" line holds it
 TRAFFIC_SOURCE = {"c2": "profiles/decode_dma_kernel_c2_llama3_8b_b64_ctx4096.md",
                   "c3": "profiles/prefill_kernel_c3_qwen25_7b_chunked.md",

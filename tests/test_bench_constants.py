@@ -12,7 +12,7 @@ def test_traffic_constants_are_the_figures_of_the_committed_summaries():
     for key, path in bench.TRAFFIC_SOURCE.items():
         text = open(os.path.join(ROOT, path)).read()
         section = text[text.index("## HBM traffic per launch"):]
-        rows = re.findall(r"^\| `(\w+)` \| \d+ \| [\d.]+ \| [\d.]+ \| ([\d.]+) \|", section, flags=re.M)
+        rows = re.findall(r"^\| `([^`]+)` \| \d+ \| [\d.]+ \| [\d.]+ \| ([\d.]+) \|", section, flags=re.M)
         assert rows, path
         megabytes = float(rows[0][1])   # the dominant kernel comes first
         assert abs(megabytes - bench.MEASURED_TRAFFIC_BYTES[key] / 1e6) <= 0.051, (key, megabytes)
