@@ -155,7 +155,9 @@ int launch_kv_dequant(hipStream_t stream, AttentionArgs *a)
     if (a->workspace == nullptr || a->workspace_bytes < l.total) {
         return fail(XLITE_HIP_ENOSPC, __func__,
                     "workspace too small: this batch over a quantised cache needs " + std::to_string(l.total) +
-                        " bytes for the 16-bit copy of its blocks, have " + std::to_string(a->workspace_bytes));
+                        " bytes for the 16-bit copy of its blocks (2 tensors x batch x max_num_block x block_size x "
+                        "n_kv_heads x head_dim x 2 bytes, plus a table of batch x max_num_block entries: every block the "
+                        "tables can name, whatever the sequences' lengths), have " + std::to_string(a->workspace_bytes));
     }
     char *ws = static_cast<char *>(a->workspace);
     uint16_t *k_out = reinterpret_cast<uint16_t *>(ws);

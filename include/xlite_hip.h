@@ -76,7 +76,10 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  *             query heads per kv head, block size a multiple of 16) read the bytes directly;
  *             every other batch over a quantised cache (prefill, chunked prefill, mixed
  *             batches, other decode shapes) first copies the blocks it can see into a 16-bit
- *             cache in the workspace, which xlite_hip_attention_workspace_bytes_kv() sizes.
+ *             cache in the workspace, which xlite_hip_attention_workspace_bytes_kv() sizes:
+ *             2 tensors x batch x max_num_block x block_size x n_kv_heads x head_dim x 2 bytes
+ *             (every block the tables can name, whatever the sequences' lengths: keep
+ *             max_num_block close to what the batch needs).
  * output      [total_tokens, n_heads * head_dim]
  * query_start_loc, lens, cached_lens  [batch] int32
  * block_tables [batch * max_num_block] int32
