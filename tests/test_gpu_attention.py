@@ -603,3 +603,15 @@ def test_short_block_tables_run_whole_rows_and_agree_with_the_split_path(rt, mod
     split = run_attention(rt, wide)
     check(split, ref, 5e-2 if int8 else MAX_ABS, 5e-3 if int8 else MEAN_ABS)
     assert float((split - narrow).abs().max()) <= 1e-2
+
+
+def test_whole_row_mode_with_more_rows_than_workgroups(rt):
+    """600 decode rows behind narrow block tables: the whole-row kernel's workgroups take several rows each."""
+    rng = np.random.default_rng(11)
+    ctx = [int(x) for x in rng.integers(1, 257, size=600)]
+    w = generic_case(82, [1] * len(ctx), [c - 1 for c in ctx], 32, 8, 128, 16, torch.bfloat16)
+    assert w["max_num_block"] * 16 <= 256
+    got = run_attention(rt, w)
+    rows = list(range(0, 600, 7)) + [599]
+    check(got, oracle_attention(w, seqs=rows), rows=rows)
+    assert bool(torch.isfinite(got).all())
