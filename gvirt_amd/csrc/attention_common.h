@@ -117,6 +117,8 @@ struct MlaDecodeParams {
     const int32_t *topk_indices;   // [total_rows][top_k] position lists (top_k == 0: none)
     uint32_t top_k;
     unsigned long long *clock_probe;   // nullptr, or where workgroup 0 leaves its shader-clock and wall-clock stamps
+    uint32_t by_pos;      // 1: block sizes that are not a multiple of 32 - every row walks a list of positions, its own
+                          // (0, 1, 2, ...) unless topk_indices gives it one
 };
 bool mla_decode_supported(const MlaArgs &a);
 size_t mla_decode_workspace_bytes(const MlaArgs &a);

@@ -170,7 +170,11 @@ mla_decode_kernel(const MlaDecodeParams p)
         const uint32_t t1 = min(limit, step_b * kStep);
         const uint32_t n_steps = step_b - step_a;
         const bool single = n_slots == 1;
-        const bool listed = LISTS && causal > p.top_k;
+        // (by_pos: a block size that is not a multiple of 32 - a step's positions do not share a block, so every row
+        // is walked position by position through the same staging of cache rows; rows without a list of their own
+        // walk 0, 1, 2, ...)
+        const bool by_list = LISTS && p.top_k != 0 && causal > p.top_k;
+        const bool listed = LISTS && (by_list || p.by_pos != 0);
         const uint32_t blk0 = dense || listed ? 0 : t0 / p.block_size;
         // ---- [q_absorb | qr] of the lane's head: 16 bytes of every 64-byte k-step. Heads past the end repeat
         // the last one; their results are never stored. The first pass's loads are issued here, ahead of the
@@ -208,8 +212,13 @@ mla_decode_kernel(const MlaDecodeParams p)
                 int32_t x = -1;
                 bool ok = false;
                 if (i < n_steps * kStep && j < t1) {
-                    x = list[j];
-                    ok = x >= 0 && static_cast<uint32_t>(x) < causal && (j == 0 || list[j - 1] != x);
+                    if (by_list) {
+                        x = list[j];
+                        ok = x >= 0 && static_cast<uint32_t>(x) < causal && (j == 0 || list[j - 1] != x);
+                    } else {   // the row's own positions
+                        x = static_cast<int32_t>(j);
+                        ok = true;
+                    }
                 }
                 const uint32_t pos = ok ? static_cast<uint32_t>(x) : 0u;
                 if (i < n_steps * kStep) {
@@ -712,7 +721,7 @@ mla_decode_kernel(const MlaDecodeParams p)
     // positions the row walks: its causal range, or its list of top_k entries when the range is longer
     auto row_limit = [&](uint32_t t, uint32_t seq) -> uint32_t {
         const uint32_t causal = row_causal(t, seq);
-        return LISTS && causal > p.top_k ? p.top_k : causal;
+        return LISTS && p.top_k != 0 && causal > p.top_k ? p.top_k : causal;
     };
     uint32_t chunk_cap = (kTblCap - 2) * p.block_size / kStep;
     if (LISTS) {
@@ -732,7 +741,7 @@ mla_decode_kernel(const MlaDecodeParams p)
             const bool own = (lane < B) & (g_start == static_cast<int32_t>(lane)) & (g_len == 1);
             my_seq = own ? lane : seq_of(lane);
             my_causal = own && !dense ? guess + 1 : row_causal(lane, my_seq);
-            my_limit = LISTS && my_causal > p.top_k ? p.top_k : my_causal;
+            my_limit = LISTS && p.top_k != 0 && my_causal > p.top_k ? p.top_k : my_causal;
             my_n = ceil_div(my_limit, static_cast<uint32_t>(kStep));
             if (my_n == 0 && blockIdx.x == 0 && wave == 0) {
                 reinterpret_cast<int4 *>(p.part_meta)[lane] = make_int4(0, 0, 0, 0);   // a row without keys: nothing to merge
@@ -896,8 +905,8 @@ bool mla_decode_supported(const MlaArgs &a)
 {
     const bool dense = a.block_tables == nullptr;
     // position lists (top_k) go with the paged cache only
-    return a.kv_lora_rank == C && a.rope_head_dim == R && (dense ? a.top_k == 0 : a.block_size % kStep == 0) &&
-           a.top_k <= 2048;
+    // (a paged cache of any block size: those that are not a multiple of 32 are walked position by position)
+    return a.kv_lora_rank == C && a.rope_head_dim == R && (dense ? a.top_k == 0 : a.block_size > 0) && a.top_k <= 2048;
 }
 
 namespace {
@@ -933,7 +942,8 @@ int mla_decode_plan(const MlaArgs &a, MlaPlan *pl)
     pl->n_workgroups = static_cast<uint32_t>(n_cu);
     const uint64_t max_steps = (max_len + kStep - 1) / kStep;
     uint64_t chunk_cap = static_cast<uint64_t>(kTblCap - 2) * (dense ? kStep : a.block_size) / kStep;
-    if (a.top_k != 0 && chunk_cap > kTblCap / kStep) {
+    const bool by_pos = !dense && a.block_size % kStep != 0;
+    if ((a.top_k != 0 || by_pos) && chunk_cap > kTblCap / kStep) {
         chunk_cap = kTblCap / kStep;
     }
     const uint64_t by_cap = (static_cast<uint64_t>(a.total_tokens) * max_steps + chunk_cap - 1) / chunk_cap;
@@ -996,7 +1006,8 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a)
     const size_t lds = static_cast<size_t>(kStages) * STAGE_BYTES + 2 * P_BYTES + 3 * F_BYTES +
                        (kTblCap + kTblCap / kStep + 2) * sizeof(uint32_t);
     // the kernel also has a few words of static LDS: ask for exactly the dynamic part
-    const bool lists = a.top_k != 0;
+    p.by_pos = a.block_tables != nullptr && a.block_size % kStep != 0 ? 1u : 0u;
+    const bool lists = a.top_k != 0 || p.by_pos != 0;
     const bool few = a.n_heads <= 32;
     const void *kernel = lists ? (few ? reinterpret_cast<const void *>(mla_decode_kernel<true, 1>)
                                       : reinterpret_cast<const void *>(mla_decode_kernel<true, 4>))

@@ -161,6 +161,8 @@ int xlite_hip_decode_step(void *stream, void *qkv, void *k_cache, void *v_cache,
  * the predecessor are ignored); shorter rows see their whole range
  * (xlite/csrc/kernels/mla_v2.h:697-699). The workspace size depends on top_k: pass the
  * call's value to xlite_hip_mla_workspace_bytes. bf16 only (xlite/csrc/op.cpp:1014).
+ * Any block size (kv_lora_rank 512 with rope_head_dim 64: the streaming kernel; other
+ * sizes: a plain kernel).
  * workspace: at least xlite_hip_mla_workspace_bytes() for the same shape (required:
  * XLITE_HIP_ENOSPC otherwise; split-KV partials, no initialisation needed).
  * ---------------------------------------------------------------------- */

@@ -342,3 +342,35 @@ def test_clock_probe_reports_a_plausible_shader_clock_and_switches_off(rt):
     got = run_mla(rt, c, 192 ** -0.5)
     assert torch.equal(got, want)
     assert int(buf.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("bs", [16, 48, 8, 1])
+@pytest.mark.parametrize("nH", [16, 128])
+def test_mla_block_sizes_that_are_not_a_multiple_of_32(rt, bs, nH):
+    """The streaming kernel walks such caches position by position (a step's 32 positions do not share a block):
+    decode rows, prefill rows and a chunked prefill, against the oracle."""
+    if bs == 1:
+        lens, clens = [1, 5, 1], [300, 40, 77]
+    else:
+        lens, clens = [1, 1, 40, 1, 9], [1500, 31, 200, 4099 if nH == 16 else 1100, 0]
+    c = mla_case(91, lens, clens, nH, bs=bs)
+    scale = 192 ** -0.5
+    check(run_mla(rt, c, scale), oracle_mla(c, scale))
+
+
+@pytest.mark.parametrize("bs", [16, 48])
+def test_mla_topk_lists_over_block_sizes_that_are_not_a_multiple_of_32(rt, bs):
+    """Position lists over such caches: rows longer than top_k walk their lists, shorter rows their own positions."""
+    from gvirt_amd._C import mla_attention
+    lens, clens, top_k = [1, 1, 6, 1], [900, 100, 700, 3000], 256
+    c = mla_case(92, lens, clens, 16, bs=bs)
+    scale = 192 ** -0.5
+    topk = _topk_indices(c, top_k, 93)
+    out = torch.zeros(c["T"], c["nH"], c["C"], dtype=torch.bfloat16, device=DEV)
+    mla_attention(rt, c["qa"].to(DEV), c["qr"].to(DEV), c["kc"].to(DEV), c["pc"].to(DEV), out, c["qsl"].to(DEV),
+                  c["lens"].to(DEV), c["clens"].to(DEV), c["tables"].to(DEV), c["nH"], c["R"], c["C"], c["bs"], c["batch"],
+                  c["maxblk"], scale, topk.to(DEV), top_k)
+    rt.synchronize()
+    ref = O.mla_attention_ref(c["qa"], c["qr"], c["kc"], c["pc"], c["qsl"], c["lens"], c["clens"], c["tables"], c["nH"],
+                              c["R"], c["C"], c["bs"], c["batch"], c["maxblk"], scale, topk, top_k)
+    check(out.float().cpu(), ref)
