@@ -23,6 +23,10 @@ size_t workspace_bytes_16(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv
                           uint32_t block_size, uint32_t batch, uint32_t max_num_block)
 {
     const uint32_t max_ctx = max_num_block * block_size;
+    if (is_decode_batch(total_tokens, batch) &&
+        decode_dma256_supported(n_heads, n_kv_heads, head_dim, block_size, XLITE_HIP_KV_SAME)) {
+        return decode_mfma_workspace_bytes(batch, n_heads, head_dim, block_size, max_num_block);
+    }
     if (is_decode_batch(total_tokens, batch) && decode_supported(head_dim)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
             return decode_mfma_workspace_bytes(batch, n_heads, head_dim, block_size, max_num_block);
@@ -175,7 +179,12 @@ static int run_16bit(hipStream_t s, AttentionArgs &a)
     const uint32_t total_tokens = a.total_tokens, n_heads = a.n_heads, n_kv_heads = a.n_kv_heads, head_dim = a.head_dim,
                    block_size = a.block_size, batch = a.batch, max_num_block = a.max_num_block;
     // head_dim 256 (the reference kernel is generic over headSize, xlite/csrc/kernels/attention.h:39-74, and ships
-    // such models): the generic matrix-core kernel serves decode and prefill batches alike
+    // such models): decode batches of up to 16 query heads per kv head stream the cache like head_dim 128 does, a
+    // head as two 256-byte units; the generic matrix-core kernel serves every other batch
+    if (is_decode_batch(total_tokens, batch) &&
+        decode_dma256_supported(n_heads, n_kv_heads, head_dim, block_size, a.kv_dtype)) {
+        return launch_decode_mfma(s, a);
+    }
     if (is_decode_batch(total_tokens, batch) && decode_supported(head_dim)) {
         if (decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
             return launch_decode_mfma(s, a);

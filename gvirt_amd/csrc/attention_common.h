@@ -81,6 +81,7 @@ size_t decode_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t 
 int launch_decode(hipStream_t stream, const AttentionArgs &a, uint32_t tile_tokens);
 
 // decode_mfma.hip
+bool decode_dma256_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size, int kv_dtype);
 bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
                            uint32_t total_tokens);
 struct DecodeSplitPlan {

@@ -902,12 +902,17 @@ __device__ __forceinline__ void dma_wait()
 // NKV: kv heads of a pass. 8, or all of a model's 4, 2 or 1: then 8 / NKV waves share a kv head, a step is
 // 16 positions for each of them (wave w: kv head w % NKV, positions 16 (w / NKV) .. + 15 of the step), and
 // their results meet in the head's first wave at the end of the segment.
-template <typename T, int NKV>
+// HD = 2: head_dim 256. A head is then two adjacent 256-byte units of a cache row, NKV counts units (8, 4 or 2: a
+// model's 4 kv heads per pass, or all of its 2 or 1), and the stage layout and the copies are those of a head_dim-128
+// model with twice the kv heads. The two waves of a head both form its scores over all 256 elements (K rows of both
+// units; the kernel waits for memory, not for the matrix pipe) and each takes the 128 output columns of its own unit.
+template <typename T, int NKV, int HD = 1>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_dma_kernel(const DecodeMfmaParams p)
 {
-    constexpr int D = 128;
-    constexpr int KS = D / 32, MT = D / 16;
+    constexpr int D = 128;                       // elements of a unit
+    constexpr int DT = D * HD;                   // elements of a head
+    constexpr int KS = DT / 32, MT = D / 16;
     constexpr int HEADB = D * 2;                 // bytes of one (position, kv head) row
     constexpr int NSUB = kWaves / NKV;           // 16-position groups of a step
     constexpr int POSB = NKV * HEADB;            // LDS bytes of one position: the kv heads of the pass
@@ -928,11 +933,12 @@ decode_dma_kernel(const DecodeMfmaParams p)
     const uint32_t jq = lane >> 4;
 
     // read roles: this wave's kv head inside the pass and its group of 16 positions inside the step
-    const uint32_t kvl = wave % NKV, sub = wave / NKV;
+    const uint32_t kvl = wave % NKV, sub = wave / NKV;   // (kvl: the wave's unit inside the pass)
+    const uint32_t hsel = kvl / HD, hh = kvl % HD;       // its head inside the pass, and which unit of the head
     uint32_t kr_off[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-        kr_off[ks] = (16 * sub + col) * POSB + kvl * HEADB + (((4 * ks + jq) ^ swizzle<D>(col)) << 4);
+        kr_off[ks] = (16 * sub + col) * POSB + (hsel * HD + ks / 4) * HEADB + (((4 * (ks % 4) + jq) ^ swizzle<D>(col)) << 4);
     }
     uint32_t vr_off[MT];
     {
@@ -960,7 +966,7 @@ decode_dma_kernel(const DecodeMfmaParams p)
     }
 
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
-    const uint32_t row_bytes = p.n_kv_heads * HEADB;
+    const uint32_t row_bytes = p.n_kv_heads * HD * HEADB;
 
     DecodeSplit<> split(p, tbl_lds + kSplitTblCap, lane, wave);
     split.scan();
@@ -980,7 +986,7 @@ decode_dma_kernel(const DecodeMfmaParams p)
             // (every lane loads: columns past the group's heads repeat its last head and are never stored; a load under
             // a per-lane condition is compiled into a branch with a wait of its own, one trip to memory per load)
             const uint16_t *qrow = p.q + static_cast<uint64_t>(tok) * p.q_row_stride +
-                                   static_cast<uint64_t>((kv0 + kvl) * p.group + min(col, g_valid - 1)) * D;
+                                   static_cast<uint64_t>((kv0 / HD + hsel) * p.group + min(col, g_valid - 1)) * DT;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 qreg[ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8);
@@ -998,8 +1004,8 @@ decode_dma_kernel(const DecodeMfmaParams p)
             __syncthreads();
         }
 
-        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += NKV) {
-            const uint32_t kvh = kv0 + kvl;
+        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads * HD; kv0 += NKV) {   // (kv0 counts units)
+            const uint32_t kvh = kv0 / HD + hsel;
             const uint32_t head0 = kvh * p.group;
 
             if (kv0 > 0) {
@@ -1161,7 +1167,7 @@ decode_dma_kernel(const DecodeMfmaParams p)
             if (col < g_valid && sub == 0) {
                 if (whole) {
                     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-                    uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * D;
+                    uint16_t *dst = p.out + (static_cast<uint64_t>(tok) * p.n_heads + head0 + col) * DT + hh * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         uint2 o;
@@ -1171,12 +1177,12 @@ decode_dma_kernel(const DecodeMfmaParams p)
                     }
                 } else {
                     const uint64_t slot = static_cast<uint64_t>(pslot) * p.n_heads + head0 + col;
-                    float *dst = p.part_acc + slot * D;
+                    float *dst = p.part_acc + slot * DT + hh * D;
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         *reinterpret_cast<float4 *>(dst + mt * 16 + jq * 4) = make_float4(O[mt][0], O[mt][1], O[mt][2], O[mt][3]);
                     }
-                    if (jq == 0) {
+                    if (jq == 0 && hh == 0) {
                         *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_tot);
                     }
                 }
@@ -1187,12 +1193,12 @@ decode_dma_kernel(const DecodeMfmaParams p)
     split.for_each_segment(run_segment);
 }
 
-template <typename T, int NKV>
+template <typename T, int NKV, int HD = 1>
 int launch_dma_nkv(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
 {
     const size_t lds = 2 * static_cast<size_t>(2 * kStep * kWaves * 128 * 2) +
                        (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
-    auto kernel = decode_dma_kernel<T, NKV>;
+    auto kernel = decode_dma_kernel<T, NKV, HD>;
     if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
         return rc;
     }
@@ -1200,6 +1206,16 @@ int launch_dma_nkv(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_wor
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
+}
+// head_dim 256: the units of a cache row are twice the kv heads
+template <typename T>
+int launch_dma256(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
+{
+    switch (p.n_kv_heads) {
+    case 1: return launch_dma_nkv<T, 2, 2>(stream, p, n_workgroups);
+    case 2: return launch_dma_nkv<T, 4, 2>(stream, p, n_workgroups);
+    default: return launch_dma_nkv<T, 8, 2>(stream, p, n_workgroups);
+    }
 }
 template <typename T>
 int launch_dma(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgroups)
@@ -1728,6 +1744,14 @@ int launch_fmt(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x, i
 
 }  // namespace
 
+// head_dim 256 over a 16-bit cache: the direct-to-LDS kernel with two units per head (4 kv heads per pass, or a
+// model's 2 or 1)
+bool decode_dma256_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size, int kv_dtype)
+{
+    return head_dim == 256 && kv_dtype == XLITE_HIP_KV_SAME && block_size % kStep == 0 && n_kv_heads > 0 &&
+           n_heads / n_kv_heads <= 16 && (n_kv_heads % 4 == 0 || n_kv_heads == 2 || n_kv_heads == 1);
+}
+
 bool decode_mfma_supported(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
                            uint32_t total_tokens)
 {
@@ -1832,7 +1856,7 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     // step is bound by its launches: Qwen2-0.5B, 4 sequences of up to 512 positions, 12.7 us + 3.9 us of merge -> one
     // kernel.
     const uint32_t waves_per_kv = a.n_kv_heads >= kWaves ? 1u : kWaves / a.n_kv_heads;
-    const bool whole_rows = !p.only_single && a.kv_dtype == XLITE_HIP_KV_SAME &&
+    const bool whole_rows = !p.only_single && a.kv_dtype == XLITE_HIP_KV_SAME && a.head_dim != 256 &&
                             ceil_div(static_cast<uint64_t>(a.max_num_block) * a.block_size, static_cast<uint64_t>(kStep)) <=
                                 16ull * waves_per_kv &&
                             a.max_num_block <= kSplitTblCap - 2;
@@ -1848,6 +1872,11 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
         if (whole_rows) {   // (the register-staged kernel, whatever the shape: these contexts are a few steps long)
             rc = a.head_dim == 128 ? (bf ? launch_whole<BF16, 128>(stream, p, gx) : launch_whole<FP16, 128>(stream, p, gx))
                                    : (bf ? launch_whole<BF16, 64>(stream, p, gx) : launch_whole<FP16, 64>(stream, p, gx));
+        } else if (a.head_dim == 256) {
+            XL_REQUIRE(decode_dma256_supported(a.n_heads, a.n_kv_heads, a.head_dim, a.block_size, a.kv_dtype),
+                       "head_dim 256: shape not served by the streaming decode kernel");
+            p.step_mult = 2 * a.n_kv_heads < kWaves ? kWaves / (2 * a.n_kv_heads) : 1;
+            rc = bf ? launch_dma256<BF16>(stream, p, gx) : launch_dma256<FP16>(stream, p, gx);
         } else if (decode_dma_supported(a.n_kv_heads, a.head_dim, a.kv_dtype)) {
             p.step_mult = a.n_kv_heads < kWaves ? kWaves / a.n_kv_heads : 1;
             rc = bf ? launch_dma<BF16>(stream, p, gx) : launch_dma<FP16>(stream, p, gx);

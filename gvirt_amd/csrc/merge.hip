@@ -296,7 +296,7 @@ merge_meta_kernel(uint16_t *__restrict__ out, const float *__restrict__ part_acc
         const uint32_t ps = s == 0 ? 2 * c0 + (1 - first_flag) : 2 * (c0 + s);
         return static_cast<uint64_t>(ps) * n_heads + head;
     };
-    const uint32_t lanes_per = dv / 4;                 // 16 or 32
+    const uint32_t lanes_per = dv / 4;                 // 16, 32 or 64
     const uint32_t c = lane % lanes_per;
     const uint32_t streams = 64 / lanes_per * WPR;     // slots summed side by side
     const uint32_t stream = (wave % WPR) * (64 / lanes_per) + lane / lanes_per;
@@ -494,8 +494,8 @@ int launch_merge_meta(hipStream_t stream, int dtype, void *out, const float *acc
     if (rows == 0) {
         return XLITE_HIP_OK;
     }
-    if (dv != 64 && dv != 128) {
-        return fail(XLITE_HIP_EINVAL, __func__, "value width " + std::to_string(dv) + " is neither 64 nor 128");
+    if (dv != 64 && dv != 128 && dv != 256) {
+        return fail(XLITE_HIP_EINVAL, __func__, "value width " + std::to_string(dv) + " is none of 64, 128, 256");
     }
     const uint64_t total_rh = static_cast<uint64_t>(rows) * n_heads;
     const int4 *m4 = reinterpret_cast<const int4 *>(meta);

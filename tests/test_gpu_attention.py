@@ -569,6 +569,22 @@ def test_head_dim_256_split_decode_and_chunked_prefill(rt, bs):
     check(run_attention(rt, w), oracle_attention(w))
 
 
+@pytest.mark.parametrize("heads", [(4, 1), (16, 1), (6, 2), (16, 4), (32, 8), (36, 12), (5, 5)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_dim_256_decode_batches_of_every_kv_head_count(rt, heads, dtype):
+    """head_dim-256 decode batches stream the cache with a head as two 256-byte units: one, two, four kv heads per
+    pass, several passes (8 and 12 kv heads), groups that fill and do not fill the 16 columns; 5 kv heads is a count
+    the streaming kernel does not take and runs through the generic one. Contexts from one position to several
+    chunks, with and without a remainder of a step; narrow block tables (no split) and wide ones."""
+    nH, nKV = heads
+    ctx = [1, 15, 16, 17, 31, 33, 64, 100, 127, 128, 129, 255, 300]
+    w = generic_case(84, [1] * len(ctx), [c - 1 for c in ctx], nH, nKV, 256, 16, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+    ctx = [6000, 1, 2049, 700, 0, 4096]
+    w = generic_case(85, [1 if c else 0 for c in ctx], [max(c - 1, 0) for c in ctx], nH, nKV, 256, 64, dtype, rms=True)
+    check(run_attention(rt, w), oracle_attention(w))
+
+
 def test_head_dim_256_quantised_cache_is_refused(rt):
     w = generic_case(83, [1], [100], 8, 2, 256, 128, torch.bfloat16)
     kq, ks = O.quantize_kv_int8(w["k_cache"].float())
