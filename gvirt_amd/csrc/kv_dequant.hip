@@ -48,8 +48,13 @@ __device__ __forceinline__ uint4 dequant8(const uint2 &raw, float scale)
     return make_uint4(T::pack(x[0], x[1]), T::pack(x[2], x[3]), T::pack(x[4], x[5]), T::pack(x[6], x[7]));
 }
 
-// workgroup (x = block j of the sequence, y = sequence, z = K | V): block j of sequence i lands at block
-// i * max_num_block + j of the compact cache; blocks beyond the sequence's visible range are skipped.
+// workgroup (x = block j of the sequence and a part of it, y = sequence, z = K | V): block j of sequence i lands at
+// block i * max_num_block + j of the compact cache; blocks beyond the sequence's visible range are skipped. A part is
+// kDequantPart 16-byte chunks: a thread takes four of them, 256 apart, with their loads (bytes and scales) all in
+// flight before the first conversion.
+constexpr uint32_t kDequantUnroll = 4;
+constexpr uint32_t kDequantPart = 256 * kDequantUnroll;
+
 template <typename T, int KVF>
 __global__ void __launch_bounds__(256)
 dequant_blocks_kernel(const unsigned char *__restrict__ k_cache, const unsigned char *__restrict__ v_cache,
@@ -57,38 +62,53 @@ dequant_blocks_kernel(const unsigned char *__restrict__ k_cache, const unsigned 
                       const int32_t *__restrict__ block_tables, const int32_t *__restrict__ lens,
                       const int32_t *__restrict__ cached_lens, uint16_t *__restrict__ k_out, uint16_t *__restrict__ v_out,
                       int32_t *__restrict__ table_out, uint32_t block_size, uint32_t max_num_block, uint32_t n_kv_heads,
-                      uint32_t head_dim, uint32_t skip_single)
+                      uint32_t head_dim, uint32_t parts, uint32_t skip_single)
 {
-    const uint32_t j = blockIdx.x, i = blockIdx.y;
+    const uint32_t j = blockIdx.x / parts, part = blockIdx.x % parts, i = blockIdx.y;
     const bool is_v = blockIdx.z != 0;
     const uint64_t out_block = static_cast<uint64_t>(i) * max_num_block + j;
-    if (!is_v && threadIdx.x == 0) {
+    const int32_t n_rows = lens[i], n_cached = cached_lens[i];
+    const uint64_t phys = static_cast<uint32_t>(block_tables[out_block]);
+    if (!is_v && part == 0 && threadIdx.x == 0) {
         table_out[out_block] = static_cast<int32_t>(out_block);
     }
     // sequences without rows need nothing; with skip_single those with one row read the bytes themselves
-    const int32_t visible = lens[i] > 0 && !(skip_single && lens[i] == 1) ? cached_lens[i] + lens[i] : 0;
+    const int32_t visible = n_rows > 0 && !(skip_single && n_rows == 1) ? n_cached + n_rows : 0;
     if (static_cast<int64_t>(j) * block_size >= visible) {
         return;
     }
     const uint32_t rows_here = min(block_size, static_cast<uint32_t>(visible) - j * block_size);   // positions of the block
-    const uint64_t phys = static_cast<uint32_t>(block_tables[out_block]);
     const uint32_t cpr = head_dim / 16;                              // 16-element chunks per (position, kv head) row
-    const uint64_t chunks = static_cast<uint64_t>(rows_here) * n_kv_heads * cpr;
+    const uint32_t chunks = rows_here * n_kv_heads * cpr;            // (a block is well below 2^32 chunks)
+    const uint32_t all_chunks = block_size * n_kv_heads * cpr;
     const unsigned char *src = (is_v ? v_cache : k_cache) + phys * block_size * n_kv_heads * head_dim;
     const float *sc = (is_v ? v_scale : k_scale) + phys * block_size * n_kv_heads;
     uint16_t *dst = (is_v ? v_out : k_out) + out_block * block_size * n_kv_heads * head_dim;
-    for (uint64_t c = threadIdx.x; c < chunks; c += blockDim.x) {
-        const uint4 raw = *reinterpret_cast<const uint4 *>(src + c * 16);
-        const float scale = sc[c / cpr];
-        *reinterpret_cast<uint4 *>(dst + c * 16) = dequant8<T, KVF>(make_uint2(raw.x, raw.y), scale);
-        *reinterpret_cast<uint4 *>(dst + c * 16 + 8) = dequant8<T, KVF>(make_uint2(raw.z, raw.w), scale);
+    const uint32_t c0 = part * kDequantPart + threadIdx.x;
+    // (every load is issued, from a clamped address: a load under a condition is compiled into a branch with a wait
+    // of its own)
+    uint4 raw[kDequantUnroll];
+    float scale[kDequantUnroll];
+#pragma unroll
+    for (uint32_t u = 0; u < kDequantUnroll; u++) {
+        const uint32_t c = min(c0 + u * 256, chunks - 1);
+        typedef uint32_t words_t __attribute__((ext_vector_type(4)));
+        const words_t w = __builtin_nontemporal_load(reinterpret_cast<const words_t *>(src + static_cast<uint64_t>(c) * 16));
+        raw[u] = make_uint4(w[0], w[1], w[2], w[3]);
+        scale[u] = sc[c / cpr];
     }
-    // the rest of a partly visible block: zeros (the 16-bit kernels may load whole tiles and give the positions
-    // past the end probability zero, which stale workspace bits that read as NaN would turn into NaN)
-    const uint64_t all_chunks = static_cast<uint64_t>(block_size) * n_kv_heads * cpr;
-    for (uint64_t c = chunks + threadIdx.x; c < all_chunks; c += blockDim.x) {
-        *reinterpret_cast<uint4 *>(dst + c * 16) = make_uint4(0, 0, 0, 0);
-        *reinterpret_cast<uint4 *>(dst + c * 16 + 8) = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (uint32_t u = 0; u < kDequantUnroll; u++) {
+        const uint32_t c = c0 + u * 256;
+        if (c < chunks) {
+            *reinterpret_cast<uint4 *>(dst + static_cast<uint64_t>(c) * 16) = dequant8<T, KVF>(make_uint2(raw[u].x, raw[u].y), scale[u]);
+            *reinterpret_cast<uint4 *>(dst + static_cast<uint64_t>(c) * 16 + 8) = dequant8<T, KVF>(make_uint2(raw[u].z, raw[u].w), scale[u]);
+        } else if (c < all_chunks) {
+            // the rest of a partly visible block: zeros (the 16-bit kernels may load whole tiles and give the positions
+            // past the end probability zero, which stale workspace bits that read as NaN would turn into NaN)
+            *reinterpret_cast<uint4 *>(dst + static_cast<uint64_t>(c) * 16) = make_uint4(0, 0, 0, 0);
+            *reinterpret_cast<uint4 *>(dst + static_cast<uint64_t>(c) * 16 + 8) = make_uint4(0, 0, 0, 0);
+        }
     }
 }
 
@@ -163,14 +183,18 @@ int launch_kv_dequant(hipStream_t stream, AttentionArgs *a)
     uint16_t *k_out = reinterpret_cast<uint16_t *>(ws);
     uint16_t *v_out = reinterpret_cast<uint16_t *>(ws + l.cache_bytes);
     int32_t *table = reinterpret_cast<int32_t *>(ws + 2 * l.cache_bytes);
-    const dim3 grid(a->max_num_block, a->batch, 2);
+    const uint64_t block_chunks = static_cast<uint64_t>(a->block_size) * a->n_kv_heads * (a->head_dim / 16);
+    XL_REQUIRE(block_chunks < (1ull << 31), "a cache block of more than 2^31 16-byte chunks");
+    const uint32_t parts = static_cast<uint32_t>((block_chunks + kDequantPart - 1) / kDequantPart);
+    XL_REQUIRE(static_cast<uint64_t>(a->max_num_block) * parts < (1ull << 31), "block tables too wide for the dequantising copy");
+    const dim3 grid(a->max_num_block * parts, a->batch, 2);
     XL_REQUIRE(a->batch <= 65535, "more than 65535 sequences over a quantised cache outside the decode kernels");
     auto launch = [&](auto tag, auto kv) {
         using T = decltype(tag);
         dequant_blocks_kernel<T, decltype(kv)::value><<<grid, 256, 0, stream>>>(
             static_cast<const unsigned char *>(a->k_cache), static_cast<const unsigned char *>(a->v_cache), a->k_scale,
             a->v_scale, a->block_tables, a->lens, a->cached_lens, k_out, v_out, table, a->block_size, a->max_num_block,
-            a->n_kv_heads, a->head_dim, a->rows_mode == kSkipSingle ? 1u : 0u);
+            a->n_kv_heads, a->head_dim, parts, a->rows_mode == kSkipSingle ? 1u : 0u);
     };
     using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
     using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;
