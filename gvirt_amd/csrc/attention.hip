@@ -1,5 +1,6 @@
 // C entry points of the attention operators: argument checks and kernel selection.
 #include "attention_common.h"
+#include "rope_item.h"
 
 using namespace xlite;
 
@@ -228,7 +229,27 @@ extern "C" int xlite_hip_decode_step(void *stream, void *qkv, void *k_cache, voi
                                      uint32_t max_num_block, int is_neox, uint64_t mrope_mask_h,
                                      uint64_t mrope_mask_w, int dtype, void *workspace, size_t workspace_bytes)
 {
-    // the two calls of a layer's attention block, enqueued back to back on the caller's stream
+    // Decode batches that the decode kernel takes as whole rows (contexts that are short by the width of the block
+    // tables: such a step is bound by its launches): one launch, the kernel rotates and stores the rows itself. The
+    // arguments are checked as the two calls check them.
+    if (total_tokens != 0 && batch != 0 && qkv && k_cache && v_cache && output && query_start_loc && lens && cached_lens &&
+        block_tables && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && block_size > 0 && max_num_block > 0 &&
+        (dtype == XLITE_HIP_FP16 || dtype == XLITE_HIP_BF16) && is_decode_batch(total_tokens, batch) &&
+        decode_supported(head_dim) && decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, total_tokens)) {
+        AttentionArgs a{qkv, k_cache, v_cache, output, query_start_loc, lens, cached_lens, block_tables,
+                        total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
+                        dtype, XLITE_HIP_KV_SAME, nullptr, nullptr, workspace, workspace_bytes};
+        if (decode_mfma_whole_rows(a)) {
+            RopeArgs rope{};
+            if (const int rc = rope_prepare(qkv, k_cache, v_cache, position, cosin, slot_mapping, total_tokens, n_heads,
+                                            n_kv_heads, head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w,
+                                            dtype, true, &rope)) {
+                return rc;
+            }
+            return launch_decode_mfma(as_stream(stream), a, &rope);
+        }
+    }
+    // otherwise the two calls of a layer's attention block, enqueued back to back on the caller's stream
     if (const int rc = xlite_hip_rope_and_cache(stream, qkv, k_cache, v_cache, position, cosin, slot_mapping, total_tokens,
                                                 n_heads, n_kv_heads, head_dim, rot_dim, block_size, is_neox, mrope_mask_h,
                                                 mrope_mask_w, dtype)) {

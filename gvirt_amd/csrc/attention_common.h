@@ -90,7 +90,11 @@ struct DecodeSplitPlan {
 };
 size_t decode_mfma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t head_dim, uint32_t block_size,
                                    uint32_t max_num_block);
-int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a);
+// `rope`: the batch's rope_and_cache arguments, for a batch that decode_mfma_whole_rows accepts: the kernel then
+// rotates and stores the rows itself
+struct RopeArgs;
+bool decode_mfma_whole_rows(const AttentionArgs &a);
+int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a, const RopeArgs *rope = nullptr);
 uint32_t decode_mfma_slice_units();   // units (rows, sequences) one launch of the decode kernels can split
 
 // mla_decode.hip

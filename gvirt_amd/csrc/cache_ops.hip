@@ -1,63 +1,9 @@
 // Paged KV-cache writers and gathers: rope_and_cache, gather_sparse_kv_cache, rope_complex,
 // mla_prepare, int8 quantisation. All are HBM-bound copy/elementwise kernels: every thread
 // moves 16-byte vectors, adjacent lanes touch adjacent addresses.
-#include "common.h"
+#include "rope_item.h"
 
 namespace xlite {
-
-union Vec16 {
-    uint4 v;
-    uint16_t h[8];
-    uint32_t w[4];
-};
-
-// One chunk pair of a q or k head: elements e0 .. e0+7 of the rotary span's first half (`a`) with their partners
-// in the second half (`b`), rotated in place; q is then scaled. Rounding follows calc_cossin_cast
-// (xlite/csrc/kernels/rope_and_cache.h:93-129): each product is rounded to the storage type, the difference /
-// sum is formed in fp32 and rounded again; the q scale is applied in fp32 and rounded once more (:576-586).
-template <typename T>
-__device__ __forceinline__ void rotate_chunk_pair(Vec16 &a, Vec16 &b, uint32_t e0, uint32_t half, uint32_t t, int64_t pos_t,
-                                                  uint32_t num_tokens, uint32_t rot_dim, const int64_t *position,
-                                                  const uint16_t *cosin, uint64_t mask_h, uint64_t mask_w, bool is_q,
-                                                  float q_scale)
-{
-    Vec16 c, s;
-    if ((mask_h | mask_w) == 0) {
-        const uint16_t *cs = cosin + static_cast<uint64_t>(pos_t) * rot_dim;
-        c.v = *reinterpret_cast<const uint4 *>(cs + e0);
-        s.v = *reinterpret_cast<const uint4 *>(cs + half + e0);
-    } else {
-        // lane j of the rotary half takes its angle from the height / width position
-        // when bit j of the matching mask is set, else from the temporal position
-        const uint16_t *cs_t = cosin + static_cast<uint64_t>(pos_t) * rot_dim;
-        const uint16_t *cs_h = cosin + static_cast<uint64_t>(position[num_tokens + t]) * rot_dim;
-        const uint16_t *cs_w = cosin + static_cast<uint64_t>(position[2ull * num_tokens + t]) * rot_dim;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t lane = e0 + j;
-            const uint16_t *src = ((mask_h >> lane) & 1) ? cs_h : ((mask_w >> lane) & 1) ? cs_w : cs_t;
-            c.h[j] = src[lane];
-            s.h[j] = src[half + lane];
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float x1 = T::to_f32(a.h[j]), x2 = T::to_f32(b.h[j]);
-        const float cc = T::to_f32(c.h[j]), ss = T::to_f32(s.h[j]);
-        const float p1 = T::to_f32(T::from_f32(x1 * cc));
-        const float p2 = T::to_f32(T::from_f32(x2 * ss));
-        const float p3 = T::to_f32(T::from_f32(x2 * cc));
-        const float p4 = T::to_f32(T::from_f32(x1 * ss));
-        uint16_t o1 = T::from_f32(p1 - p2);
-        uint16_t o2 = T::from_f32(p3 + p4);
-        if (is_q) {
-            o1 = T::from_f32(T::to_f32(o1) * q_scale);
-            o2 = T::from_f32(T::to_f32(o2) * q_scale);
-        }
-        a.h[j] = o1;
-        b.h[j] = o2;
-    }
-}
 
 // ---------------------------------------------------------------------------------------
 // rope_and_cache (xlite/csrc/kernels/rope_and_cache.h:206-610)
@@ -70,71 +16,13 @@ __device__ __forceinline__ void rotate_chunk_pair(Vec16 &a, Vec16 &b, uint32_t e
 // ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
-rope_and_cache_kernel(uint16_t *__restrict__ inout, uint16_t *__restrict__ k_cache,
-                      uint16_t *__restrict__ v_cache, const int64_t *__restrict__ position,
-                      const uint16_t *__restrict__ cosin, const int32_t *__restrict__ slot_mapping,
-                      uint32_t num_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
-                      uint32_t rot_dim, uint32_t block_size, float q_scale, uint64_t mask_h,
-                      uint64_t mask_w)
+rope_and_cache_kernel(const RopeArgs r)
 {
-    const uint32_t chunks = head_dim / 8;       // 16-byte chunks per head
-    const uint32_t rot_pairs = rot_dim / 16;    // chunk pairs inside the rotary span
-    const uint32_t items_per_head = chunks - rot_pairs;
-    const uint32_t slots = n_heads + 2 * n_kv_heads;
-    const uint32_t items_per_token = slots * items_per_head;
-    const uint64_t total = static_cast<uint64_t>(num_tokens) * items_per_token;
-    const uint32_t half = rot_dim / 2;
-
+    const uint32_t items_per_token = rope_items_per_token(r);
+    const uint64_t total = static_cast<uint64_t>(r.num_tokens) * items_per_token;
     for (uint64_t idx = blockIdx.x * static_cast<uint64_t>(blockDim.x) + threadIdx.x; idx < total;
          idx += static_cast<uint64_t>(gridDim.x) * blockDim.x) {
-        const uint32_t t = static_cast<uint32_t>(idx / items_per_token);
-        const uint32_t rem = static_cast<uint32_t>(idx % items_per_token);
-        const uint32_t hs = rem / items_per_head;
-        const uint32_t item = rem % items_per_head;
-        uint16_t *row = inout + (static_cast<uint64_t>(t) * slots + hs) * head_dim;
-
-        const bool is_q = hs < n_heads;
-        const bool is_k = !is_q && hs < n_heads + n_kv_heads;
-        // the token's position and slot are requested together with its row (every thread loads both: under a
-        // condition each would be a trip to memory of its own); only the cos / sin row waits for the position
-        const int64_t pos_t = position[t];
-        const uint32_t slot = static_cast<uint32_t>(slot_mapping[t]);
-        const uint32_t e_first = item < rot_pairs ? item * 8 : (item + rot_pairs) * 8;
-        Vec16 a, b;
-        a.v = *reinterpret_cast<const uint4 *>(row + e_first);
-        b.v = *reinterpret_cast<const uint4 *>(row + (item < rot_pairs ? e_first + half : e_first));
-        uint16_t *cache_row = nullptr;
-        if (!is_q && k_cache != nullptr) {   // no 16-bit caches: the caller quantises the rows afterwards
-            const uint32_t kvh = is_k ? hs - n_heads : hs - n_heads - n_kv_heads;
-            const uint64_t off =
-                ((static_cast<uint64_t>(slot / block_size) * block_size + slot % block_size) * n_kv_heads +
-                 kvh) * head_dim;
-            cache_row = (is_k ? k_cache : v_cache) + off;
-        }
-
-        if (item < rot_pairs) {
-            const uint32_t e0 = item * 8;  // first-half elements e0..e0+7, partners at +half
-            if (is_q || is_k) {
-                rotate_chunk_pair<T>(a, b, e0, half, t, pos_t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
-                *reinterpret_cast<uint4 *>(row + e0) = a.v;
-                *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
-            }
-            if (cache_row) {
-                *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
-                *reinterpret_cast<uint4 *>(cache_row + e0 + half) = b.v;
-            }
-        } else {
-            const uint32_t e0 = (item + rot_pairs) * 8;  // beyond the rotary span
-            if (is_q) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    a.h[j] = T::from_f32(T::to_f32(a.h[j]) * q_scale);
-                }
-                *reinterpret_cast<uint4 *>(row + e0) = a.v;
-            } else if (cache_row) {
-                *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
-            }
-        }
+        rope_item<T>(r, static_cast<uint32_t>(idx / items_per_token), static_cast<uint32_t>(idx % items_per_token));
     }
 }
 
@@ -597,31 +485,60 @@ static int rope_check(const void *inout, const int64_t *position, const void *co
     return XLITE_HIP_OK;
 }
 
-// Launch of the rope kernel; with `with_cache` false the 16-bit caches are not written.
-static int rope_launch(void *stream, void *inout, void *k_cache, void *v_cache, const int64_t *position,
-                       const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads,
-                       uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, int is_neox,
-                       uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, bool with_cache)
+// Checks the arguments of a rope_and_cache call and gathers them for the kernels (`with_cache` false: the 16-bit caches
+// are not written).
+int xlite::rope_prepare(void *inout, void *k_cache, void *v_cache, const int64_t *position, const void *cosin,
+                        const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads, uint32_t n_kv_heads,
+                        uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, int is_neox, uint64_t mrope_mask_h,
+                        uint64_t mrope_mask_w, int dtype, bool with_cache, RopeArgs *out)
 {
     float scale = 0.f;
     if (const int rc = rope_check(inout, position, cosin, slot_mapping, num_tokens, n_heads, n_kv_heads, head_dim, rot_dim,
                                   block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype, &scale)) {
         return rc;
     }
+    XL_REQUIRE(num_tokens == 0 || !with_cache || (k_cache && v_cache), "null tensor");
+    RopeArgs r{};
+    r.inout = static_cast<uint16_t *>(inout);
+    r.k_cache = with_cache ? static_cast<uint16_t *>(k_cache) : nullptr;
+    r.v_cache = with_cache ? static_cast<uint16_t *>(v_cache) : nullptr;
+    r.position = position;
+    r.cosin = static_cast<const uint16_t *>(cosin);
+    r.slot_mapping = slot_mapping;
+    r.num_tokens = num_tokens;
+    r.n_heads = n_heads;
+    r.n_kv_heads = n_kv_heads;
+    r.head_dim = head_dim;
+    r.rot_dim = rot_dim;
+    r.block_size = block_size;
+    r.q_scale = scale;
+    r.mask_h = mrope_mask_h;
+    r.mask_w = mrope_mask_w;
+    *out = r;
+    return XLITE_HIP_OK;
+}
+
+// Launch of the rope kernel; with `with_cache` false the 16-bit caches are not written.
+static int rope_launch(void *stream, void *inout, void *k_cache, void *v_cache, const int64_t *position,
+                       const void *cosin, const int32_t *slot_mapping, uint32_t num_tokens, uint32_t n_heads,
+                       uint32_t n_kv_heads, uint32_t head_dim, uint32_t rot_dim, uint32_t block_size, int is_neox,
+                       uint64_t mrope_mask_h, uint64_t mrope_mask_w, int dtype, bool with_cache)
+{
+    RopeArgs r{};
+    if (const int rc = rope_prepare(inout, k_cache, v_cache, position, cosin, slot_mapping, num_tokens, n_heads, n_kv_heads,
+                                    head_dim, rot_dim, block_size, is_neox, mrope_mask_h, mrope_mask_w, dtype, with_cache,
+                                    &r)) {
+        return rc;
+    }
     if (num_tokens == 0) {
         return XLITE_HIP_OK;
     }
-    XL_REQUIRE(!with_cache || (k_cache && v_cache), "null tensor");
     const uint64_t items = static_cast<uint64_t>(num_tokens) * (n_heads + 2 * n_kv_heads) *
                            (head_dim / 8 - rot_dim / 16);
     const uint32_t grid = grid_for(items, 256);
     auto launch = [&](auto tag) {
         using T = decltype(tag);
-        rope_and_cache_kernel<T><<<grid, 256, 0, as_stream(stream)>>>(
-            static_cast<uint16_t *>(inout), with_cache ? static_cast<uint16_t *>(k_cache) : nullptr,
-            with_cache ? static_cast<uint16_t *>(v_cache) : nullptr, position, static_cast<const uint16_t *>(cosin),
-            slot_mapping, num_tokens, n_heads, n_kv_heads, head_dim, rot_dim, block_size, scale,
-            mrope_mask_h, mrope_mask_w);
+        rope_and_cache_kernel<T><<<grid, 256, 0, as_stream(stream)>>>(r);
     };
     if (dtype == XLITE_HIP_BF16) {
         launch(BF16{});

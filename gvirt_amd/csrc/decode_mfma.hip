@@ -24,6 +24,7 @@
 // step every sequence has one, but sequences without rows and sequences with several (row r sees
 // cached + r + 1 positions) are served alike.
 #include "attention_common.h"
+#include "rope_item.h"
 
 namespace xlite {
 
@@ -91,6 +92,8 @@ struct DecodeMfmaParams {
     uint32_t step_mult;    // steps (of 16 positions) the kernel takes at a time: chunks are multiples of it
     uint32_t block_magic;  // floor(2^32 / block_size) + 1: position / block_size == mulhi(position, magic) for positions
                            // below 2^32 / block_size; 0 when a table reaches further (then the kernels divide)
+    uint32_t kv_per_wg;    // whole rows: kv heads of a workgroup (all of them, or 1 with n_sub = 8); blockIdx.y counts the groups
+    RopeArgs rope;         // the whole-row kernel that rotates and stores the step's rows itself: that call's arguments
 };
 
 // block and offset inside it of position t (a division by a run-time block size is some twenty instructions)
@@ -206,7 +209,8 @@ __device__ __forceinline__ uint32_t uni(uint32_t x)
 // WHOLE: no split - workgroup i walks the whole range of the rows i, i + grid, ...: nothing to merge (a template
 // parameter, so that each kernel has one call site for its segment body: a second copy of that body, or the extra live
 // values of a run-time choice, cost the streaming kernels 4 %)
-template <bool WHOLE = false>
+// ROPE (with WHOLE): the units are the sequences; `before_rows(first row, rows)` runs ahead of a sequence's rows.
+template <bool WHOLE = false, bool ROPE = false>
 struct DecodeSplit {
     const DecodeMfmaParams &p;
     uint32_t *wave_tot, *pref;   // LDS: kWaves words, units + 1 words
@@ -394,10 +398,28 @@ struct DecodeSplit {
         return in_lanes ? uni(__shfl(ln_tok, static_cast<int>(unit))) : uni(static_cast<uint32_t>(p.query_start_loc[uni(unit + p.unit0)]));
     }
     // segment(seq, row, t0, t1, whole, partial slot, first piece of its row, meta of the row)
-    template <typename F>
-    __device__ __forceinline__ void for_each_segment(F &&segment) const
+    struct NoPrologue {
+        __device__ __forceinline__ void operator()(uint32_t, uint32_t) const {}
+    };
+    template <typename F, typename G = NoPrologue>
+    __device__ __forceinline__ void for_each_segment(F &&segment, G &&before_rows = G()) const
     {
-        if constexpr (WHOLE) {
+        if constexpr (WHOLE && ROPE) {
+            // by sequence: the rows of a sequence see each other's new cache rows, so one workgroup writes them all
+            // before it walks any (a plain decode step has one row per sequence)
+            for (uint32_t s = blockIdx.x; s < p.batch; s += gridDim.x) {
+                const int32_t start = p.query_start_loc[s], ql = p.lens[s], cached = p.cached_lens[s];
+                if (ql <= 0) {
+                    continue;
+                }
+                before_rows(uni(static_cast<uint32_t>(start)), uni(static_cast<uint32_t>(ql)));
+                for (int32_t r = 0; r < ql; r++) {
+                    const int32_t lim = cached + r + 1;
+                    segment(uni(s), uni(static_cast<uint32_t>(start + r)), 0u, uni(static_cast<uint32_t>(lim > 1 ? lim : 1)), true,
+                            0u, false, make_int4(0, 0, 0, 0));
+                }
+            }
+        } else if constexpr (WHOLE) {
             // batches whose contexts are short by the width of their block tables: a row is one segment, stored
             // directly, and there is no second launch to merge anything (a step of such a batch is bound by its
             // launches, not by its bytes)
@@ -434,7 +456,10 @@ struct DecodeSplit {
     }
 };
 
-template <typename T, int D, int KVF, bool MULTI_SUB, bool WHOLE = false>
+// ROPE (whole rows over a 16-bit cache): the kernel is a layer's rope_and_cache and attention in one launch. The
+// workgroup of a sequence rotates the sequence's new rows in place and stores their k and v in the cache (the items of
+// rope_and_cache, spread over its 512 threads), and walks the rows behind a barrier: a workgroup sees its own stores.
+template <typename T, int D, int KVF, bool MULTI_SUB, bool WHOLE = false, bool ROPE = false>
 __global__ void __launch_bounds__(kWaves * 64)
 decode_mfma_kernel(const DecodeMfmaParams p)
 {
@@ -514,6 +539,13 @@ decode_mfma_kernel(const DecodeMfmaParams p)
     const gvec_t *vc = static_cast<const gvec_t *>(p.v_cache);
     const uint32_t g_valid = p.group < 16 ? p.group : 16;
     const uint32_t my_kvl = wave & (kvw - 1), my_sub = wave >> kvw_shift;
+    // the workgroup's kv heads: all of them, or (whole rows of a batch that leaves compute units idle) one group of
+    // kv_per_wg per workgroup - heads are independent, so rows cut this way still need no merge
+    uint32_t kv_begin = 0, kv_end = p.n_kv_heads;
+    if constexpr (WHOLE) {
+        kv_begin = blockIdx.y * p.kv_per_wg;
+        kv_end = min(p.n_kv_heads, kv_begin + p.kv_per_wg);
+    }
 
     // one segment: positions [t0, t1) of the row `tok` of sequence `seq`. `single`: the result is final;
     // otherwise it goes to partial slot `pslot`. With fewer than 8 kv heads the waves of a kv head take equal
@@ -542,7 +574,7 @@ decode_mfma_kernel(const DecodeMfmaParams p)
                 qreg[ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 32 + jq * 8);
             }
         };
-        request_q(0);
+        request_q(kv_begin);
         {
             const uint32_t nblk = (t1 - 1) / p.block_size - blk0 + 1;
             for (uint32_t i = threadIdx.x; i < nblk; i += NT) {
@@ -555,13 +587,13 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         }
 
         // passes over groups of `kvw` kv heads
-        for (uint32_t kv0 = 0; kv0 < p.n_kv_heads; kv0 += kvw) {
+        for (uint32_t kv0 = kv_begin; kv0 < kv_end; kv0 += kvw) {
             const uint32_t kvh = kv0 + my_kvl;
-            const bool kv_ok = kvh < p.n_kv_heads;
+            const bool kv_ok = kvh < kv_end;
             const uint32_t head0 = kvh * p.group;
 
             {
-                if (kv0 != 0) {
+                if (kv0 != kv_begin) {
                     request_q(kv0);
                 }
 #pragma unroll
@@ -868,12 +900,30 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         __syncthreads();   // tbl_lds and the stages are rewritten by the next segment
     };
 
-    DecodeSplit<WHOLE> split(p, tbl_lds + kSplitTblCap, lane, wave, !(MULTI_SUB && D == 128));
+    DecodeSplit<WHOLE, ROPE> split(p, tbl_lds + kSplitTblCap, lane, wave, !(MULTI_SUB && D == 128));
     split.scan();
     if (split.total == 0) {
         return;
     }
-    split.for_each_segment(run_segment);
+    if constexpr (ROPE) {
+        static_assert(WHOLE && !KV8, "the kernel rotates rows only when it takes them whole, over a 16-bit cache");
+        // the head slots of the workgroup's kv heads: their query heads, then their k rows, then their v rows
+        const uint32_t per_head = p.rope.head_dim / 8 - p.rope.rot_dim / 16;
+        const uint32_t kvn = kv_end - kv_begin, nq = kvn * p.group;
+        const uint32_t per_row = (nq + 2 * kvn) * per_head;
+        split.for_each_segment(run_segment, [&](uint32_t row0, uint32_t rows) {
+            for (uint32_t i = threadIdx.x; i < rows * per_row; i += NT) {
+                const uint32_t row = i / per_row, j = i % per_row, jh = j / per_head;
+                const uint32_t hs = jh < nq ? kv_begin * p.group + jh
+                                            : (jh < nq + kvn ? p.n_heads + kv_begin + (jh - nq)
+                                                             : p.n_heads + p.n_kv_heads + kv_begin + (jh - nq - kvn));
+                rope_item<T>(p.rope, row0 + row, hs * per_head + j % per_head);
+            }
+            __syncthreads();   // the rotated queries and the new cache rows are in memory before anyone reads them
+        });
+    } else {
+        split.for_each_segment(run_segment);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -1696,19 +1746,19 @@ int launch_dma8(hipStream_t stream, const DecodeMfmaParams &p, uint32_t n_workgr
     }
 }
 
-template <typename T, int D, int KVF, bool MULTI_SUB, bool WHOLE = false>
+template <typename T, int D, int KVF, bool MULTI_SUB, bool WHOLE = false, bool ROPE = false>
 int launch_inst(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;
     const size_t lds = 2 * static_cast<size_t>(kWaves) * 2 * kStep * D * 2 + (KV8 ? 2 * 2 * kWaves * kStep * 4 : 0) +
                        (kSplitLdsWords + p.n_units + 1) * sizeof(uint32_t);
-    auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB, WHOLE>;
+    auto kernel = decode_mfma_kernel<T, D, KVF, MULTI_SUB, WHOLE, ROPE>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
             return rc;
         }
     }
-    dim3 grid(grid_x, 1, 1);
+    dim3 grid(grid_x, WHOLE ? ceil_div(p.n_kv_heads, p.kv_per_wg) : 1u, 1);
     kernel<<<grid, kWaves * 64, lds, stream>>>(p);
     XL_LAUNCH_CHECK();
     return XLITE_HIP_OK;
@@ -1727,6 +1777,14 @@ int launch_whole(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
 {
     return p.n_sub > 1 ? launch_inst<T, D, XLITE_HIP_KV_SAME, true, true>(stream, p, grid_x)
                        : launch_inst<T, D, XLITE_HIP_KV_SAME, false, true>(stream, p, grid_x);
+}
+
+// ... that rotate and store the rows themselves
+template <typename T, int D>
+int launch_whole_rope(hipStream_t stream, const DecodeMfmaParams &p, uint32_t grid_x)
+{
+    return p.n_sub > 1 ? launch_inst<T, D, XLITE_HIP_KV_SAME, true, true, true>(stream, p, grid_x)
+                       : launch_inst<T, D, XLITE_HIP_KV_SAME, false, true, true>(stream, p, grid_x);
 }
 
 template <typename T, int D>
@@ -1803,7 +1861,19 @@ size_t decode_mfma_workspace_bytes(uint32_t batch, uint32_t n_heads, uint32_t he
     return pl.meta_bytes + pl.ml_bytes + pl.acc_bytes;
 }
 
-int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
+// Contexts that are short by the width of the block tables (at most 16 steps per wave: the waves of a kv head
+// share a row when there are fewer than 8 kv heads): no split, one workgroup per row, no merge launch. Such a
+// step is bound by its launches: Qwen2-0.5B, 4 sequences of up to 512 positions, 12.7 us + 3.9 us of merge -> one
+// kernel.
+bool decode_mfma_whole_rows(const AttentionArgs &a)
+{
+    const uint32_t waves_per_kv = a.n_kv_heads >= kWaves ? 1u : kWaves / a.n_kv_heads;
+    return a.rows_mode != kOnlySingle && a.kv_dtype == XLITE_HIP_KV_SAME && a.head_dim != 256 &&
+           ceil_div(static_cast<uint64_t>(a.max_num_block) * a.block_size, static_cast<uint64_t>(kStep)) <= 16ull * waves_per_kv &&
+           a.max_num_block <= kSplitTblCap - 2;
+}
+
+int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a, const RopeArgs *rope)
 {
     const bool bf = a.dtype == XLITE_HIP_BF16;
     DecodeMfmaParams p{};
@@ -1851,15 +1921,35 @@ int launch_decode_mfma(hipStream_t stream, const AttentionArgs &a)
     // slice. (Sequences' rows lie anywhere among the batch's rows, so a batch served by two kernels is one slice.)
     const uint32_t units = p.only_single ? a.batch : a.total_tokens;
     XL_REQUIRE(!p.only_single || units <= kSplitSeqCap, "too many sequences for a batch served by two kernels");
-    // Contexts that are short by the width of the block tables (at most 16 steps per wave: the waves of a kv head
-    // share a row when there are fewer than 8 kv heads): no split, one workgroup per row, no merge launch. Such a
-    // step is bound by its launches: Qwen2-0.5B, 4 sequences of up to 512 positions, 12.7 us + 3.9 us of merge -> one
-    // kernel.
-    const uint32_t waves_per_kv = a.n_kv_heads >= kWaves ? 1u : kWaves / a.n_kv_heads;
-    const bool whole_rows = !p.only_single && a.kv_dtype == XLITE_HIP_KV_SAME && a.head_dim != 256 &&
-                            ceil_div(static_cast<uint64_t>(a.max_num_block) * a.block_size, static_cast<uint64_t>(kStep)) <=
-                                16ull * waves_per_kv &&
-                            a.max_num_block <= kSplitTblCap - 2;
+    const bool whole_rows = decode_mfma_whole_rows(a);
+    if (whole_rows) {
+        // Few rows: a workgroup per (row, kv head), its eight waves sharing the head's range, so that a row's cache
+        // bytes come in through n_kv_heads compute units instead of one (with nothing in the caches a compute unit
+        // takes in some 50 GB/s: Qwen2-0.5B, 4 rows of up to 512 positions, 248 KB each). Otherwise a workgroup per
+        // row, all kv heads in passes of up to 8.
+        const uint32_t rows = rope != nullptr ? a.batch : a.total_tokens;
+        p.kv_per_wg = a.n_kv_heads;
+        if (static_cast<uint64_t>(rows) * a.n_kv_heads <= grid_x) {
+            p.kv_per_wg = 1;
+            p.n_sub = kWaves;
+        }
+    }
+    if (rope != nullptr) {
+        // one launch for the layer's rope_and_cache and attention: by sequence, whatever the batch size
+        XL_REQUIRE(whole_rows && rope->num_tokens == a.total_tokens && rope->n_heads == a.n_heads &&
+                       rope->n_kv_heads == a.n_kv_heads && rope->head_dim == a.head_dim && rope->k_cache != nullptr,
+                   "the decode kernel rotates rows only for batches it takes whole");
+        p.rope = *rope;
+        p.unit0 = 0;
+        p.n_units = 1;   // (sizes the prefix sums in LDS, which this mode does not keep)
+        p.step_mult = 1;
+        p.block_magic = static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32)
+                            ? static_cast<uint32_t>((1ull << 32) / a.block_size) + 1
+                            : 0u;
+        const uint32_t gx = min(grid_x, a.batch);
+        return a.head_dim == 128 ? (bf ? launch_whole_rope<BF16, 128>(stream, p, gx) : launch_whole_rope<FP16, 128>(stream, p, gx))
+                                 : (bf ? launch_whole_rope<BF16, 64>(stream, p, gx) : launch_whole_rope<FP16, 64>(stream, p, gx));
+    }
     for (uint32_t u0 = 0; u0 < units; u0 += kSplitSeqCap) {
         p.unit0 = u0;
         p.n_units = min(kSplitSeqCap, units - u0);
