@@ -133,7 +133,10 @@ int xlite_hip_set_clock_probe(void *device_words);
  * xlite_hip_rope_and_cache followed by xlite_hip_attention with the arguments of the
  * two (16-bit caches), same results bit for bit. For serving loops whose small batches
  * are bound by the cost of a call, not of the kernels. Any batch the two accept, not
- * only decode rows.
+ * only decode rows. A decode batch whose contexts are short by the width of its block
+ * tables (the batches the decode kernel serves a whole row per workgroup, without a merge
+ * launch) is a single kernel launch: the workgroup of a sequence rotates and stores the
+ * sequence's rows, then walks them.
  * ---------------------------------------------------------------------- */
 int xlite_hip_decode_step(void *stream, void *qkv, void *k_cache, void *v_cache, void *output,
                           const int64_t *position, const void *cosin, const int32_t *slot_mapping,
