@@ -109,9 +109,10 @@ class MhaLayer:
         if c.qk_norm:
             _C.qk_rms_norm(rt, qkv, self.q_norm, None, self.k_norm, None, qkv, c.norm_eps, c.head_dim, c.n_heads,
                            c.head_dim, c.n_kv_heads, c.n_heads * c.head_dim)
-        _C.rope_and_cache(rt, qkv, k_cache, v_cache, meta.position, cosin, meta.slot_mapping, c.n_heads, c.n_kv_heads,
-                          c.head_dim, c.rot_dim, c.block_size, True)
         attn = torch.empty(hidden.shape[0], c.n_heads * c.head_dim, dtype=hidden.dtype, device=hidden.device)
-        _C.attention(rt, qkv, k_cache, v_cache, attn, meta.query_start_loc, meta.lens, meta.cached_lens, meta.block_tables,
-                     c.n_heads, c.n_kv_heads, c.head_dim, c.block_size, meta.batch, meta.max_num_blocks)
+        # rope_and_cache, then attention (xlite/csrc/model.cpp:544-571), from one call into the library: a single
+        # kernel launch for decode steps over short contexts, the two launches otherwise, the same bits either way
+        _C.decode_step(rt, qkv, k_cache, v_cache, attn, meta.position, cosin, meta.slot_mapping, meta.query_start_loc,
+                       meta.lens, meta.cached_lens, meta.block_tables, c.n_heads, c.n_kv_heads, c.head_dim, c.rot_dim,
+                       c.block_size, meta.batch, meta.max_num_blocks)
         return torch.matmul(attn, self.wo)
