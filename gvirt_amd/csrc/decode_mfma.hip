@@ -209,7 +209,7 @@ __device__ __forceinline__ uint32_t uni(uint32_t x)
 // WHOLE: no split - workgroup i walks the whole range of the rows i, i + grid, ...: nothing to merge (a template
 // parameter, so that each kernel has one call site for its segment body: a second copy of that body, or the extra live
 // values of a run-time choice, cost the streaming kernels 4 %)
-// ROPE (with WHOLE): the units are the sequences; `before_rows(first row, rows)` runs ahead of a sequence's rows.
+// ROPE (with WHOLE): the units are the sequences; `before.rows(first row, rows, ...)` runs ahead of a sequence's rows.
 template <bool WHOLE = false, bool ROPE = false>
 struct DecodeSplit {
     const DecodeMfmaParams &p;
@@ -399,20 +399,26 @@ struct DecodeSplit {
     }
     // segment(seq, row, t0, t1, whole, partial slot, first piece of its row, meta of the row)
     struct NoPrologue {
-        __device__ __forceinline__ void operator()(uint32_t, uint32_t) const {}
+        __device__ __forceinline__ int guess(uint32_t) const { return 0; }
+        __device__ __forceinline__ void together(int &, int32_t &, int32_t &, int32_t &) const {}
+        __device__ __forceinline__ void rows(uint32_t, uint32_t, uint32_t, int) const {}
     };
     template <typename F, typename G = NoPrologue>
-    __device__ __forceinline__ void for_each_segment(F &&segment, G &&before_rows = G()) const
+    __device__ __forceinline__ void for_each_segment(F &&segment, G &&before = G()) const
     {
         if constexpr (WHOLE && ROPE) {
             // by sequence: the rows of a sequence see each other's new cache rows, so one workgroup writes them all
-            // before it walks any (a plain decode step has one row per sequence)
+            // before it walks any. A plain decode step has one row per sequence, row s for sequence s: what the
+            // prologue needs of that row is requested (`guess`) together with the three words that say whether the
+            // guess holds.
             for (uint32_t s = blockIdx.x; s < p.batch; s += gridDim.x) {
-                const int32_t start = p.query_start_loc[s], ql = p.lens[s], cached = p.cached_lens[s];
+                auto guessed = before.guess(s);
+                int32_t start = p.query_start_loc[s], ql = p.lens[s], cached = p.cached_lens[s];
+                before.together(guessed, start, ql, cached);
                 if (ql <= 0) {
                     continue;
                 }
-                before_rows(uni(static_cast<uint32_t>(start)), uni(static_cast<uint32_t>(ql)));
+                before.rows(uni(static_cast<uint32_t>(start)), uni(static_cast<uint32_t>(ql)), s, guessed);
                 for (int32_t r = 0; r < ql; r++) {
                     const int32_t lim = cached + r + 1;
                     segment(uni(s), uni(static_cast<uint32_t>(start + r)), 0u, uni(static_cast<uint32_t>(lim > 1 ? lim : 1)), true,
@@ -911,16 +917,45 @@ decode_mfma_kernel(const DecodeMfmaParams p)
         const uint32_t per_head = p.rope.head_dim / 8 - p.rope.rot_dim / 16;
         const uint32_t kvn = kv_end - kv_begin, nq = kvn * p.group;
         const uint32_t per_row = (nq + 2 * kvn) * per_head;
-        split.for_each_segment(run_segment, [&](uint32_t row0, uint32_t rows) {
-            for (uint32_t i = threadIdx.x; i < rows * per_row; i += NT) {
-                const uint32_t row = i / per_row, j = i % per_row, jh = j / per_head;
-                const uint32_t hs = jh < nq ? kv_begin * p.group + jh
-                                            : (jh < nq + kvn ? p.n_heads + kv_begin + (jh - nq)
-                                                             : p.n_heads + p.n_kv_heads + kv_begin + (jh - nq - kvn));
-                rope_item<T>(p.rope, row0 + row, hs * per_head + j % per_head);
+        auto slot_of = [&](uint32_t j) {
+            const uint32_t jh = j / per_head;
+            const uint32_t hs = jh < nq ? kv_begin * p.group + jh
+                                        : (jh < nq + kvn ? p.n_heads + kv_begin + (jh - nq)
+                                                         : p.n_heads + p.n_kv_heads + kv_begin + (jh - nq - kvn));
+            return hs * per_head + j % per_head;
+        };
+        struct Prologue {
+            const DecodeMfmaParams &p;
+            decltype(slot_of) &slot_of;
+            uint32_t per_row;
+            // the thread's first item of row s, should that be the sequence's only row
+            __device__ __forceinline__ RopeItemRegs guess(uint32_t s) const
+            {
+                return rope_item_load(p.rope, min(s, p.rope.num_tokens - 1), slot_of(min(threadIdx.x, per_row - 1)));
             }
-            __syncthreads();   // the rotated queries and the new cache rows are in memory before anyone reads them
-        });
+            // One wait for all of it: left alone the compiler orders the loads by their first use, a trip to memory
+            // for the row count, one for the other two words, one for the row.
+            __device__ __forceinline__ void together(RopeItemRegs &x, int32_t &start, int32_t &ql, int32_t &cached) const
+            {
+                asm volatile("" : "+v"(x.a.v.x), "+v"(x.a.v.y), "+v"(x.a.v.z), "+v"(x.a.v.w), "+v"(x.b.v.x), "+v"(x.b.v.y),
+                                  "+v"(x.b.v.z), "+v"(x.b.v.w), "+v"(x.pos_t), "+v"(x.slot), "+v"(start), "+v"(ql), "+v"(cached));
+            }
+            __device__ __forceinline__ void rows(uint32_t row0, uint32_t n, uint32_t s, const RopeItemRegs &guessed) const
+            {
+                uint32_t i = threadIdx.x;
+                if (row0 == s && n == 1) {
+                    if (i < per_row) {
+                        rope_item_finish<T>(p.rope, row0, slot_of(i), guessed);
+                    }
+                    i += NT;
+                }
+                for (; i < n * per_row; i += NT) {
+                    rope_item<T>(p.rope, row0 + i / per_row, slot_of(i % per_row));
+                }
+                __syncthreads();   // the rotated queries and the new cache rows are in memory before anyone reads them
+            }
+        };
+        split.for_each_segment(run_segment, Prologue{p, slot_of, per_row});
     } else {
         split.for_each_segment(run_segment);
     }

@@ -87,71 +87,83 @@ __device__ __forceinline__ uint32_t rope_items_per_token(const RopeArgs &r)
 
 // Item `rem` of token `t`: a thread rotates 8 elements of the first half of the rotary span together with their 8
 // partners in the second half (both are written in place, so one thread must own both), or copies / scales one
-// pass-through chunk; k and v rows also go to the token's cache slot.
+// pass-through chunk; k and v rows also go to the token's cache slot. In two parts, so that a caller can have the
+// item's loads in flight while it finds out whether `t` is the token it wants.
+struct RopeItemRegs {
+    Vec16 a, b;        // the chunk (pair) of the row
+    int64_t pos_t;     // the token's position and cache slot
+    uint32_t slot;
+};
+
+__device__ __forceinline__ RopeItemRegs rope_item_load(const RopeArgs &r, uint32_t t, uint32_t rem)
+{
+    const uint32_t rot_pairs = r.rot_dim / 16;    // chunk pairs inside the rotary span
+    const uint32_t items_per_head = r.head_dim / 8 - rot_pairs;
+    const uint32_t hs = rem / items_per_head, item = rem % items_per_head;
+    const uint16_t *row = r.inout + (static_cast<uint64_t>(t) * (r.n_heads + 2 * r.n_kv_heads) + hs) * r.head_dim;
+    // the token's position and slot are requested together with its row (every thread loads both: under a
+    // condition each would be a trip to memory of its own); only the cos / sin row waits for the position
+    RopeItemRegs x;
+    x.pos_t = r.position[t];
+    x.slot = static_cast<uint32_t>(r.slot_mapping[t]);
+    const uint32_t e_first = item < rot_pairs ? item * 8 : (item + rot_pairs) * 8;
+    x.a.v = *reinterpret_cast<const uint4 *>(row + e_first);
+    x.b.v = *reinterpret_cast<const uint4 *>(row + (item < rot_pairs ? e_first + r.rot_dim / 2 : e_first));
+    return x;
+}
+
+template <typename T>
+__device__ __forceinline__ void rope_item_finish(const RopeArgs &r, uint32_t t, uint32_t rem, const RopeItemRegs &x)
+{
+    uint16_t *const k_cache = r.k_cache, *const v_cache = r.v_cache;
+    const uint32_t n_heads = r.n_heads, n_kv_heads = r.n_kv_heads, head_dim = r.head_dim, rot_dim = r.rot_dim,
+                   block_size = r.block_size;
+    const uint32_t rot_pairs = rot_dim / 16;
+    const uint32_t items_per_head = head_dim / 8 - rot_pairs;
+    const uint32_t half = rot_dim / 2;
+    const uint32_t hs = rem / items_per_head;
+    const uint32_t item = rem % items_per_head;
+    uint16_t *row = r.inout + (static_cast<uint64_t>(t) * (n_heads + 2 * n_kv_heads) + hs) * head_dim;
+    const bool is_q = hs < n_heads;
+    const bool is_k = !is_q && hs < n_heads + n_kv_heads;
+    Vec16 a = x.a, b = x.b;
+    uint16_t *cache_row = nullptr;
+    if (!is_q && k_cache != nullptr) {   // no 16-bit caches: the caller quantises the rows afterwards
+        const uint32_t kvh = is_k ? hs - n_heads : hs - n_heads - n_kv_heads;
+        const uint64_t off =
+            ((static_cast<uint64_t>(x.slot / block_size) * block_size + x.slot % block_size) * n_kv_heads + kvh) * head_dim;
+        cache_row = (is_k ? k_cache : v_cache) + off;
+    }
+    if (item < rot_pairs) {
+        const uint32_t e0 = item * 8;  // first-half elements e0..e0+7, partners at +half
+        if (is_q || is_k) {
+            rotate_chunk_pair<T>(a, b, e0, half, t, x.pos_t, r.num_tokens, rot_dim, r.position, r.cosin, r.mask_h, r.mask_w, is_q,
+                                 r.q_scale);
+            *reinterpret_cast<uint4 *>(row + e0) = a.v;
+            *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
+        }
+        if (cache_row) {
+            *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
+            *reinterpret_cast<uint4 *>(cache_row + e0 + half) = b.v;
+        }
+    } else {
+        const uint32_t e0 = (item + rot_pairs) * 8;  // beyond the rotary span
+        if (is_q) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                a.h[j] = T::from_f32(T::to_f32(a.h[j]) * r.q_scale);
+            }
+            *reinterpret_cast<uint4 *>(row + e0) = a.v;
+        } else if (cache_row) {
+            *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
+        }
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ void rope_item(const RopeArgs &r, uint32_t t, uint32_t rem)
 {
-    uint16_t *const inout = r.inout, *const k_cache = r.k_cache, *const v_cache = r.v_cache;
-    const int64_t *const position = r.position;
-    const uint16_t *const cosin = r.cosin;
-    const int32_t *const slot_mapping = r.slot_mapping;
-    const uint32_t num_tokens = r.num_tokens, n_heads = r.n_heads, n_kv_heads = r.n_kv_heads, head_dim = r.head_dim,
-                   rot_dim = r.rot_dim, block_size = r.block_size;
-    const float q_scale = r.q_scale;
-    const uint64_t mask_h = r.mask_h, mask_w = r.mask_w;
-    const uint32_t chunks = head_dim / 8;       // 16-byte chunks per head
-    const uint32_t rot_pairs = rot_dim / 16;    // chunk pairs inside the rotary span
-    const uint32_t items_per_head = chunks - rot_pairs;
-    const uint32_t slots = n_heads + 2 * n_kv_heads;
-    const uint32_t half = rot_dim / 2;
-    {
-        const uint32_t hs = rem / items_per_head;
-        const uint32_t item = rem % items_per_head;
-        uint16_t *row = inout + (static_cast<uint64_t>(t) * slots + hs) * head_dim;
-
-        const bool is_q = hs < n_heads;
-        const bool is_k = !is_q && hs < n_heads + n_kv_heads;
-        // the token's position and slot are requested together with its row (every thread loads both: under a
-        // condition each would be a trip to memory of its own); only the cos / sin row waits for the position
-        const int64_t pos_t = position[t];
-        const uint32_t slot = static_cast<uint32_t>(slot_mapping[t]);
-        const uint32_t e_first = item < rot_pairs ? item * 8 : (item + rot_pairs) * 8;
-        Vec16 a, b;
-        a.v = *reinterpret_cast<const uint4 *>(row + e_first);
-        b.v = *reinterpret_cast<const uint4 *>(row + (item < rot_pairs ? e_first + half : e_first));
-        uint16_t *cache_row = nullptr;
-        if (!is_q && k_cache != nullptr) {   // no 16-bit caches: the caller quantises the rows afterwards
-            const uint32_t kvh = is_k ? hs - n_heads : hs - n_heads - n_kv_heads;
-            const uint64_t off =
-                ((static_cast<uint64_t>(slot / block_size) * block_size + slot % block_size) * n_kv_heads +
-                 kvh) * head_dim;
-            cache_row = (is_k ? k_cache : v_cache) + off;
-        }
-
-        if (item < rot_pairs) {
-            const uint32_t e0 = item * 8;  // first-half elements e0..e0+7, partners at +half
-            if (is_q || is_k) {
-                rotate_chunk_pair<T>(a, b, e0, half, t, pos_t, num_tokens, rot_dim, position, cosin, mask_h, mask_w, is_q, q_scale);
-                *reinterpret_cast<uint4 *>(row + e0) = a.v;
-                *reinterpret_cast<uint4 *>(row + e0 + half) = b.v;
-            }
-            if (cache_row) {
-                *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
-                *reinterpret_cast<uint4 *>(cache_row + e0 + half) = b.v;
-            }
-        } else {
-            const uint32_t e0 = (item + rot_pairs) * 8;  // beyond the rotary span
-            if (is_q) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    a.h[j] = T::from_f32(T::to_f32(a.h[j]) * q_scale);
-                }
-                *reinterpret_cast<uint4 *>(row + e0) = a.v;
-            } else if (cache_row) {
-                *reinterpret_cast<uint4 *>(cache_row + e0) = a.v;
-            }
-        }
-    }
+    rope_item_finish<T>(r, t, rem, rope_item_load(r, t, rem));
 }
 
 }  // namespace xlite
