@@ -223,10 +223,14 @@ def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
               cached_lens: torch.Tensor, block_tables: torch.Tensor, n_heads: int, n_kv_heads: int,
               head_dim: int, block_size: int, batch: int, max_num_block: int,
               enable_flash_attention: bool = False, tile_size_of_cached_kv: int = 8192, *,
-              k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+              k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+              workspace_limit: Optional[int] = None) -> None:
     """Paged GQA attention, decode and causal (chunked) prefill. `enable_flash_attention` and
     `tile_size_of_cached_kv` select between two kernels in the reference; here they are hints
-    only (the KV split is chosen from the batch shape)."""
+    only (the KV split is chosen from the batch shape). `workspace_limit` (keyword-only, bytes): hand the
+    library at most that much scratch, as a caller with little memory would; paths that need more are not
+    taken (a multi-row batch over a quantised cache is then read by the prefill kernel itself instead of
+    through a 16-bit copy of its blocks) or fail with the library's error."""
     for n, t in (("qkv", qkv), ("k_cache", k_cache), ("v_cache", v_cache), ("output", output)):
         _dev(n, t)
     for n, t in (("query_start_loc", query_start_loc), ("lens", lens), ("cached_lens", cached_lens),
@@ -255,10 +259,11 @@ def attention(rt: Runtime, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     need = rt._lib.xlite_hip_attention_workspace_bytes_kv(T, n_heads, n_kv_heads, head_dim, block_size, batch,
                                                           max_num_block, kv)
     ws = rt.workspace(need)
+    ws_bytes = ws.numel() if workspace_limit is None else min(ws.numel(), int(workspace_limit))
     _lib.check(rt._lib.xlite_hip_attention(
         rt.stream(), _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(output), _ptr(query_start_loc), _ptr(lens),
         _ptr(cached_lens), _ptr(block_tables), T, n_heads, n_kv_heads, head_dim, block_size, batch, max_num_block,
-        dt, kv, _ptr(k_scale), _ptr(v_scale), _ptr(ws), ws.numel()))
+        dt, kv, _ptr(k_scale), _ptr(v_scale), _ptr(ws), ws_bytes))
     rt.finish()
 
 

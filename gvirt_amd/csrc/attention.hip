@@ -58,6 +58,12 @@ bool mixed_split(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, u
            decode_mfma_supported(n_heads, n_kv_heads, head_dim, block_size, batch);
 }
 
+// M rows (query rows x query heads of a kv head) per sequence, on average, up to which a multi-row batch over a
+// quantised cache is read on the fly by the prefill kernel instead of through a 16-bit copy. Measured, int8, by copy /
+// on the fly: Llama-3-8B 32 x 64 tokens 0.030 / 0.022 ms, 128 after 16384 cached 0.095 / 0.082, 8 x 256 after 4096
+// 0.231 / 0.211, 8 x 512 after 4096 0.354 / 0.356 (the break-even: 2048 M rows), 8 x 2048 after 4096 1.45 / 1.60.
+constexpr uint64_t kKv8DirectRows = 2048;
+
 // A quantised cache is read directly by the streaming decode kernel (and, int8 only, by the vector decode
 // kernel); every other batch goes through a 16-bit copy of its blocks.
 bool quantised_direct(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t block_size,
@@ -148,6 +154,17 @@ extern "C" int xlite_hip_attention(void *stream, const void *qkv, const void *k_
     if (kv_dtype != XLITE_HIP_KV_SAME &&
         !quantised_direct(total_tokens, n_heads, n_kv_heads, head_dim, block_size, batch, kv_dtype)) {
         XL_REQUIRE(decode_supported(head_dim), "quantised KV caches: head_dim must be 64 or 128");
+        // Multi-row batches of head_dim 128: the prefill kernel reads the bytes itself when the chunks are short (the
+        // copy below dequantises the whole visible cache of the batch, five bytes of traffic per cached element,
+        // whatever the number of query rows; reading on the fly costs the kernel a tenth of its time on long chunks)
+        // or when the workspace cannot hold the copy.
+        if (!is_decode_batch(total_tokens, batch) && prefill_kv8_supported(a)) {
+            const size_t copy_bytes = kv_dequant_bytes(n_kv_heads, head_dim, block_size, batch, max_num_block);
+            const bool short_chunks = static_cast<uint64_t>(total_tokens) * (n_heads / n_kv_heads) <= kKv8DirectRows * static_cast<uint64_t>(batch);
+            if (short_chunks || a.workspace == nullptr || a.workspace_bytes < copy_bytes) {
+                return launch_prefill_mfma(s, a);
+            }
+        }
         if (const int rc = launch_kv_dequant(s, &a)) {   // from here on: fp16 caches in the workspace
             return rc;
         }

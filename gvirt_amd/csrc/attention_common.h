@@ -131,6 +131,7 @@ int launch_mla_decode(hipStream_t stream, const MlaArgs &a);
 
 // prefill_mfma.hip
 bool prefill_mfma_supported(const AttentionArgs &a);
+bool prefill_kv8_supported(const AttentionArgs &a);
 int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a);
 size_t prefill_mfma_workspace_bytes(uint32_t total_tokens, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                                     uint32_t batch, uint32_t max_ctx);

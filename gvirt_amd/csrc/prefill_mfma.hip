@@ -23,6 +23,7 @@
 #include <type_traits>
 
 #include "attention_common.h"
+#include "kv8.h"
 
 namespace xlite {
 
@@ -85,6 +86,8 @@ struct PrefillParams {
     float *part_acc;           // [token][head][max_splits][D]
     float *part_ml;            // [token][head][max_splits][2]: reference maximum (log2 domain), normaliser
     unsigned long long *clock_probe;   // nullptr, or where workgroup 0 leaves its shader-clock and wall-clock stamps
+    const float *k_scale;      // 8-bit caches read by the kernel itself: [slot][kv head] fp32
+    const float *v_scale;
 };
 
 // XOR pattern of the 16-byte chunk index of LDS row `row` (rows are 256 bytes = one bank window). The
@@ -135,11 +138,17 @@ __device__ __forceinline__ uint4 convert8(const uint4 &x)
 
 // T: the type of the caches and of the products; TIO: the type of the query rows and of the output (the same, or
 // bf16 over fp16 caches: a bf16 model over the fp16 copy of a quantised cache)
-template <typename T, int D, typename TIO = T>
+// KVF: the cache is 16-bit (copied straight into LDS), or int8 / fp8 bytes with one fp32 scale per (position, kv head):
+// then a wave loads the bytes and scales of its eight positions of a tile into registers, two tiles ahead, and writes
+// them to the tile's stage as fp16 (value x scale, the arithmetic of the dequantising copy in kv_dequant.hip: same
+// bits) one iteration later; everything behind the stages is the 16-bit kernel. head_dim 128, T = FP16.
+template <typename T, int D, typename TIO = T, int KVF = XLITE_HIP_KV_SAME>
 __global__ void __launch_bounds__(kThreads, 1)
 prefill_kernel(const PrefillParams p)
 {
-    constexpr int ROWB = D * 2;               // bytes of one (position, kv head) row
+    constexpr bool KV8 = KVF != XLITE_HIP_KV_SAME;
+    static_assert(!KV8 || (D == 128 && std::is_same<T, FP16>::value), "8-bit caches: head_dim 128, fp16 products");
+    constexpr int ROWB = D * 2;               // bytes of one (position, kv head) row in LDS
     constexpr int KBYTES = BN * ROWB;         // 16 KiB (8 KiB for head_dim 64)
     constexpr int STAGE = 2 * KBYTES;         // K tile, then V tile
     constexpr int KS = D / 16;                // k-steps of the QK product
@@ -289,7 +298,7 @@ prefill_kernel(const PrefillParams p)
         n_tiles = min(n_tiles, first_tile + per);
     }
     const int32_t *table = p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
-    const uint32_t row_bytes = p.n_kv_heads * ROWB;
+    const uint32_t row_bytes = p.n_kv_heads * (KV8 ? D : ROWB);   // of a position in the cache
     uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(smem + kStages * STAGE);
 
     // ---- this lane's M row ---------------------------------------------------------------------------
@@ -396,6 +405,34 @@ prefill_kernel(const PrefillParams p)
             dma_1k(st + pos * ROWB, voff, kb);
             dma_1k(st + KBYTES + pos * ROWB, voff, vb);
         }
+    };
+
+    // 8-bit caches: lane l of wave w holds bytes 16 (l % 8) .. + 15 of position 8 w + l / 8 of the tile (K and V) and
+    // the position's two scales. The eight positions share a block (block sizes are multiples of 8); positions at or
+    // beyond the end of the range re-read the last valid one.
+    uint4 kraw = make_uint4(0, 0, 0, 0), vraw = make_uint4(0, 0, 0, 0);
+    float ksc = 0.f, vsc = 0.f;
+    auto fetch8 = [&](uint32_t tile) {
+        const uint32_t lim = range_end - 1;
+        const uint32_t t_raw = tile * BN + 8 * wave;
+        const uint32_t t = min(t_raw, lim) & ~7u;
+        const uint32_t rel = min(t_raw + (lane >> 3), lim) - t;
+        const uint32_t blk = __umulhi(t, p.block_magic), off = t - blk * p.block_size;
+        const uint32_t phys = __builtin_amdgcn_readfirstlane(tbl_lds[blk]);
+        const uint64_t row = static_cast<uint64_t>(phys) * p.block_size + off + rel;
+        const uint64_t at = (row * p.n_kv_heads + kvh) * D + (lane & 7u) * 16;
+        kraw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const unsigned char *>(p.k_cache) + at);
+        vraw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const unsigned char *>(p.v_cache) + at);
+        ksc = p.k_scale[row * p.n_kv_heads + kvh];
+        vsc = p.v_scale[row * p.n_kv_heads + kvh];
+    };
+    auto store8 = [&](uint32_t tile) {
+        unsigned char *st = smem + (tile % kStages) * STAGE;
+        const uint32_t pos = 8 * wave + (lane >> 3), c = 2 * (lane & 7u);
+        *reinterpret_cast<uint4 *>(st + tile_off<D>(pos, c)) = dequant8<FP16, KVF>(make_uint2(kraw.x, kraw.y), ksc);
+        *reinterpret_cast<uint4 *>(st + tile_off<D>(pos, c + 1)) = dequant8<FP16, KVF>(make_uint2(kraw.z, kraw.w), ksc);
+        *reinterpret_cast<uint4 *>(st + KBYTES + tile_off<D>(pos, c)) = dequant8<FP16, KVF>(make_uint2(vraw.x, vraw.y), vsc);
+        *reinterpret_cast<uint4 *>(st + KBYTES + tile_off<D>(pos, c + 1)) = dequant8<FP16, KVF>(make_uint2(vraw.z, vraw.w), vsc);
     };
 
     // A wave issues in order, so its own softmax does not overlap its own products; what the wave itself can
@@ -539,15 +576,27 @@ prefill_kernel(const PrefillParams p)
         }
         __syncthreads();
     }
-    issue(first_tile);
-    issue(min(first_tile + 1, last));
-    issue(min(first_tile + 2, last));
+    if constexpr (KV8) {
+        // the first two tiles go to their stages now, the third stays in registers: iteration `tile` writes tile + 2
+        // (its stage was last read two iterations ago, a barrier has passed) and requests tile + 3
+        fetch8(first_tile);
+        store8(first_tile);
+        fetch8(min(first_tile + 1, last));
+        store8(first_tile + 1);
+        fetch8(min(first_tile + 2, last));
+    } else {
+        issue(first_tile);
+        issue(min(first_tile + 1, last));
+        issue(min(first_tile + 2, last));
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
         asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
         qreg[ks] = m_valid ? convert8<TIO, T>(qreg[ks]) : make_uint4(0, 0, 0, 0);
     }
-    dma_wait<2 * PER_WAVE>();
+    if constexpr (!KV8) {
+        dma_wait<2 * PER_WAVE>();
+    }
     __syncthreads();
     fetch_k((first_tile % kStages) * STAGE, 0);
     using MaskOn = std::integral_constant<bool, true>;
@@ -557,9 +606,15 @@ prefill_kernel(const PrefillParams p)
         const uint32_t so_next = (min(tile + 1, last) % kStages) * STAGE;
         const uint32_t j0 = tile * BN;
         step(so, 0, j0, so, 1, mask_tag);
-        dma_wait<PER_WAVE>();   // this wave's share of tile + 1 has landed
-        __syncthreads();        // ... and everybody else's; stage (tile - 1) % 4 is free
-        issue(min(tile + 3, last));
+        if constexpr (KV8) {
+            store8(tile + 2);
+            __syncthreads();
+            fetch8(min(tile + 3, last));
+        } else {
+            dma_wait<PER_WAVE>();   // this wave's share of tile + 1 has landed
+            __syncthreads();        // ... and everybody else's; stage (tile - 1) % 4 is free
+            issue(min(tile + 3, last));
+        }
         step(so, 1, j0 + 32, so_next, 0, mask_tag);
     };
     // Tiles wholly below the causal limit of every row of the wave need no mask. Two loops rather than a
@@ -578,9 +633,15 @@ prefill_kernel(const PrefillParams p)
         // none of the wave's 32 rows exists (the last M tile of a sequence; a decode row in a mixed batch
         // fills 4 of 256): the wave only keeps copying its share and meeting the others at the barrier
         for (; tile < n_tiles; tile++) {
-            dma_wait<PER_WAVE>();
-            __syncthreads();
-            issue(min(tile + 3, last));
+            if constexpr (KV8) {
+                store8(tile + 2);
+                __syncthreads();
+                fetch8(min(tile + 3, last));
+            } else {
+                dma_wait<PER_WAVE>();
+                __syncthreads();
+                issue(min(tile + 3, last));
+            }
         }
     }
     dma_wait<0>();
@@ -666,6 +727,18 @@ bool prefill_mfma_supported(const AttentionArgs &a)
            a.n_heads % a.n_kv_heads == 0;
 }
 
+// 8-bit caches read by the kernel itself: head_dim 128, block sizes that are multiples of 8 (a wave's eight positions of
+// a tile share a block)
+bool prefill_kv8_supported(const AttentionArgs &a)
+{
+    const size_t lds = static_cast<size_t>(kStages) * 2 * BN * a.head_dim * 2 +
+                       (static_cast<size_t>(a.max_num_block) + 1) * sizeof(uint32_t);
+    return a.head_dim == 128 && (a.kv_dtype == XLITE_HIP_KV_INT8 || a.kv_dtype == XLITE_HIP_KV_FP8) &&
+           a.k_scale != nullptr && a.v_scale != nullptr && a.block_size % 8 == 0 && lds <= kLdsLimit &&
+           static_cast<uint64_t>(a.max_num_block) * a.block_size * a.block_size < (1ull << 32) &&
+           a.n_heads % a.n_kv_heads == 0;
+}
+
 // KV splits per M tile. The cost of s splits, in units of one workgroup walking the longest possible context:
 //     (rounds of workgroups over the chip) x (1 / s of the walk + a workgroup's set-up and drain, about four KV
 //     tiles' time) + s x (the partials' trip through memory: fp32 O per row and head, written and read back)
@@ -735,6 +808,10 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     p.n_mtiles = ceil_div(a.total_tokens * G, static_cast<uint32_t>(kMTile)) + a.batch;
     p.n_heads = a.n_heads;
     p.skip_single = a.rows_mode == kSkipSingle ? 1u : 0u;
+    p.k_scale = a.k_scale;
+    p.v_scale = a.v_scale;
+    const bool kv8 = a.kv_dtype != XLITE_HIP_KV_SAME;
+    XL_REQUIRE(!kv8 || prefill_kv8_supported(a), "8-bit caches: shape not served by the prefill kernel");
     uint32_t splits = prefill_mfma_pick_splits(a.total_tokens, G, a.batch, a.n_kv_heads, a.max_num_block * a.block_size, a.head_dim);
     if (a.workspace == nullptr || a.workspace_bytes < partial_bytes(a.total_tokens, a.n_heads, a.head_dim, splits)) {
         splits = 1;   // no scratch: every M tile walks its whole KV range
@@ -751,16 +828,27 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     const bool bf = a.dtype == XLITE_HIP_BF16;
     XL_REQUIRE(lds <= kLdsLimit, "block table too long for the prefill kernel");
     XL_REQUIRE(!a.io_bf16 || a.dtype == XLITE_HIP_FP16, "bf16 rows over fp16 caches: the products are fp16");
-    const void *kernel = a.io_bf16 ? (a.head_dim == 128 ? reinterpret_cast<const void *>(prefill_kernel<FP16, 128, BF16>)
-                                                        : reinterpret_cast<const void *>(prefill_kernel<FP16, 64, BF16>))
-                         : a.head_dim == 128
-                             ? (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 128>)
-                                   : reinterpret_cast<const void *>(prefill_kernel<FP16, 128>))
-                             : (bf ? reinterpret_cast<const void *>(prefill_kernel<BF16, 64>)
-                                   : reinterpret_cast<const void *>(prefill_kernel<FP16, 64>));
-    if (const int rc = ensure_dynamic_lds(kernel, lds)) {
-        return rc;
-    }
+    // (T, D, TIO, KVF) of the launch
+    auto with_kernel = [&](auto &&f) {
+        using I8 = std::integral_constant<int, XLITE_HIP_KV_INT8>;
+        using F8 = std::integral_constant<int, XLITE_HIP_KV_FP8>;
+        using SAME = std::integral_constant<int, XLITE_HIP_KV_SAME>;
+        using D128 = std::integral_constant<int, 128>;
+        using D64 = std::integral_constant<int, 64>;
+        if (kv8) {   // fp16 products, rows and results in the model's type
+            if (a.kv_dtype == XLITE_HIP_KV_INT8) {
+                return bf ? f(FP16{}, D128{}, BF16{}, I8{}) : f(FP16{}, D128{}, FP16{}, I8{});
+            }
+            return bf ? f(FP16{}, D128{}, BF16{}, F8{}) : f(FP16{}, D128{}, FP16{}, F8{});
+        }
+        if (a.io_bf16) {
+            return a.head_dim == 128 ? f(FP16{}, D128{}, BF16{}, SAME{}) : f(FP16{}, D64{}, BF16{}, SAME{});
+        }
+        if (a.head_dim == 128) {
+            return bf ? f(BF16{}, D128{}, BF16{}, SAME{}) : f(FP16{}, D128{}, FP16{}, SAME{});
+        }
+        return bf ? f(BF16{}, D64{}, BF16{}, SAME{}) : f(FP16{}, D64{}, FP16{}, SAME{});
+    };
     uint32_t n_wg;
     if (a.n_kv_heads % kXcds == 0) {
         n_wg = a.n_kv_heads * p.n_mtiles;
@@ -769,23 +857,17 @@ int launch_prefill_mfma(hipStream_t stream, const AttentionArgs &a)
     } else {
         n_wg = a.n_kv_heads * p.n_mtiles;
     }
-    dim3 grid(n_wg, splits, 1);
-    if (a.io_bf16) {
-        if (a.head_dim == 128) {
-            prefill_kernel<FP16, 128, BF16><<<grid, kThreads, lds, stream>>>(p);
-        } else {
-            prefill_kernel<FP16, 64, BF16><<<grid, kThreads, lds, stream>>>(p);
+    const dim3 grid(n_wg, splits, 1);
+    const int rc_launch = with_kernel([&](auto t, auto d, auto tio, auto kvf) -> int {
+        auto kernel = prefill_kernel<decltype(t), decltype(d)::value, decltype(tio), decltype(kvf)::value>;
+        if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
+            return rc;
         }
-    } else if (a.head_dim == 128) {
-        if (bf) {
-            prefill_kernel<BF16, 128><<<grid, kThreads, lds, stream>>>(p);
-        } else {
-            prefill_kernel<FP16, 128><<<grid, kThreads, lds, stream>>>(p);
-        }
-    } else if (bf) {
-        prefill_kernel<BF16, 64><<<grid, kThreads, lds, stream>>>(p);
-    } else {
-        prefill_kernel<FP16, 64><<<grid, kThreads, lds, stream>>>(p);
+        kernel<<<grid, kThreads, lds, stream>>>(p);
+        return XLITE_HIP_OK;
+    });
+    if (rc_launch != XLITE_HIP_OK) {
+        return rc_launch;
     }
     XL_LAUNCH_CHECK();
     if (splits == 1) {

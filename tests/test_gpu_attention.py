@@ -305,6 +305,37 @@ def test_quantised_kv_prefill_mixed_and_other_decode_shapes(rt, kv_dtype, model,
 
 
 @pytest.mark.parametrize("kv_dtype", KV_DTYPES)
+@pytest.mark.parametrize("model", [(32, 8, 128, 128, torch.bfloat16), (32, 8, 128, 16, torch.float16), (28, 4, 128, 16, torch.float16),
+                                   (64, 16, 128, 8, torch.bfloat16)])
+@pytest.mark.parametrize("work", [([500, 0, 3000], [700, 1300, 600]), ([9000], [1500]), ([0, 6, 2047, 64], [2000, 1100, 1, 900])])
+def test_quantised_prefill_read_on_the_fly_against_the_copy_path(rt, kv_dtype, model, work):
+    """Long chunks over a quantised cache go through an fp16 copy of the visible blocks; with too little scratch for
+    the copy (and, whatever the scratch, for short chunks) the prefill kernel reads the bytes and scales itself, with
+    the copy's arithmetic. Without scratch there is no KV split either, so the two agree bit for bit where the copy
+    path does not split (kv heads a multiple of 8 here) and to the last places where it does; both within the budget
+    of the oracle."""
+    nH, nKV, d, bs, dtype = model
+    clens, lens = work
+    assert sum(lens) * (nH // nKV) > 2048 * len(lens)          # by default: the copy
+    w = quantised(generic_case(63, lens, clens, nH, nKV, d, bs, dtype, rms=True), kv_dtype)
+    by_copy = run_attention(rt, w)
+    on_the_fly = run_attention(rt, w, workspace_limit=0)
+    if nKV % 8 == 0:
+        assert torch.equal(by_copy, on_the_fly)
+    assert float((by_copy - on_the_fly).abs().max()) <= 4e-3
+    check(on_the_fly, oracle_attention(w), max_abs=MAX_ABS_INT8)
+
+
+def test_quantised_prefill_without_any_scratch(rt):
+    """No scratch at all: no copy, no KV split, one kernel; head_dim 64 has no such path and says what it needs."""
+    w = quantised(generic_case(64, [300, 40], [700, 0], 32, 8, 128, 32, torch.bfloat16, rms=True), torch.int8)
+    check(run_attention(rt, w, workspace_limit=0), oracle_attention(w), max_abs=MAX_ABS_INT8)
+    w = quantised(generic_case(65, [300, 40], [700, 0], 14, 2, 64, 32, torch.bfloat16, rms=True), torch.int8)
+    with pytest.raises(RuntimeError, match="workspace too small"):
+        run_attention(rt, w, workspace_limit=0)
+
+
+@pytest.mark.parametrize("kv_dtype", KV_DTYPES)
 def test_quantised_kv_prefill_then_decode_through_quantise_on_write(rt, kv_dtype):
     """A prompt written into a quantised cache by rope_and_cache (quantise-on-write), attended to as a prefill, then
     decode steps that append to the same cache - against the oracle over a 16-bit cache quantised after every write."""
