@@ -323,7 +323,7 @@ def bench_prefill(args, torch, rt, int8=False):
         vq, vs = W.quantize_cache(caches["v_cache"], torch.int8)
         for w in chunks:
             w["k_cache"], w["v_cache"] = kq, vq
-        caches["k_cache"] = caches["v_cache"] = None
+        caches["k_cache"] = caches["v_cache"] = None   # (the bf16 tensors are freed)
 
     def step():
         for w in chunks:
@@ -350,6 +350,15 @@ def bench_prefill(args, torch, rt, int8=False):
         d = _launch_dist(torch, call(w), 20)
         d["tflops_at_median"] = round(w["flops"] / (d["median"] * 1e-3) / 1e12, 1)
         per_call.append(d)
+    # a short chunk over the same caches: 256 tokens of every sequence behind 2048 cached ones. Over the int8 cache
+    # such chunks are read by the prefill kernel itself (no copy); the bf16 leg runs the same call for comparison.
+    if int8:
+        caches["k_cache"], caches["v_cache"] = kq, vq
+    ws = W.gqa_prefill_chunk(shape, lens, 8, 256, W.SEED_BASE + 33, device=dev, caches=caches)
+    short = _launch_dist(torch, call(ws), 20)
+    short["tflops_at_median"] = round(ws["flops"] / (short["median"] * 1e-3) / 1e12, 1)
+    short["workload"] = "%d sequences x 256 tokens behind 2048 cached" % ws["batch"]
+    short["kernel"] = "prefill_kernel reading the int8 bytes and scales itself" if int8 else "prefill_kernel"
     flops = sum(w["flops"] for w in chunks)
     tokens = sum(w["tokens"] for w in chunks)
     tf = flops / (ms * 1e-3) / 1e12
@@ -394,6 +403,7 @@ def bench_prefill(args, torch, rt, int8=False):
                                    else "c3 qwen2.5-7b chunked causal prefill", "total_lens": lens, "chunk": 2048,
                        "calls_per_step": len(chunks)},
             "tokens_per_s": round(tokens / (ms * 1e-3), 1), "step_ms_dist": step_dist, "chunk_call_ms_dist": per_call,
+            "short_chunk_call": short,
             "roofline": {"bound": "mfma", "kernel": "dequant_blocks_kernel + prefill_kernel" if int8 else "prefill_kernel",
                          "achieved": round(tf, 2),
                          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),

@@ -73,13 +73,16 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  *             XLITE_HIP_KV_FP8 they hold one byte per element and k_scale/v_scale
  *             [num_blocks, block_size, n_kv_heads] fp32 hold the per-token-per-head scales
  *             (x = q * scale). Decode batches of the streaming kernel's shapes (at most 16
- *             query heads per kv head, block size a multiple of 16) read the bytes directly;
- *             every other batch over a quantised cache (prefill, chunked prefill, mixed
- *             batches, other decode shapes) first copies the blocks it can see into a 16-bit
+ *             query heads per kv head, block size a multiple of 16) read the bytes directly,
+ *             and so do multi-row batches of head_dim 128 (block size a multiple of 8) whose
+ *             chunks are short (up to 2048 query rows x heads of the group per sequence on
+ *             average) or whose workspace is too small for what follows;
+ *             every other batch over a quantised cache (long prefill chunks, other decode
+ *             shapes, head_dim 64) first copies the blocks it can see into a 16-bit
  *             cache in the workspace, which xlite_hip_attention_workspace_bytes_kv() sizes:
  *             2 tensors x batch x max_num_block x block_size x n_kv_heads x head_dim x 2 bytes
  *             (every block the tables can name, whatever the sequences' lengths: keep
- *             max_num_block close to what the batch needs).
+ *             max_num_block close to what the batch needs). Same results either way.
  * output      [total_tokens, n_heads * head_dim]
  * query_start_loc, lens, cached_lens  [batch] int32
  * block_tables [batch * max_num_block] int32
@@ -91,9 +94,10 @@ int xlite_hip_rope_and_cache(void *stream, void *inout, void *k_cache, void *v_c
  * workspace   device scratch of at least xlite_hip_attention_workspace_bytes()
  *             (or ..._bytes_kv() for a quantised cache; split-KV partial results;
  *             contents need no initialisation and are not preserved). Decode batches
- *             and batches over a quantised cache need all of it
- *             (XLITE_HIP_ENOSPC otherwise); a prefill batch given less, or
- *             NULL, still works but does not split the KV axis.
+ *             need all of it, and so do batches over a quantised cache that go through
+ *             the 16-bit copy and have no other way (XLITE_HIP_ENOSPC otherwise); a
+ *             prefill batch given less, or NULL, still works but does not split the KV
+ *             axis (head_dim 128 over a quantised cache included: it is then read directly).
  * ---------------------------------------------------------------------- */
 
 size_t xlite_hip_attention_workspace_bytes(uint32_t total_tokens, uint32_t n_heads,
