@@ -38,7 +38,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # script scaled by the same counters' readings for a plain 1 GiB copy (see --calibrate-copy); None
 # where no counter run has been taken.
 PEAK_CLOCK_GHZ = 2.4   # the engine clock the published MI355X matrix peaks are quoted at
-MEASURED_TRAFFIC_BYTES = {"c2": 1080233421, "c3": 334714478, "c4": 274685113, "c5": 1623780115}
+MEASURED_TRAFFIC_BYTES = {"c2": 1080255689, "c3": 334666881, "c4": 274669317, "c5": 1623779956}
 # where each constant comes from: the committed counter summary whose "HBM traffic per launch" line holds it
 TRAFFIC_SOURCE = {"c2": "profiles/decode_dma_kernel_c2_llama3_8b_b64_ctx4096.md",
                   "c3": "profiles/prefill_kernel_c3_qwen25_7b_chunked.md",
@@ -352,13 +352,15 @@ def bench_prefill(args, torch, rt, int8=False):
         per_call.append(d)
     # a short chunk over the same caches: 256 tokens of every sequence behind 2048 cached ones. Over the int8 cache
     # such chunks are read by the prefill kernel itself (no copy); the bf16 leg runs the same call for comparison.
-    if int8:
-        caches["k_cache"], caches["v_cache"] = kq, vq
-    ws = W.gqa_prefill_chunk(shape, lens, 8, 256, W.SEED_BASE + 33, device=dev, caches=caches)
-    short = _launch_dist(torch, call(ws), 20)
-    short["tflops_at_median"] = round(ws["flops"] / (short["median"] * 1e-3) / 1e12, 1)
-    short["workload"] = "%d sequences x 256 tokens behind 2048 cached" % ws["batch"]
-    short["kernel"] = "prefill_kernel reading the int8 bytes and scales itself" if int8 else "prefill_kernel"
+    short = None
+    if not args.no_extras:
+        if int8:
+            caches["k_cache"], caches["v_cache"] = kq, vq
+        ws = W.gqa_prefill_chunk(shape, lens, 8, 256, W.SEED_BASE + 33, device=dev, caches=caches)
+        short = _launch_dist(torch, call(ws), 20)
+        short["tflops_at_median"] = round(ws["flops"] / (short["median"] * 1e-3) / 1e12, 1)
+        short["workload"] = "%d sequences x 256 tokens behind 2048 cached" % ws["batch"]
+        short["kernel"] = "prefill_kernel reading the int8 bytes and scales itself" if int8 else "prefill_kernel"
     flops = sum(w["flops"] for w in chunks)
     tokens = sum(w["tokens"] for w in chunks)
     tf = flops / (ms * 1e-3) / 1e12
@@ -802,6 +804,9 @@ def main():
                     help="default: configuration 2 with the other configurations attached; c1..c5, idx: that one alone; "
                          "all: one line each")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the side measurements of a configuration (the prefill legs' short chunk call), so that a "
+                         "profile of the command holds the configuration's own launches only")
     ap.add_argument("--graph", action="store_true",
                     help="decode configurations: time replays of the step captured into a HIP graph instead of eager calls")
     ap.add_argument("--calibrate-copy", action="store_true",
