@@ -189,64 +189,142 @@ mfma_attention_kernel(const MfmaParams p)
 
     const int32_t *table = dense ? nullptr : p.block_tables + static_cast<uint64_t>(seq) * p.max_num_block;
 
-    for (uint32_t j0 = range_begin; j0 < range_end; j0 += BN) {
-        // ---- cache row of every token of the tile ------------------------------------------------
-        __syncthreads();  // previous tile fully consumed
+    // ---- staging. The cache rows of a tile travel through registers: a thread's K chunks (and, for a separate value
+    // cache, its V chunks: four consecutive positions of one 16-byte column group at a time, so that the transposed
+    // tile is written four positions = 8 bytes per store) are requested one tile ahead, all loads unconditional from
+    // clamped positions (rows at or beyond the end of the range repeat its last row: finite values whose
+    // probabilities are zero), and go to LDS when the previous tile has been consumed.
+    constexpr int K_ITEMS = BN * CPR;                       // 16-byte chunks of a K tile
+    constexpr int K_IT = (K_ITEMS + kThreads - 1) / kThreads;
+    constexpr int V_ITEMS = SEPARATE_V ? (BN / 4) * VCPR : 0;   // (four positions, chunk) items of a V tile
+    constexpr int V_IT = (V_ITEMS + kThreads - 1) / kThreads;
+    uint32_t kbuf[K_IT][4];                       // (plain words: the staging registers must not end up in scratch memory)
+    uint32_t vbuf[V_IT > 0 ? V_IT : 1][4][4];
+    auto cache_row = [&](uint32_t t) __attribute__((always_inline)) -> uint64_t {
+        t = t < range_end ? t : range_end - 1;
+        if (dense) {
+            return static_cast<uint64_t>(seq) * p.dense_len + t;
+        }
+        const uint32_t b = p.block_shift >= 0 ? t >> p.block_shift : t / p.block_size;
+        const uint32_t o = p.block_shift >= 0 ? t & (p.block_size - 1) : t % p.block_size;
+        return static_cast<uint64_t>(static_cast<uint32_t>(table[b])) * p.block_size + o;
+    };
+    // the tile's rows are looked up by the first BN threads and shared through LDS (two barriers around the table)
+    auto lookup = [&](uint32_t j0) __attribute__((always_inline)) {
         if (threadIdx.x < BN) {
-            uint32_t t = j0 + threadIdx.x;
-            t = t < range_end ? t : range_end - 1;
-            uint64_t row;
-            if (dense) {
-                row = static_cast<uint64_t>(seq) * p.dense_len + t;
-            } else {
-                const uint32_t b = p.block_shift >= 0 ? t >> p.block_shift : t / p.block_size;
-                const uint32_t o = p.block_shift >= 0 ? t & (p.block_size - 1) : t % p.block_size;
-                row = static_cast<uint64_t>(static_cast<uint32_t>(table[b])) * p.block_size + o;
-            }
-            rowidx[threadIdx.x] = row;
+            rowidx[threadIdx.x] = cache_row(j0 + threadIdx.x);
         }
-        __syncthreads();
-
-        // ---- stage K (row major) and V (transposed) ------------------------------------------------
-        for (uint32_t c = threadIdx.x; c < BN * CPR; c += kThreads) {
+    };
+    auto request = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < K_IT; it++) {
+            const uint32_t c = min(threadIdx.x + it * kThreads, static_cast<uint32_t>(K_ITEMS - 1));
             const uint32_t r = c / CPR, cc = c % CPR;
-            const bool live = j0 + r < range_end;
-            uint4 val = make_uint4(0, 0, 0, 0);
-            if (live) {
-                const uint64_t row = rowidx[r];
-                if (DQ1 == 0 || cc < CPR0) {
-                    val = *reinterpret_cast<const uint4 *>(p.k0 + row * p.k0_tok_stride + (SEPARATE_V ? kvh * DQ0 : 0) + cc * 8);
-                } else {
-                    val = *reinterpret_cast<const uint4 *>(p.k1 + row * p.k1_tok_stride + (cc - CPR0) * 8);
-                }
-            }
-            *reinterpret_cast<uint4 *>(Ks + r * KSTRIDE + cc * 8) = val;
-            if (!SEPARATE_V && cc < VCPR) {
-                const uint32_t pos = vt_pos(r);
-                const uint16_t *e = reinterpret_cast<const uint16_t *>(&val);
+            const uint64_t row = rowidx[r];
+            const uint16_t *src = (DQ1 == 0 || cc < CPR0) ? p.k0 + row * p.k0_tok_stride + (SEPARATE_V ? kvh * DQ0 : 0) + cc * 8
+                                                          : p.k1 + row * p.k1_tok_stride + (cc - CPR0) * 8;
+            const uint4 x = *reinterpret_cast<const uint4 *>(src);
+            kbuf[it][0] = x.x;
+            kbuf[it][1] = x.y;
+            kbuf[it][2] = x.z;
+            kbuf[it][3] = x.w;
+        }
+        if constexpr (SEPARATE_V) {
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    Vt[(cc * 8 + i) * VSTRIDE + pos] = e[i];
+            for (int it = 0; it < V_IT; it++) {
+                const uint32_t c = min(threadIdx.x + it * kThreads, static_cast<uint32_t>(V_ITEMS - 1));
+                const uint32_t g = c / VCPR, cc = c % VCPR;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint4 x = *reinterpret_cast<const uint4 *>(p.v + rowidx[4 * g + j] * p.k0_tok_stride + kvh * DV + cc * 8);
+                    vbuf[it][j][0] = x.x;
+                    vbuf[it][j][1] = x.y;
+                    vbuf[it][j][2] = x.z;
+                    vbuf[it][j][3] = x.w;
                 }
             }
         }
-        if (SEPARATE_V) {
-            for (uint32_t c = threadIdx.x; c < BN * VCPR; c += kThreads) {
-                const uint32_t r = c / VCPR, cc = c % VCPR;
-                const bool live = j0 + r < range_end;
-                uint4 val = make_uint4(0, 0, 0, 0);
-                if (live) {
-                    val = *reinterpret_cast<const uint4 *>(p.v + rowidx[r] * p.k0_tok_stride + kvh * DV + cc * 8);
-                }
-                const uint32_t pos = vt_pos(r);
-                const uint16_t *e = reinterpret_cast<const uint16_t *>(&val);
+    };
+    auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    Vt[(cc * 8 + i) * VSTRIDE + pos] = e[i];
+        for (int it = 0; it < K_IT; it++) {
+            const uint32_t c = threadIdx.x + it * kThreads;
+            if (K_ITEMS % kThreads == 0 || c < K_ITEMS) {
+                const uint32_t r = c / CPR, cc = c % CPR;
+                *reinterpret_cast<uint4 *>(Ks + r * KSTRIDE + cc * 8) = make_uint4(kbuf[it][0], kbuf[it][1], kbuf[it][2], kbuf[it][3]);
+                if constexpr (!SEPARATE_V) {   // the value is the first DV columns of the same row
+                    if (cc < VCPR) {
+                        const uint32_t pos = vt_pos(r);
+#pragma unroll
+                        for (int i = 0; i < 8; i++) {
+                            Vt[(cc * 8 + i) * VSTRIDE + pos] = static_cast<uint16_t>(kbuf[it][i / 2] >> ((i & 1) * 16));
+                        }
+                    }
                 }
             }
+        }
+        if constexpr (SEPARATE_V) {
+#pragma unroll
+            for (int it = 0; it < V_IT; it++) {
+                const uint32_t c = threadIdx.x + it * kThreads;
+                if (V_ITEMS % kThreads == 0 || c < V_ITEMS) {
+                    const uint32_t g = c / VCPR, cc = c % VCPR;
+                    const uint32_t pos = vt_pos(4 * g);   // positions 4 g .. 4 g + 3 stay next to each other
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        // element i of the four positions
+                        const int wi = i / 2, sh = (i & 1) * 16;
+                        uint2 o;
+                        o.x = ((vbuf[it][0][wi] >> sh) & 0xffffu) | ((vbuf[it][1][wi] >> sh) << 16);
+                        o.y = ((vbuf[it][2][wi] >> sh) & 0xffffu) | ((vbuf[it][3][wi] >> sh) << 16);
+                        *reinterpret_cast<uint2 *>(Vt + (cc * 8 + i) * VSTRIDE + pos) = o;
+                    }
+                }
+            }
+        }
+    };
+    // (the latent-cache instantiation has no registers to spare: it requests a tile when it needs it)
+    constexpr bool AHEAD = SEPARATE_V;
+    lookup(range_begin);
+    __syncthreads();
+    if constexpr (AHEAD) {
+        request();
+    }
+
+    for (uint32_t j0 = range_begin; j0 < range_end; j0 += BN) {
+        __syncthreads();  // previous tile fully consumed (and its row table read by every request)
+        if constexpr (AHEAD) {
+            stage();
+        } else {
+            // chunk by chunk, in a loop the compiler keeps rolled: one staging register set
+#pragma unroll 1
+            for (uint32_t c = threadIdx.x; c < K_ITEMS; c += kThreads) {
+                const uint32_t r = c / CPR, cc = c % CPR;
+                const uint64_t row = rowidx[r];
+                const uint16_t *src = (DQ1 == 0 || cc < CPR0) ? p.k0 + row * p.k0_tok_stride + (SEPARATE_V ? kvh * DQ0 : 0) + cc * 8
+                                                              : p.k1 + row * p.k1_tok_stride + (cc - CPR0) * 8;
+                const uint4 val = *reinterpret_cast<const uint4 *>(src);
+                *reinterpret_cast<uint4 *>(Ks + r * KSTRIDE + cc * 8) = val;
+                if (cc < VCPR) {
+                    const uint32_t pos = vt_pos(r);
+                    const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        Vt[(cc * 8 + i) * VSTRIDE + pos] = static_cast<uint16_t>(w[i / 2] >> ((i & 1) * 16));
+                    }
+                }
+            }
+            __syncthreads();   // the row table has been read: the next tile's may be written
+        }
+        if (j0 + BN < range_end) {
+            lookup(j0 + BN);
         }
         __syncthreads();
+        if constexpr (AHEAD) {
+            if (j0 + BN < range_end) {
+                request();   // the next tile's rows are in flight during this tile's products
+            }
+        }
 
         // ---- S^T = K . Q^T ----------------------------------------------------------------------------
         f32x16_t S[NT];
