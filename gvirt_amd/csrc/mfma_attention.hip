@@ -75,6 +75,7 @@ struct MfmaParams {
     uint32_t split_len;
     uint32_t max_splits;
     float scale_log2e;
+    uint32_t table_in_lds;   // 1: the launch reserved LDS for the sequence's block-table row (max_num_block words)
 };
 
 // position inside a 16-token group at which token offset o is stored in the transposed V tile, so
@@ -102,6 +103,7 @@ mfma_attention_kernel(const MfmaParams p)
     uint16_t *Ks = reinterpret_cast<uint16_t *>(smem_raw);
     uint16_t *Vt = Ks + BN * KSTRIDE;
     uint64_t *rowidx = reinterpret_cast<uint64_t *>(Vt + DV * VSTRIDE);
+    uint32_t *tbl_lds = reinterpret_cast<uint32_t *>(rowidx + BN);
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
@@ -165,15 +167,18 @@ mfma_attention_kernel(const MfmaParams p)
     {
         const uint16_t *src0 = p.q0 + static_cast<uint64_t>(tok) * p.q0_tok_stride + static_cast<uint64_t>(head) * p.q0_head_stride;
         const uint16_t *src1 = DQ1 ? p.q1 + static_cast<uint64_t>(tok) * p.q1_tok_stride + static_cast<uint64_t>(head) * p.q1_head_stride : nullptr;
+        // (every lane loads: rows past the tile's end point at the sequence's first row and are cleared below; a load
+        // under a condition is compiled into a branch with a wait of its own, one trip to memory per load)
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int c = ks * 16 + half * 8;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m_valid) {
-                v = (ks * 16 < DQ0) ? *reinterpret_cast<const uint4 *>(src0 + c)
-                                    : *reinterpret_cast<const uint4 *>(src1 + (c - DQ0));
-            }
-            qreg[ks] = v;
+            qreg[ks] = (ks * 16 < DQ0) ? *reinterpret_cast<const uint4 *>(src0 + c)
+                                       : *reinterpret_cast<const uint4 *>(src1 + (c - DQ0));
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+            qreg[ks] = m_valid ? qreg[ks] : make_uint4(0, 0, 0, 0);
         }
     }
 
@@ -207,8 +212,18 @@ mfma_attention_kernel(const MfmaParams p)
         }
         const uint32_t b = p.block_shift >= 0 ? t >> p.block_shift : t / p.block_size;
         const uint32_t o = p.block_shift >= 0 ? t & (p.block_size - 1) : t % p.block_size;
-        return static_cast<uint64_t>(static_cast<uint32_t>(table[b])) * p.block_size + o;
+        // (from LDS when the row was staged: a load from memory here sits between the two barriers of every tile)
+        const uint32_t entry = p.table_in_lds ? tbl_lds[b] : static_cast<uint32_t>(table[b]);
+        return static_cast<uint64_t>(entry) * p.block_size + o;
     };
+    if (!dense && p.table_in_lds) {
+        const uint32_t b_lo = (p.block_shift >= 0 ? range_begin >> p.block_shift : range_begin / p.block_size);
+        const uint32_t b_hi = (p.block_shift >= 0 ? (range_end - 1) >> p.block_shift : (range_end - 1) / p.block_size);
+        for (uint32_t b = b_lo + threadIdx.x; b <= b_hi; b += kThreads) {
+            tbl_lds[b] = static_cast<uint32_t>(table[b]);
+        }
+        __syncthreads();
+    }
     // the tile's rows are looked up by the first BN threads and shared through LDS (two barriers around the table)
     auto lookup = [&](uint32_t j0) __attribute__((always_inline)) {
         if (threadIdx.x < BN) {
@@ -233,7 +248,7 @@ mfma_attention_kernel(const MfmaParams p)
 #pragma unroll
             for (int it = 0; it < V_IT; it++) {
                 const uint32_t c = min(threadIdx.x + it * kThreads, static_cast<uint32_t>(V_ITEMS - 1));
-                const uint32_t g = c / VCPR, cc = c % VCPR;
+                const uint32_t g = c % (BN / 4), cc = c / (BN / 4);   // (position groups across the lanes: see `stage`)
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const uint4 x = *reinterpret_cast<const uint4 *>(p.v + rowidx[4 * g + j] * p.k0_tok_stride + kvh * DV + cc * 8);
@@ -268,8 +283,11 @@ mfma_attention_kernel(const MfmaParams p)
             for (int it = 0; it < V_IT; it++) {
                 const uint32_t c = threadIdx.x + it * kThreads;
                 if (V_ITEMS % kThreads == 0 || c < V_ITEMS) {
-                    const uint32_t g = c / VCPR, cc = c % VCPR;
-                    const uint32_t pos = vt_pos(4 * g);   // positions 4 g .. 4 g + 3 stay next to each other
+                    const uint32_t g = c % (BN / 4), cc = c / (BN / 4);   // (position groups across the lanes: see `stage`)
+                    // positions 4 g .. 4 g + 3 stay next to each other. A wave's lanes are the 16 position groups of four
+                    // consecutive chunks: consecutive 8-byte words of a V^T row (with the chunk across the lanes, a
+                    // row of 8 x 144 bytes apart, every store was a 32-way bank conflict: 4300 of a tile's 12600 cycles)
+                    const uint32_t pos = vt_pos(4 * g);
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
                         // element i of the four positions
@@ -374,11 +392,14 @@ mfma_attention_kernel(const MfmaParams p)
             pb[nt][1] = make_uint4(w[4], w[5], w[6], w[7]);
         }
         l_run = l_run * alpha + psum;
+        if (!SEPARATE_V || __any(alpha != 1.0f)) {   // the running maximum rarely moves after the first tiles (the latent-cache
+                                                     // instantiation, short of registers, keeps one path)
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
+            for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
-            for (int k = 0; k < 16; k++) {
-                O[dt][k] *= alpha;
+                for (int k = 0; k < 16; k++) {
+                    O[dt][k] *= alpha;
+                }
             }
         }
 
@@ -442,9 +463,15 @@ constexpr size_t lds_bytes()
 }
 
 template <typename T, int DQ0, int DQ1, int DV, int BN, bool SEPARATE_V>
-int launch_kernel(hipStream_t stream, const MfmaParams &p, dim3 grid)
+int launch_kernel(hipStream_t stream, const MfmaParams &p_in, dim3 grid)
 {
-    constexpr size_t lds = lds_bytes<DQ0 + DQ1, DV, BN>();
+    MfmaParams p = p_in;
+    size_t lds = lds_bytes<DQ0 + DQ1, DV, BN>();
+    // the sequence's block-table row behind the tiles, when it fits
+    p.table_in_lds = p.block_tables != nullptr && lds + static_cast<size_t>(p.max_num_block) * 4 <= 150 * 1024 ? 1u : 0u;
+    if (p.table_in_lds) {
+        lds += static_cast<size_t>(p.max_num_block) * 4;
+    }
     auto kernel = mfma_attention_kernel<T, DQ0, DQ1, DV, BN, SEPARATE_V>;
     if (lds > 64 * 1024) {
         if (const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) {
