@@ -345,6 +345,8 @@ mfma_attention_kernel(const MfmaParams p)
         }
 
         // ---- S^T = K . Q^T ----------------------------------------------------------------------------
+        // (k-steps outermost: the NT score tiles are independent accumulation chains whose products alternate, and the
+        // operands of a k-step are read from LDS while the products of the one before run)
         f32x16_t S[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
@@ -352,10 +354,29 @@ mfma_attention_kernel(const MfmaParams p)
             for (int k = 0; k < 16; k++) {
                 S[nt][k] = 0.f;
             }
+        }
+        {
+            uint4 a_cur[NT], a_nxt[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                a_cur[nt] = *reinterpret_cast<const uint4 *>(Ks + (nt * 32 + col) * KSTRIDE + half * 8);
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
-                const uint4 a = *reinterpret_cast<const uint4 *>(Ks + (nt * 32 + col) * KSTRIDE + ks * 16 + half * 8);
-                S[nt] = Mfma<T>::run(a, qreg[ks], S[nt]);
+                if (ks + 1 < KS) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) {
+                        a_nxt[nt] = *reinterpret_cast<const uint4 *>(Ks + (nt * 32 + col) * KSTRIDE + (ks + 1) * 16 + half * 8);
+                    }
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) {
+                    S[nt] = Mfma<T>::run(a_cur[nt], qreg[ks], S[nt]);
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) {
+                    a_cur[nt] = a_nxt[nt];
+                }
             }
         }
 
@@ -404,12 +425,13 @@ mfma_attention_kernel(const MfmaParams p)
         }
 
         // ---- O^T += V^T . P^T -------------------------------------------------------------------------------
+        // (the position k-steps outermost: the DT accumulator tiles are independent, their products go back to back)
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
+        for (int nt = 0; nt < NT; nt++) {
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
+            for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
-                for (int kk = 0; kk < 2; kk++) {
+                for (int dt = 0; dt < DT; dt++) {
                     const uint4 a = *reinterpret_cast<const uint4 *>(Vt + (dt * 32 + col) * VSTRIDE + nt * 32 + kk * 16 + half * 8);
                     O[dt] = Mfma<T>::run(a, pb[nt][kk], O[dt]);
                 }
