@@ -369,10 +369,12 @@ mfma_attention_kernel(const MfmaParams p)
                         a_nxt[nt] = *reinterpret_cast<const uint4 *>(Ks + (nt * 32 + col) * KSTRIDE + (ks + 1) * 16 + half * 8);
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);   // (left alone the scheduler sinks the reads to just ahead of their products)
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
                     S[nt] = Mfma<T>::run(a_cur[nt], qreg[ks], S[nt]);
                 }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
                     a_cur[nt] = a_nxt[nt];
