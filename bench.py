@@ -699,8 +699,8 @@ def _bench_mla_dsa(args, torch, rt, s, ctx, sets, steps):
 
 def bench_indexer(args, torch, rt):
     """DSA indexer on the decode batch of configuration 4 (64 indexer heads of 128, one key head): the
-    `indexer_topk` operator (scores + selection of 2048 positions per row). Not a BASELINE configuration:
-    printed only with --config idx."""
+    `indexer_topk` operator (scores + selection of 2048 positions per row). Not one of the five configurations of
+    BASELINE.json: the line `idx` of `other_configs`, or alone with --config idx."""
     import numpy as np
     from gvirt_amd import workloads as W
     from gvirt_amd import _C
