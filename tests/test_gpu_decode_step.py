@@ -45,6 +45,7 @@ def test_decode_step_is_the_two_calls_bit_for_bit(rt, shape, ctx):
     (W.LLAMA3_8B, [100, 33, 256, 1]),                                            # head_dim 128, a workgroup per (row, kv head)
     (W.LLAMA3_8B, [(37 * i) % 255 + 1 for i in range(40)]),                      # ... a workgroup per row, all 8 kv heads
     (W.QWEN2_05B, [(53 * i) % 511 + 1 for i in range(150)]),                     # head_dim 64, more rows than compute units / kv heads
+    (W.QWEN2_05B, [(29 * i) % 300 + 1 for i in range(700)]),                     # more sequences than workgroups: several per workgroup
     (W.GqaShape("g3", 12, 3, 64, 16, torch.float16), [1, 16, 17, 200, 5]),       # 3 kv heads, fp16, block size 16
     (W.GqaShape("g12", 24, 12, 128, 32, torch.bfloat16), [9, 130, 64]),          # two passes of kv heads
 ])
